@@ -1,0 +1,582 @@
+/*
+ * CPU oracle: a plain-C restatement of what the reference's example kernels
+ * compute when they are lowered through its cpu/ (Triton-CPU) path.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is the checker that the HIP kernels
+ * are compared against and the "port" CPU baseline that the benchmark times;
+ * nothing in the shipped package links, imports or calls it.
+ *
+ * Every function cites the reference file:line it restates.  The execution
+ * model is the reference's persistent one: the logical grid of
+ * gridX*gridY*gridZ programs is cut into one contiguous [block_start,
+ * block_end) range per worker and each worker loops over its range calling the
+ * kernel body with pid = block index
+ * (cpu/lib/Dialect/TritonCPU/Transforms/MakePersistentKernel.cpp:144-198,
+ *  cpu/lib/TritonCPUToLLVM/GPUOpToLLVM.cpp:16-22).  Workers are OpenMP threads.
+ *
+ * Pinning status (what independent check fixes each function) is listed in
+ * oracle/README.md and exercised by tests/test_oracle_*.py:
+ *   orc_block_range, orc_pid_decode, orc_tile_of_pid : brute-force coverage /
+ *       bijection properties
+ *   orc_add_*      : closed form (numpy), bit-exact
+ *   orc_sin_f32    : float64 libm sin rounded once to fp32
+ *   orc_matmul_*   : textbook sum_k a*b vs numpy float64 on exactly
+ *       representable inputs, B = I, tile-order independence
+ *   orc_attn_fwd   : textbook softmax attention in float64, row-0 closed form,
+ *       uniform-K running mean, base-2 log-sum-exp identity
+ *   GELU epilogue, fp8 scaled GEMM: NOT in the reference; "parity unpinned" by
+ *       it (pinned only against torch/numpy closed forms).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* element type codes shared with the python wrapper */
+enum { ORC_F32 = 0, ORC_I32 = 1, ORC_BF16 = 2, ORC_F16 = 3, ORC_FP8E4M3 = 4 };
+/* epilogue codes for orc_matmul */
+enum {
+  ORC_EPI_NONE = 0,         /* C = cast(acc)                       09-persistent-matmul.py:141 */
+  ORC_EPI_BIAS_FULL = 1,    /* C = cast(acc) + bias[M,N] in half   09-matmul-fused.py:139-146  */
+  ORC_EPI_BIAS_ROW_GELU = 2,/* C = cast(gelu(acc + bias[n])) fp32  (not in the reference)      */
+  ORC_EPI_LEAKY_RELU = 3,   /* C = cast(leaky_relu(acc)) fp32      03-matrix-multiplication.py:370-374 */
+  ORC_EPI_BIAS_ROW = 4      /* C = cast(acc + bias[n]) fp32        (row bias without activation) */
+};
+
+/* ------------------------------------------------------------------ */
+/* scalar conversions                                                  */
+/* ------------------------------------------------------------------ */
+static inline float u32_as_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static inline uint32_t f32_as_u32(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+static inline float bf16_to_f32(uint16_t h) { return u32_as_f32((uint32_t)h << 16); }
+
+/* round-to-nearest-even fp32 -> bf16 (what `acc.to(bf16)` does) */
+static inline uint16_t f32_to_bf16(float f) {
+  uint32_t u = f32_as_u32(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+static inline float f16_to_f32(uint16_t h) {
+  uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  if (exp == 0) {
+    if (man == 0) return u32_as_f32(sign);
+    /* subnormal: value = man * 2^-24 */
+    float v = (float)man * 5.9604644775390625e-08f;
+    return sign ? -v : v;
+  }
+  if (exp == 31) return u32_as_f32(sign | 0x7f800000u | (man << 13));
+  return u32_as_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/* round-to-nearest-even fp32 -> fp16 */
+static inline uint16_t f32_to_f16(float f) {
+  uint32_t u = f32_as_u32(f);
+  uint32_t sign = (u >> 16) & 0x8000u;
+  uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);           /* NaN */
+  if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);          /* >= 65520 -> inf */
+  if (a < 0x38800000u) {                                            /* subnormal half / zero */
+    /* result = rne(|f| * 2^24) as an integer in [0, 1024] */
+    float scaled = u32_as_f32(a) * 16777216.0f;
+    float r = nearbyintf(scaled); /* default rounding mode = RNE */
+    return (uint16_t)(sign | (uint32_t)r);
+  }
+  uint32_t m = a + 0xc8000000u;   /* rebias exponent by -112 */
+  m += 0xfffu + ((m >> 13) & 1u); /* RNE on the 13 dropped bits */
+  return (uint16_t)(sign | (m >> 13));
+}
+
+/* OCP fp8 e4m3fn: 1-4-3, bias 7, no inf, NaN = S.1111.111, max finite 448 */
+static inline float fp8e4m3_to_f32(uint8_t b) {
+  uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+  uint32_t exp = (b >> 3) & 0xfu;
+  uint32_t man = b & 7u;
+  if (exp == 15 && man == 7) return u32_as_f32(sign | 0x7fc00000u);
+  if (exp == 0) {
+    float v = (float)man * 0.001953125f; /* man * 2^-9 */
+    return sign ? -v : v;
+  }
+  return u32_as_f32(sign | ((exp + 120u) << 23) | (man << 20));
+}
+
+/* saturating RNE fp32 -> e4m3fn (the host-side quantiser of the fp8 config) */
+static inline uint8_t f32_to_fp8e4m3(float f) {
+  uint32_t u = f32_as_u32(f);
+  uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  float a = fabsf(f);
+  if (a != a) return (uint8_t)(sign | 0x7f);
+  if (a >= 448.0f) return (uint8_t)(sign | 0x7e); /* saturate to 448 */
+  if (a < 0.015625f) {                            /* below 2^-6: subnormal grid 2^-9 */
+    float r = nearbyintf(a * 512.0f);
+    return (uint8_t)(sign | (uint8_t)r);          /* r == 8 lands on exp=1,man=0 */
+  }
+  uint32_t au = f32_as_u32(a);
+  au += 0x7ffffu + ((au >> 20) & 1u);             /* RNE on the 20 dropped bits */
+  uint32_t exp = (au >> 23) - 120u;
+  uint32_t man = (au >> 20) & 7u;
+  uint32_t code = (exp << 3) | man;
+  if (code > 0x7e) code = 0x7e;
+  return (uint8_t)(sign | code);
+}
+
+static inline float load_elem(const void *p, int64_t i, int dt) {
+  switch (dt) {
+  case ORC_BF16: return bf16_to_f32(((const uint16_t *)p)[i]);
+  case ORC_F16: return f16_to_f32(((const uint16_t *)p)[i]);
+  case ORC_FP8E4M3: return fp8e4m3_to_f32(((const uint8_t *)p)[i]);
+  default: return ((const float *)p)[i];
+  }
+}
+
+static inline float round_to(float v, int dt) {
+  switch (dt) {
+  case ORC_BF16: return bf16_to_f32(f32_to_bf16(v));
+  case ORC_F16: return f16_to_f32(f32_to_f16(v));
+  case ORC_FP8E4M3: return fp8e4m3_to_f32(f32_to_fp8e4m3(v));
+  default: return v;
+  }
+}
+
+static inline void store_elem(void *p, int64_t i, int dt, float v) {
+  switch (dt) {
+  case ORC_BF16: ((uint16_t *)p)[i] = f32_to_bf16(v); break;
+  case ORC_F16: ((uint16_t *)p)[i] = f32_to_f16(v); break;
+  case ORC_FP8E4M3: ((uint8_t *)p)[i] = f32_to_fp8e4m3(v); break;
+  default: ((float *)p)[i] = v; break;
+  }
+}
+
+ORC_API void orc_convert(const void *src, int src_dt, void *dst, int dst_dt, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) store_elem(dst, i, dst_dt, load_elem(src, i, src_dt));
+}
+
+/* ------------------------------------------------------------------ */
+/* SPMD plumbing                                                       */
+/* ------------------------------------------------------------------ */
+
+/* Contiguous balanced split of num_blocks logical programs over num_workers:
+ * base = nb / nw, rem = nb % nw, start(w) = w*base + min(w, rem),
+ * end = start + base + (w < rem)
+ * (npu/lib/TritonNPUToTenstorrent/D2M/SPMDOpToD2M.cpp:38-112; the host mirror
+ *  is examples/matmul_tensor_descriptor/matmul_multi_core_tma.cpp:139-158). */
+ORC_API void orc_block_range(int64_t num_blocks, int num_workers, int worker,
+                             int64_t *start, int64_t *end) {
+  int64_t base = num_blocks / num_workers;
+  int64_t rem = num_blocks % num_workers;
+  int64_t w = worker;
+  int64_t s = w * base + (w < rem ? w : rem);
+  *start = s;
+  *end = s + base + (w < rem ? 1 : 0);
+}
+
+/* Linear block index -> 3-D program id: x = b % gX, y = (b % (gX*gY)) / gX,
+ * z = b / (gX*gY)   (cpu/lib/TritonCPUToLLVM/GPUOpToLLVM.cpp:73-101). */
+ORC_API void orc_pid_decode(int64_t b, int gx, int gy, int *x, int *y, int *z) {
+  int64_t gxy = (int64_t)gx * gy;
+  *x = (int)(b % gx);
+  *y = (int)((b % gxy) / gx);
+  *z = (int)(b / gxy);
+}
+
+/* GROUP_SIZE_M swizzle of the descriptor matmuls
+ * (examples/matmul_tensor_descriptor/09-persistent-matmul.py:118-126). */
+ORC_API void orc_tile_of_pid(int pid, int num_pid_m, int num_pid_n, int group_m,
+                             int *pid_m, int *pid_n) {
+  int num_pid_in_group = group_m * num_pid_n;
+  int group_id = pid / num_pid_in_group;
+  int first_pid_m = group_id * group_m;
+  int group_size_m = num_pid_m - first_pid_m;
+  if (group_size_m > group_m) group_size_m = group_m;
+  *pid_m = first_pid_m + (pid % group_size_m);
+  *pid_n = (pid % num_pid_in_group) / group_size_m;
+}
+
+static int pick_threads(int nthreads) {
+#ifdef _OPENMP
+  if (nthreads <= 0) nthreads = omp_get_max_threads();
+#else
+  nthreads = 1;
+#endif
+  return nthreads;
+}
+
+/* ------------------------------------------------------------------ */
+/* Elementwise                                                         */
+/* ------------------------------------------------------------------ */
+
+/* add_kernel (python/tutorials/01-vector-add.py:29-54): program pid owns
+ * offsets pid*BLOCK + [0, BLOCK); lanes with offset >= n are masked: loads
+ * yield 0 and stores are dropped
+ * (cpu/lib/TritonCPUToLLVM/LoadStoreOpToLLVM.cpp:248-253,349-366).
+ * Only `grid` programs run: elements past grid*BLOCK stay untouched. */
+ORC_API void orc_add_f32(const float *x, const float *y, float *out, int32_t n,
+                         int32_t block, int32_t grid, int nthreads) {
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      for (int64_t i = lo; i < hi; ++i) out[i] = x[i] + y[i];
+    }
+  }
+}
+
+/* int32 variant: arith.addi, two's-complement wraparound. */
+ORC_API void orc_add_i32(const int32_t *x, const int32_t *y, int32_t *out, int32_t n,
+                         int32_t block, int32_t grid, int nthreads) {
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      for (int64_t i = lo; i < hi; ++i)
+        out[i] = (int32_t)((uint32_t)x[i] + (uint32_t)y[i]);
+    }
+  }
+}
+
+/* muladd_kernel (python/tutorials/01-vector-mul-add.py:30-57): x*y + z with
+ * enable_fp_fusion on by default (backend/compiler.py:29) => contraction to one
+ * fused multiply-add is what the cpu/ path emits; `fused`=0 gives the unfused
+ * two-rounding form. */
+ORC_API void orc_muladd_f32(const float *x, const float *y, const float *z, float *out,
+                            int32_t n, int32_t block, int32_t grid, int fused,
+                            int nthreads) {
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      if (fused) {
+        for (int64_t i = lo; i < hi; ++i) out[i] = fmaf(x[i], y[i], z[i]);
+      } else {
+        for (int64_t i = lo; i < hi; ++i) {
+          volatile float p = x[i] * y[i];
+          out[i] = p + z[i];
+        }
+      }
+    }
+  }
+}
+
+/* sin_kernel (examples/01-sin-kernel.py:17-29).  The cpu/ path calls an LLVM
+ * sin intrinsic resolved by libm or SLEEF; neither is bit-specified, so the
+ * oracle is the correctly rounded value: float64 sin rounded once to fp32. */
+ORC_API void orc_sin_f32(const float *x, float *out, int32_t n, int32_t block,
+                         int32_t grid, int nthreads) {
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      for (int64_t i = lo; i < hi; ++i) out[i] = (float)sin((double)x[i]);
+    }
+  }
+}
+
+/* Faster fp32 libm variant used only as the timed CPU baseline of the sin
+ * config (what a libm-backed cpu/ build would execute). */
+ORC_API void orc_sinf_f32(const float *x, float *out, int32_t n, int32_t block,
+                          int32_t grid, int nthreads) {
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      for (int64_t i = lo; i < hi; ++i) out[i] = sinf(x[i]);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ */
+/* Tile matmul family                                                  */
+/* ------------------------------------------------------------------ */
+
+static inline float gelu_erf(float x) {
+  /* exact-erf GELU in fp32: 0.5*x*(1+erf(x/sqrt(2))) */
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+
+/*
+ * matmul_kernel_tma / matmul_kernel_fused, one logical program per
+ * BM x BN output tile
+ * (examples/matmul_tensor_descriptor/09-persistent-matmul.py:102-145,
+ *  python/tutorials/09-matmul-fused.py:100-148).
+ *   - pid -> (pid_m, pid_n) through the GROUP_SIZE_M swizzle (:118-126)
+ *   - fp32 accumulator, K walked in BK steps (:131-139); A is [M,K] row-major
+ *     with leading stride lda, B is [K,N] row-major (NOT transposed) with ldb
+ *   - descriptor loads beyond the tensor are zero-padded, stores are clipped
+ *     (triton/tools/tensor_descriptor.py padding="zero")
+ *   - one RNE rounding fp32 -> out dtype (:141), then the epilogue selected by
+ *     `epi` (see the enum above for the reference line each follows)
+ * acc64 != 0 accumulates in double instead (used to state tolerances against a
+ * rounding-free sum, never as the parity target).
+ * scale multiplies the accumulator before the cast (fp8 per-tensor scales;
+ * pass 1.0f otherwise).
+ */
+ORC_API int orc_matmul(const void *a, int64_t lda, const void *b, int64_t ldb, void *c,
+                       int64_t ldc, const void *bias, int64_t ldbias, int32_t M,
+                       int32_t N, int32_t K, int32_t BM, int32_t BN, int32_t BK,
+                       int32_t group_m, int32_t grid, int in_dt, int out_dt, int epi,
+                       float scale, int acc64, int nthreads) {
+  if (BM <= 0 || BN <= 0 || BK <= 0 || group_m <= 0) return -1;
+  int num_pid_m = (M + BM - 1) / BM, num_pid_n = (N + BN - 1) / BN;
+  if (grid > num_pid_m * num_pid_n) return -2; /* pid outside the tile grid */
+  nthreads = pick_threads(nthreads);
+  int k_tiles = (K + BK - 1) / BK;
+#pragma omp parallel num_threads(nthreads)
+  {
+#ifdef _OPENMP
+    int w = omp_get_thread_num(), nw = omp_get_num_threads();
+#else
+    int w = 0, nw = 1;
+#endif
+    float *accf = (float *)malloc(sizeof(float) * (size_t)BM * BN);
+    double *accd = acc64 ? (double *)malloc(sizeof(double) * (size_t)BM * BN) : NULL;
+    float *at = (float *)malloc(sizeof(float) * (size_t)BM * BK);
+    float *bt = (float *)malloc(sizeof(float) * (size_t)BK * BN);
+    int64_t bs, be;
+    orc_block_range(grid, nw, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int pid_m, pid_n;
+      orc_tile_of_pid((int)pid, num_pid_m, num_pid_n, group_m, &pid_m, &pid_n);
+      int64_t om = (int64_t)pid_m * BM, on = (int64_t)pid_n * BN;
+      for (int i = 0; i < BM * BN; ++i) accf[i] = 0.0f;
+      if (acc64) for (int i = 0; i < BM * BN; ++i) accd[i] = 0.0;
+      for (int kt = 0; kt < k_tiles; ++kt) {
+        int64_t ok = (int64_t)kt * BK;
+        /* descriptor loads with zero padding */
+        for (int i = 0; i < BM; ++i)
+          for (int k = 0; k < BK; ++k)
+            at[i * BK + k] = (om + i < M && ok + k < K)
+                                 ? load_elem(a, (om + i) * lda + ok + k, in_dt) : 0.0f;
+        for (int k = 0; k < BK; ++k)
+          for (int j = 0; j < BN; ++j)
+            bt[k * BN + j] = (ok + k < K && on + j < N)
+                                 ? load_elem(b, (ok + k) * ldb + on + j, in_dt) : 0.0f;
+        /* acc = dot(a, b, acc) */
+        if (!acc64) {
+          for (int i = 0; i < BM; ++i) {
+            float *arow = accf + (size_t)i * BN;
+            for (int k = 0; k < BK; ++k) {
+              float av = at[i * BK + k];
+              const float *brow = bt + (size_t)k * BN;
+              for (int j = 0; j < BN; ++j) arow[j] += av * brow[j];
+            }
+          }
+        } else {
+          for (int i = 0; i < BM; ++i) {
+            double *arow = accd + (size_t)i * BN;
+            for (int k = 0; k < BK; ++k) {
+              double av = at[i * BK + k];
+              const float *brow = bt + (size_t)k * BN;
+              for (int j = 0; j < BN; ++j) arow[j] += av * (double)brow[j];
+            }
+          }
+        }
+      }
+      /* epilogue + clipped store */
+      for (int i = 0; i < BM; ++i) {
+        if (om + i >= M) break;
+        for (int j = 0; j < BN; ++j) {
+          if (on + j >= N) break;
+          float acc = acc64 ? (float)(accd[(size_t)i * BN + j] * (double)scale)
+                            : (scale == 1.0f ? accf[(size_t)i * BN + j]
+                                             : accf[(size_t)i * BN + j] * scale);
+          float v;
+          switch (epi) {
+          case ORC_EPI_BIAS_FULL: {
+            /* c = acc.to(dtype); c = c + bias  -- the add is done in the
+             * half-precision type: exact fp32 sum of two half values rounded
+             * once to the half type is the IEEE half add. */
+            float cv = round_to(acc, out_dt);
+            float bv = load_elem(bias, (om + i) * ldbias + on + j, out_dt);
+            v = cv + bv;
+            break;
+          }
+          case ORC_EPI_BIAS_ROW_GELU:
+            v = gelu_erf(acc + load_elem(bias, on + j, ORC_F32));
+            break;
+          case ORC_EPI_BIAS_ROW:
+            v = acc + load_elem(bias, on + j, ORC_F32);
+            break;
+          case ORC_EPI_LEAKY_RELU:
+            v = acc >= 0.0f ? acc : 0.01f * acc;
+            break;
+          default:
+            v = acc;
+          }
+          store_elem(c, (om + i) * ldc + on + j, out_dt, v);
+        }
+      }
+    }
+    free(accf); free(accd); free(at); free(bt);
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
+/* Fused attention forward                                             */
+/* ------------------------------------------------------------------ */
+
+/*
+ * _attn_fwd + _attn_fwd_inner (examples/fused-attn/06-fused-attention.py:143-215,
+ * 33-90).  q,k,v,o are bf16 viewed as 2-D [Z*H*N_CTX, D] with strides [D,1]
+ * (:243-246); Mout is fp32 [Z*H*N_CTX].  grid = (cdiv(N_CTX,BLOCK_M), Z*H, 1)
+ * (:253-254); linear block index b decodes to start_m = b % gridX,
+ * off_hz = b / gridX.  stage = 3 causal, 1 non-causal (:235).
+ * Recipe restated line by line:
+ *   qk_scale = sm_scale * 1.44269504                       (:188-189)
+ *   m_i = -inf, l_i = 1.0, acc = 0                          (:184-186)
+ *   off-band blocks:  m_ij = max(m_i, rowmax(qk)*qk_scale);
+ *                     qk = qk*qk_scale - m_ij               (:63-64)
+ *   on-band block:    qk = qk*qk_scale + (m >= n ? 0 : -1.0e6);
+ *                     m_ij = max(m_i, rowmax(qk)); qk -= m_ij (:57-61)
+ *   p = exp2(qk); alpha = exp2(m_i - m_ij); l_ij = rowsum(p) in fp32 (:65-68)
+ *   acc = acc*alpha + dot(bf16(p), v)                       (:79-83)
+ *   l_i = l_i*alpha + l_ij; m_i = m_ij                      (:86-87)
+ *   epilogue: m_i += log2(l_i); acc /= l_i; store M, bf16(acc) (:211-215)
+ */
+static void attn_block(const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                       uint16_t *o, float *Mout, float sm_scale, int H, int N_CTX, int D,
+                       int BLOCK_M, int BLOCK_N, int stage, int start_m, int off_hz,
+                       float *qf, float *acc, float *qk, float *m_i, float *l_i) {
+  (void)H;
+  int64_t offset_y = (int64_t)off_hz * N_CTX; /* off_z*(N_CTX*H) + off_h*N_CTX */
+  int64_t qo = offset_y + (int64_t)start_m * BLOCK_M;
+  float qk_scale = sm_scale * 1.44269504f;
+  int rows = BLOCK_M;
+  if ((int64_t)start_m * BLOCK_M + rows > N_CTX) rows = N_CTX - start_m * BLOCK_M;
+  for (int i = 0; i < rows; ++i) {
+    m_i[i] = -INFINITY;
+    l_i[i] = 1.0f;
+    for (int d = 0; d < D; ++d) {
+      acc[(size_t)i * D + d] = 0.0f;
+      qf[(size_t)i * D + d] = bf16_to_f32(q[(qo + i) * D + d]);
+    }
+  }
+  for (int pass = 0; pass < 2; ++pass) {
+    int inner; /* STAGE seen by _attn_fwd_inner */
+    if (pass == 0) { if (!(stage & 1)) continue; inner = 4 - stage; }
+    else { if (!(stage & 2)) continue; inner = 2; }
+    int lo, hi;
+    if (inner == 1) { lo = 0; hi = start_m * BLOCK_M; }
+    else if (inner == 2) { lo = start_m * BLOCK_M; hi = (start_m + 1) * BLOCK_M; }
+    else { lo = 0; hi = N_CTX; }
+    for (int start_n = lo; start_n < hi; start_n += BLOCK_N) {
+      int cols = BLOCK_N;
+      for (int i = 0; i < rows; ++i) {
+        int om = start_m * BLOCK_M + i;
+        float rmax = -INFINITY;
+        for (int j = 0; j < cols; ++j) {
+          int64_t kn = start_n + j;
+          float s = 0.0f;
+          if (kn < N_CTX) { /* rows past the tensor read as zero */
+            const uint16_t *kr = k + (offset_y + kn) * D;
+            const float *qr = qf + (size_t)i * D;
+            for (int d = 0; d < D; ++d) s += qr[d] * bf16_to_f32(kr[d]);
+          }
+          if (inner == 2) s = s * qk_scale + (om >= start_n + j ? 0.0f : -1.0e6f);
+          qk[j] = s;
+          if (s > rmax) rmax = s;
+        }
+        float m_ij;
+        if (inner == 2) {
+          m_ij = fmaxf(m_i[i], rmax);
+          for (int j = 0; j < cols; ++j) qk[j] -= m_ij;
+        } else {
+          m_ij = fmaxf(m_i[i], rmax * qk_scale);
+          for (int j = 0; j < cols; ++j) qk[j] = qk[j] * qk_scale - m_ij;
+        }
+        float l_ij = 0.0f;
+        for (int j = 0; j < cols; ++j) { qk[j] = exp2f(qk[j]); l_ij += qk[j]; }
+        float alpha = exp2f(m_i[i] - m_ij);
+        float *ar = acc + (size_t)i * D;
+        for (int d = 0; d < D; ++d) ar[d] *= alpha;
+        for (int j = 0; j < cols; ++j) {
+          int64_t kn = start_n + j;
+          if (kn >= N_CTX) continue;
+          float p = bf16_to_f32(f32_to_bf16(qk[j]));
+          const uint16_t *vr = v + (offset_y + kn) * D;
+          for (int d = 0; d < D; ++d) ar[d] += p * bf16_to_f32(vr[d]);
+        }
+        l_i[i] = l_i[i] * alpha + l_ij;
+        m_i[i] = m_ij;
+      }
+    }
+  }
+  for (int i = 0; i < rows; ++i) {
+    Mout[qo + i] = m_i[i] + log2f(l_i[i]);
+    float *ar = acc + (size_t)i * D;
+    for (int d = 0; d < D; ++d) o[(qo + i) * D + d] = f32_to_bf16(ar[d] / l_i[i]);
+  }
+}
+
+ORC_API int orc_attn_fwd(float sm_scale, float *Mout, int32_t Z, int32_t H,
+                         const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                         uint16_t *o, int32_t N_CTX, int32_t D, int32_t BLOCK_M,
+                         int32_t BLOCK_N, int32_t stage, int32_t grid_x, int32_t grid_y,
+                         int nthreads) {
+  if (BLOCK_N > D) return -1;               /* static_assert(BLOCK_N <= HEAD_DIM) (:158) */
+  if (stage != 1 && stage != 3) return -2;
+  if (grid_y > Z * H) return -3;
+  if ((int64_t)grid_x * BLOCK_M > N_CTX + BLOCK_M - 1) return -4;
+  nthreads = pick_threads(nthreads);
+  int64_t nblocks = (int64_t)grid_x * grid_y;
+#pragma omp parallel num_threads(nthreads)
+  {
+#ifdef _OPENMP
+    int w = omp_get_thread_num(), nw = omp_get_num_threads();
+#else
+    int w = 0, nw = 1;
+#endif
+    float *qf = (float *)malloc(sizeof(float) * (size_t)BLOCK_M * D);
+    float *acc = (float *)malloc(sizeof(float) * (size_t)BLOCK_M * D);
+    float *qk = (float *)malloc(sizeof(float) * (size_t)BLOCK_N);
+    float *m_i = (float *)malloc(sizeof(float) * (size_t)BLOCK_M);
+    float *l_i = (float *)malloc(sizeof(float) * (size_t)BLOCK_M);
+    int64_t bs, be;
+    orc_block_range(nblocks, nw, w, &bs, &be);
+    for (int64_t b = bs; b < be; ++b) {
+      int px, py, pz;
+      orc_pid_decode(b, grid_x, grid_y, &px, &py, &pz);
+      attn_block(q, k, v, o, Mout, sm_scale, H, N_CTX, D, BLOCK_M, BLOCK_N, stage, px, py,
+                 qf, acc, qk, m_i, l_i);
+    }
+    free(qf); free(acc); free(qk); free(m_i); free(l_i);
+  }
+  return 0;
+}
+
+ORC_API int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
