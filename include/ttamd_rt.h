@@ -1,0 +1,231 @@
+/*
+ * libttamd_rt.so -- C ABI of the MI355X (gfx950) host runtime.
+ *
+ * Two layers:
+ *   rt_*  a thin loader/launcher over the HIP module API (hipModuleLoadData /
+ *         hipModuleGetFunction / hipModuleLaunchKernel, hipMalloc'd buffers,
+ *         hipEvents).  It takes the place of the device handle that the
+ *         reference launcher drives through knexus:
+ *         device.load_library / lib.get_kernel   backend/driver.py:68-74
+ *         create_schedule / create_command / set_arg / finalize / run
+ *                                                backend/driver.py:114-170
+ *   tt_*  one entry point per kernel NAME of the reference examples, taking the
+ *         same launch-time arguments (pointers, i32 sizes, tensor descriptors,
+ *         the constexpr BLOCK sizes and the logical grid) and binding them to a
+ *         hand-written gfx950 kernel.  The logical grid keeps the reference's
+ *         meaning: program `pid` of gridX*gridY*gridZ does exactly the work the
+ *         example kernel source gives it; the runtime is free to execute those
+ *         programs on a persistent physical grid sized to the CU count
+ *         (cpu/lib/Dialect/TritonCPU/Transforms/MakePersistentKernel.cpp:144-198).
+ *
+ * Conventions: every function returns 0 on success and a negative rt_status on
+ * failure, never aborts and never throws; rt_last_error() gives the message of
+ * the calling thread's last failure.  The caller owns every buffer and keeps it
+ * alive until the stream has run the launch.  `stream` is a hipStream_t (NULL =
+ * the default stream); launches are asynchronous on it.  Pointers handed to
+ * tt_* are device pointers.  Distinct streams may be driven from distinct
+ * threads; kernels are immutable after rt_init.
+ */
+#ifndef TTAMD_RT_H
+#define TTAMD_RT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTAMD_API __attribute__((visibility("default")))
+
+typedef enum rt_status {
+  RT_OK = 0,
+  RT_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, bad grid) */
+  RT_ERR_HIP = -2,         /* a HIP call failed; rt_last_error() has its string    */
+  RT_ERR_NOT_FOUND = -3,   /* unknown kernel / symbol name                         */
+  RT_ERR_UNSUPPORTED = -4, /* valid request this build has no kernel for           */
+  RT_ERR_NOT_INIT = -5     /* rt_init has not succeeded on this device             */
+} rt_status;
+
+/* element types of tensors and descriptors (Triton type strings in comments) */
+typedef enum tt_dtype {
+  TT_F32 = 0,     /* *fp32    */
+  TT_I32 = 1,     /* *i32     */
+  TT_BF16 = 2,    /* *bf16    */
+  TT_F16 = 3,     /* *fp16    */
+  TT_FP8E4M3 = 4  /* *fp8e4nv (OCP e4m3fn) */
+} tt_dtype;
+
+/* ----------------------------------------------------------------------- */
+/* rt_*: device, memory, modules, launches, events                          */
+/* ----------------------------------------------------------------------- */
+
+/* What TTUtils.get_device_properties reports (backend/driver.py:76-82), read
+ * from hipGetDeviceProperties. */
+typedef struct rt_props {
+  int32_t device;
+  int32_t multiprocessor_count; /* CUs */
+  int32_t warp_size;            /* 64 */
+  int32_t max_shared_mem;       /* LDS bytes per workgroup */
+  int32_t max_num_regs;         /* 32-bit registers per workgroup */
+  int32_t clock_khz;            /* max engine clock */
+  int32_t mem_clock_khz;
+  int32_t mem_bus_bits;
+  int32_t l2_bytes;
+  int32_t reserved;
+  uint64_t total_mem;           /* HBM bytes */
+  char name[128];
+  char arch[64];                /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+} rt_props;
+
+typedef struct rt_module_s *rt_module;
+typedef struct rt_kernel_s *rt_kernel;
+typedef struct rt_event_s *rt_event;
+
+/* Selects `device`, creates its context and loads the built-in code objects.
+ * Idempotent.  Replaces torch.nexus.get_device / set_runtime
+ * (backend/driver.py:462-468). */
+TTAMD_API int rt_init(int device);
+TTAMD_API int rt_device_count(int *count);
+TTAMD_API int rt_device_props(rt_props *out);
+
+/* Raw device memory for callers without torch (C++ benches, tests).
+ * kind: 0 host->host, 1 host->device, 2 device->host, 3 device->device. */
+TTAMD_API int rt_malloc(void **ptr, size_t bytes);
+TTAMD_API int rt_free(void *ptr);
+TTAMD_API int rt_memcpy(void *dst, const void *src, size_t bytes, int kind);
+TTAMD_API int rt_memset(void *dst, int value, size_t bytes, void *stream);
+
+/* Code objects.  rt_module_load takes a gfx950 code object image in memory
+ * (device.load_library, backend/driver.py:72); rt_builtin_module returns one of
+ * the images embedded in this library ("elementwise", "gemm", "attention"). */
+TTAMD_API int rt_module_load(const void *image, size_t bytes, rt_module *out);
+TTAMD_API int rt_module_unload(rt_module m);
+TTAMD_API int rt_builtin_module(const char *which, rt_module *out);
+/* lib.get_kernel(name) (backend/driver.py:73): a device symbol of module m. */
+TTAMD_API int rt_get_kernel(rt_module m, const char *name, rt_kernel *out);
+/* command.set_arg... + finalize(grid, block, shared) + schedule.run()
+ * (backend/driver.py:117-168), asynchronous on `stream`.  args[i] points at
+ * the i-th kernel parameter value. */
+TTAMD_API int rt_launch(rt_kernel k, const uint32_t grid[3], const uint32_t block[3],
+              uint32_t shared_bytes, void *stream, void **args, size_t nargs);
+TTAMD_API int rt_sync(void *stream);
+
+/* hipEvent timing: the device-side counterpart of TTDeviceInterface.Event
+ * (backend/driver.py:390-442). */
+TTAMD_API int rt_event_create(rt_event *out);
+TTAMD_API int rt_event_record(rt_event e, void *stream);
+TTAMD_API int rt_event_sync(rt_event e);
+TTAMD_API int rt_event_elapsed_ms(rt_event start, rt_event stop, float *ms);
+TTAMD_API int rt_event_destroy(rt_event e);
+
+TTAMD_API const char *rt_last_error(void);
+
+/* ----------------------------------------------------------------------- */
+/* tt_*: the example kernels                                                */
+/* ----------------------------------------------------------------------- */
+
+/* A rank-2 host tensor descriptor as the launcher flattens it:
+ * base, shape..., strides..., padding flag (backend/driver.py:141-159, 322-329;
+ * device-side type list test/Tenstorrent/dot_op_to_ttkernel.mlir:412).
+ * Strides are in elements; the last stride must be 1. */
+typedef struct tt_desc2d {
+  void *base;
+  int32_t shape[2];
+  int64_t strides[2];
+  int32_t block_shape[2];
+  int32_t padding_nan; /* 1 if padding == "nan" (driver.py:326); only 0 is supported */
+  int32_t dtype;       /* tt_dtype */
+} tt_desc2d;
+
+/* Epilogues of the fused tile matmul. */
+typedef enum tt_epilogue {
+  TT_EPI_NONE = 0,
+  /* c = acc.to(half) + bias[M,N], added in the half type
+   * (python/tutorials/09-matmul-fused.py:139-146) */
+  TT_EPI_BIAS_FULL = 1,
+  /* c = (gelu_erf(acc + bias[n])).to(half), epilogue in fp32 on the accumulator
+   * (no counterpart in the reference; placement follows the leaky_relu
+   * precedent examples/matmul/03-matrix-multiplication.py:370-374) */
+  TT_EPI_BIAS_ROW_GELU = 2,
+  /* c = leaky_relu(acc).to(half) (03-matrix-multiplication.py:370-374,393-395) */
+  TT_EPI_LEAKY_RELU = 3,
+  /* c = (acc + bias[n]).to(half) */
+  TT_EPI_BIAS_ROW = 4
+} tt_epilogue;
+
+/* add_kernel(x_ptr, y_ptr, output_ptr, n_elements, BLOCK_SIZE)
+ * python/tutorials/01-vector-add.py:29-54.  dtype TT_F32 or TT_I32.
+ * Programs 0..grid[0]-1 each own BLOCK_SIZE consecutive elements; lanes at or
+ * past n_elements are masked, elements past grid[0]*BLOCK_SIZE are untouched. */
+TTAMD_API int tt_add_kernel(const void *x, const void *y, void *out, int32_t n_elements,
+                  int32_t BLOCK_SIZE, int32_t dtype, const uint32_t grid[3], void *stream);
+
+/* add_kernel(x_ptr, y_ptr, output_ptr, n_elements, row_count, BLOCK_SIZE)
+ * python/tutorials/01-vector-add.loop.py:30-62: program pid owns
+ * [pid*BLOCK_SIZE*row_count, min(.. + BLOCK_SIZE*row_count, n_elements)). */
+TTAMD_API int tt_add_kernel_loop(const void *x, const void *y, void *out, int32_t n_elements,
+                       int32_t row_count, int32_t BLOCK_SIZE, int32_t dtype,
+                       const uint32_t grid[3], void *stream);
+
+/* muladd_kernel(x_ptr, y_ptr, z_ptr, output_ptr, n_elements, BLOCK_SIZE)
+ * python/tutorials/01-vector-mul-add.py:30-57; fp32, x*y+z contracted to one
+ * fused multiply-add (enable_fp_fusion default, backend/compiler.py:29). */
+TTAMD_API int tt_muladd_kernel(const void *x, const void *y, const void *z, void *out,
+                     int32_t n_elements, int32_t BLOCK_SIZE, const uint32_t grid[3],
+                     void *stream);
+
+/* sin_kernel(x_ptr, output_ptr, n_elements, BLOCK_SIZE)
+ * examples/01-sin-kernel.py:17-29; fp32. */
+TTAMD_API int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
+                  const uint32_t grid[3], void *stream);
+
+/* matmul_kernel_tma(a_desc, b_desc, c_desc, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
+ *                   BLOCK_SIZE_K, GROUP_SIZE_M, FP8_OUTPUT, WARP_SPECIALIZE)
+ * examples/matmul_tensor_descriptor/09-persistent-matmul.py:102-145.
+ * A [M,K] and B [K,N] (not transposed) row-major, fp32 accumulate, one
+ * round-to-nearest-even cast to c->dtype.  grid[0] logical programs, one per
+ * BLOCK_SIZE_M x BLOCK_SIZE_N tile in GROUP_SIZE_M-swizzled order. */
+TTAMD_API int tt_matmul_kernel_tma(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c,
+                         int32_t M, int32_t N, int32_t K, int32_t BLOCK_SIZE_M,
+                         int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K, int32_t GROUP_SIZE_M,
+                         const uint32_t grid[3], void *stream);
+
+/* matmul_kernel_fused(a_desc, b_desc, c_desc, bias_desc, M, N, K, ...)
+ * python/tutorials/09-matmul-fused.py:100-148.  `epilogue` is a tt_epilogue;
+ * TT_EPI_BIAS_FULL is the reference kernel, the row-bias forms take a bias
+ * descriptor of shape [1,N] (or [N,1] viewed as such) holding fp32. */
+TTAMD_API int tt_matmul_kernel_fused(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c,
+                           const tt_desc2d *bias, int32_t M, int32_t N, int32_t K,
+                           int32_t BLOCK_SIZE_M, int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K,
+                           int32_t GROUP_SIZE_M, int32_t epilogue, const uint32_t grid[3],
+                           void *stream);
+
+/* matmul_kernel_tma with fp8 e4m3 descriptors and two per-tensor fp32 scales:
+ * c = (acc * scale_a * scale_b).to(c->dtype).  The reference has fp8 inputs
+ * (09-persistent-matmul.py:116,173) but no scales; this sibling name is new. */
+TTAMD_API int tt_matmul_kernel_tma_fp8_scaled(const tt_desc2d *a, const tt_desc2d *b,
+                                    const tt_desc2d *c, int32_t M, int32_t N, int32_t K,
+                                    float scale_a, float scale_b, int32_t BLOCK_SIZE_M,
+                                    int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K,
+                                    int32_t GROUP_SIZE_M, const uint32_t grid[3],
+                                    void *stream);
+
+/* _attn_fwd(sm_scale, M, Z, H, desc_q, desc_k, desc_v, desc_o, N_CTX, HEAD_DIM,
+ *           BLOCK_M, BLOCK_N, FP8_OUTPUT, STAGE, warp_specialize, IS_HOPPER)
+ * examples/fused-attn/06-fused-attention.py:143-215.  bf16 descriptors of shape
+ * [Z*H*N_CTX, HEAD_DIM]; M receives m_i + log2(l_i); STAGE 3 = causal, 1 = full;
+ * grid = (cdiv(N_CTX, BLOCK_M), Z*H, 1). */
+TTAMD_API int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const tt_desc2d *desc_q,
+                const tt_desc2d *desc_k, const tt_desc2d *desc_v, const tt_desc2d *desc_o,
+                int32_t N_CTX, int32_t HEAD_DIM, int32_t BLOCK_M, int32_t BLOCK_N,
+                int32_t STAGE, const uint32_t grid[3], void *stream);
+
+/* Name of the device kernel the last tt_* call on this thread launched (for
+ * profiles and tests that assert which path ran). */
+TTAMD_API const char *tt_last_kernel_name(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTAMD_RT_H */

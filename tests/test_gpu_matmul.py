@@ -1,0 +1,163 @@
+"""GPU parity: the tile-matmul family through the launcher and the C ABI against the CPU
+oracle.  Tolerance (bf16/fp16/fp8 inputs, fp32 accumulate): abs(err) <= 1e-2*abs(ref) + 1e-4
+against the fp64-accumulated oracle, and PCC >= 0.9999 (the reference's bar is 0.97)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from triton_tenstorrent_amd import kernels as K
+from triton_tenstorrent_amd import runtime as rt
+from triton_tenstorrent_amd.tensor_descriptor import TensorDescriptor
+from util import ORC_DT, bits, close_bf16, decode, from_bits
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL, PCC = 1e-2, 1e-4, 0.9999
+
+
+def _ab(M, N, K_, dtype=torch.bfloat16, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    a = (torch.randn(M, K_, generator=g) / K_ ** 0.5 * 4).to(dtype)
+    b = (torch.randn(K_, N, generator=g)).to(dtype)
+    return a, b
+
+
+def _check(c, a, b, **okw):
+    dt = ORC_DT[a.dtype]
+    ref = orc.matmul(bits(a), bits(b), in_dt=dt, out_dt=ORC_DT[c.dtype], acc64=True, **okw)
+    ref = orc.decode(ref, ORC_DT[c.dtype])
+    got = decode(c)
+    assert close_bf16(got, ref, RTOL, ATOL), f"max err {np.max(np.abs(got - ref))}"
+    assert orc.pcc(ref, got) >= PCC
+
+
+# the reference's validate shapes (09-persistent-matmul.py:326-327, .ttnn.py:334-336) and more
+@pytest.mark.parametrize("M,N,K_", [(32, 32, 32), (64, 32, 32), (64, 32, 64), (256, 256, 256), (1024, 1024, 1024), (384, 640, 192)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matmul_tma(M, N, K_, dtype):
+    a, b = _ab(M, N, K_, dtype)
+    c = K.matmul_tma(a.cuda(), b.cuda())
+    _check(c, a, b)
+
+
+@pytest.mark.parametrize("cfg", [dict(BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64, GROUP_SIZE_M=1),
+                                 dict(BLOCK_SIZE_M=32, BLOCK_SIZE_N=32, BLOCK_SIZE_K=32, GROUP_SIZE_M=3),
+                                 dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=256, BLOCK_SIZE_K=64, GROUP_SIZE_M=8),
+                                 dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=128, BLOCK_SIZE_K=32, GROUP_SIZE_M=2)])
+def test_matmul_small_integers_exact_for_every_tiling(cfg):
+    # every partial sum is exact in fp32 => bit-exact against the oracle for any tile size/order
+    g = torch.Generator().manual_seed(3)
+    M, N, K_ = 320, 448, 256
+    a = torch.randint(-4, 5, (M, K_), generator=g).to(torch.bfloat16)
+    b = torch.randint(-4, 5, (K_, N), generator=g).to(torch.bfloat16)
+    c = K.matmul_tma(a.cuda(), b.cuda(), **cfg)
+    want = orc.matmul(bits(a), bits(b), BM=cfg["BLOCK_SIZE_M"], BN=cfg["BLOCK_SIZE_N"], BK=cfg["BLOCK_SIZE_K"],
+                      group_m=cfg["GROUP_SIZE_M"])
+    assert np.array_equal(bits(c), want)
+
+
+def test_matmul_ragged_shapes_strided_views_and_sentinel():
+    # descriptor zero-padding on loads, clipped stores, non-contiguous rows; sentinel proves
+    # nothing outside C[:M,:N] is written
+    M, N, K_ = 200, 136, 104
+    a, b = _ab(M + 8, N + 8, K_ + 8)
+    a, b = a.cuda()[:M, :K_], b.cuda()[:K_, :N]
+    cbuf = torch.full((M + 8, N + 8), 7.5, dtype=torch.bfloat16, device="cuda")
+    c = cbuf[:M, :N]
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+    K.matmul_kernel_tma[(K.cdiv(M, 64) * K.cdiv(N, 64), )](ad, bd, cd, M, N, K_, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64,
+                                                          BLOCK_SIZE_K=64, GROUP_SIZE_M=2, FP8_OUTPUT=False,
+                                                          WARP_SPECIALIZE=False)
+    _check(c, a.cpu(), b.cpu(), BM=64, BN=64, BK=64, group_m=2)
+    assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
+
+
+def test_matmul_partial_grid_runs_only_its_programs():
+    a, b = _ab(256, 256, 128)
+    c = torch.full((256, 256), 7.5, dtype=torch.bfloat16, device="cuda")
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a.cuda(), b.cuda(), c))
+    K.matmul_kernel_tma[(5, )](ad, bd, cd, 256, 256, 128, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64,
+                               GROUP_SIZE_M=2, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    want = np.full((256, 256), 0x40F0, dtype=np.uint16)
+    orc.matmul(bits(a), bits(b), BM=64, BN=64, BK=64, group_m=2, grid=5, out=want, acc64=True)
+    touched = want != 0x40F0
+    assert np.array_equal(bits(c) != 0x40F0, touched)
+    assert close_bf16(decode(c)[touched], orc.from_bf16(want)[touched], RTOL, ATOL)
+    with pytest.raises(ValueError):
+        K.matmul_kernel_tma[(17, )](ad, bd, cd, 256, 256, 128, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64,
+                                    GROUP_SIZE_M=2, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_full_bias_adds_in_half_after_the_cast(dtype):
+    M, N, K_ = 192, 256, 128
+    a, b = _ab(M, N, K_, dtype, seed=4)
+    bias = torch.randn(M, N, generator=torch.Generator().manual_seed(5)).to(dtype)
+    c = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda())
+    dt = ORC_DT[dtype]
+    ref = orc.decode(orc.matmul(bits(a), bits(b), in_dt=dt, out_dt=dt, bias=bits(bias), epi=orc.EPI_BIAS_FULL, acc64=True), dt)
+    assert close_bf16(decode(c), ref, RTOL, 1e-2)
+    # identity on the epilogue: exactly half(c0) + bias in the half type
+    c0 = K.matmul_tma(a.cuda(), b.cuda())
+    assert torch.equal(c, c0 + bias.cuda())
+
+
+def test_fused_row_bias_gelu():
+    # BASELINE's fused-epilogue config shape class; exact-erf GELU in fp32 on the accumulator
+    M, N, K_ = 256, 512, 256
+    a, b = _ab(M, N, K_, seed=6)
+    bias = torch.randn(N, generator=torch.Generator().manual_seed(7)) * 0.02
+    c = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda(), epilogue="gelu")
+    ref = orc.from_bf16(orc.matmul(bits(a), bits(b), bias=bias.numpy(), epi=orc.EPI_BIAS_ROW_GELU, acc64=True))
+    assert close_bf16(decode(c), ref, RTOL, ATOL)
+    tref = torch.nn.functional.gelu(a.double() @ b.double() + bias.double()).float().numpy()
+    assert close_bf16(decode(c), tref, RTOL, 1e-3)
+    c2 = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda(), epilogue="bias_row")
+    ref2 = orc.from_bf16(orc.matmul(bits(a), bits(b), bias=bias.numpy(), epi=orc.EPI_BIAS_ROW, acc64=True))
+    assert close_bf16(decode(c2), ref2, RTOL, ATOL)
+    c3 = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda(), epilogue="leaky_relu")
+    ref3 = orc.from_bf16(orc.matmul(bits(a), bits(b), epi=orc.EPI_LEAKY_RELU, acc64=True))
+    assert close_bf16(decode(c3), ref3, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("M,N,K_", [(64, 64, 64), (256, 384, 512), (1024, 1024, 1024)])
+def test_fp8_scaled(M, N, K_):
+    g = torch.Generator().manual_seed(8)
+    x, w = torch.randn(M, K_, generator=g), torch.randn(K_, N, generator=g)
+    qa, sa = K.quantize_fp8(x)
+    qb, sb = K.quantize_fp8(w)
+    # host quantiser agrees with the oracle's
+    oa, osa = orc.quantize_fp8(x.numpy())
+    assert np.array_equal(bits(qa), oa) and abs(sa - osa) <= 1e-9
+    c = K.matmul_fp8_scaled(qa.cuda(), qb.cuda(), sa, sb)
+    ref = orc.from_bf16(orc.matmul(bits(qa), bits(qb), in_dt=orc.FP8E4M3, out_dt=orc.BF16,
+                                   scale=float(np.float32(sa) * np.float32(sb)), acc64=True))
+    assert close_bf16(decode(c), ref, RTOL, 1e-3)
+    assert orc.pcc(ref, decode(c)) >= PCC
+
+
+def test_fp8_inputs_fp8_output_unscaled():
+    g = torch.Generator().manual_seed(9)
+    a = (torch.randn(128, 64, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    b = (torch.randn(64, 96, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    c = K.matmul_tma(a.cuda(), b.cuda(), BLOCK_SIZE_M=32, BLOCK_SIZE_N=32, BLOCK_SIZE_K=32, GROUP_SIZE_M=1)
+    assert c.dtype == torch.float8_e4m3fn
+    want = orc.matmul(bits(a), bits(b), in_dt=orc.FP8E4M3, out_dt=orc.FP8E4M3, BM=32, BN=32, BK=32, acc64=True)
+    got = bits(c)
+    # fp8 output: one e4m3 ulp of slack where fp32 vs fp64 accumulation straddles a rounding boundary
+    assert np.mean(got != want) < 0.02
+    assert np.max(np.abs(orc.from_fp8(got) - orc.from_fp8(want))) <= 0.125 * np.max(np.abs(orc.from_fp8(want)))
+
+
+def test_matmul_errors():
+    a, b = _ab(64, 64, 64)
+    with pytest.raises(NotImplementedError):
+        K.matmul_tma(a.cuda(), b.cuda(), BLOCK_SIZE_M=48, BLOCK_SIZE_N=64)   # not a multiple of 32
+    with pytest.raises(NotImplementedError):
+        K.matmul_tma(a.cuda().float(), b.cuda().float())
+    ad, bd = (TensorDescriptor.from_tensor(t.cuda(), [32, 32]) for t in (a, b))
+    c = torch.empty(64, 32, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        K.matmul_kernel_tma[(1, )](ad, bd, TensorDescriptor.from_tensor(c, [32, 32]), 64, 64, 64, FP8_OUTPUT=False,
+                                   WARP_SPECIALIZE=False)
+    assert rt.last_error() != ""

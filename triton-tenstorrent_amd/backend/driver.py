@@ -1,0 +1,478 @@
+"""Driver and launcher of the plugin surface, MI355X edition.
+
+Mirrors the reference's ``backend/driver.py``: ``TTUtils`` (:63-82),
+``TTLauncher`` (:85-170), ``TTDeviceInterface`` (:390-442) and ``TTDriver``
+(:445-535), with the knexus/ttrt device replaced by ``libttamd_rt.so``.  The
+launcher keeps the reference's call signature and argument walk, then binds the
+kernel NAME to the matching ``tt_*`` entry point of the C ABI.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import time
+from typing import Any, Callable
+
+from .. import runtime as rt
+from ..tensor_descriptor import is_tensor_descriptor
+
+try:  # Triton present: be a real DriverBase so set_active()/backends discovery accept us
+    from triton.backends.driver import DriverBase as _DriverBase
+    from triton.backends.compiler import GPUTarget
+    _HAVE_TRITON = True
+except Exception:  # C-ABI-only use
+    _HAVE_TRITON = False
+
+    class _DriverBase:  # type: ignore
+        def __init__(self) -> None:
+            pass
+
+    class GPUTarget:  # type: ignore
+        def __init__(self, backend, arch, warp_size):
+            self.backend, self.arch, self.warp_size = backend, arch, warp_size
+
+        def __repr__(self):
+            return f"GPUTarget(backend={self.backend!r}, arch={self.arch!r}, warp_size={self.warp_size})"
+
+
+BINARY_EXT = "ttamd"  # the "binary" of a kernel is a small JSON record naming the prebuilt kernel
+
+
+# --------------------------------------------------------------------------
+# signature handling
+# --------------------------------------------------------------------------
+def _typestr_dtype(ty: str) -> int:
+    """'*fp32' / '*bf16' / 'tensordesc<bf16[128,64]>' -> tt_dtype."""
+    t = ty
+    if t.startswith("tensordesc<"):
+        t = t[len("tensordesc<"):].split("[")[0]
+    t = t.lstrip("*")
+    if t not in rt.DTYPE_OF_TYPESTR:
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"element type {ty!r} has no kernel")
+    return rt.DTYPE_OF_TYPESTR[t]
+
+
+def _torch_dtype_code(t) -> int:
+    import torch
+    table = {torch.float32: rt.TT_F32, torch.int32: rt.TT_I32, torch.bfloat16: rt.TT_BF16,
+             torch.float16: rt.TT_F16, torch.float8_e4m3fn: rt.TT_FP8E4M3}
+    if t.dtype not in table:
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"tensor dtype {t.dtype} has no kernel")
+    return table[t.dtype]
+
+
+def flatten_launch_args(sig_types: list[str], args: tuple, ranks_out: list | None = None) -> list:
+    """The reference launcher's argument walk (backend/driver.py:134-164):
+    constexprs are skipped, a tensor contributes itself, a rank-r descriptor
+    contributes ``base, shape*r, strides*r, pad, shape*r, strides*r`` and
+    anything else is passed through.  The pad flag is 1 for ``padding == "nan"``
+    (driver.py:326).  ``ranks_out`` receives the rank of each descriptor met."""
+    flat: list = []
+    for ty, arg in zip(sig_types, args):
+        if ty == "constexpr":
+            continue
+        if is_tensor_descriptor(arg):
+            if ranks_out is not None:
+                ranks_out.append(len(arg.shape))
+            flat.append(arg.base)
+            flat.extend(int(d) for d in arg.shape)
+            flat.extend(int(s) for s in arg.strides)
+            flat.append(1 if arg.padding == "nan" else 0)
+            flat.extend(int(d) for d in arg.shape)
+            flat.extend(int(s) for s in arg.strides)
+        else:
+            flat.append(arg)
+    return flat
+
+
+class _Cursor:
+    """Reads the flattened argument list back in signature order."""
+
+    def __init__(self, flat: list, keep: list, ranks: list | None = None):
+        self.flat, self.i, self.keep = flat, 0, keep
+        self.ranks = list(ranks or [])
+
+    def _next(self):
+        v = self.flat[self.i]
+        self.i += 1
+        return v
+
+    def tensor(self, dtype_hint: int | None = None):
+        t = self._next()
+        if not hasattr(t, "data_ptr"):
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"expected a tensor argument, got {type(t).__name__}")
+        if not t.is_cuda:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "tensor arguments must live on the GPU")
+        self.keep.append(t)
+        return t
+
+    def scalar(self):
+        return self._next()
+
+    def desc(self) -> rt.tt_desc2d:
+        rank = self.ranks.pop(0) if self.ranks else 2
+        base = self.tensor()
+        shape = [self._next() for _ in range(rank)]
+        strides = [self._next() for _ in range(rank)]
+        pad = self._next()
+        shape2 = [self._next() for _ in range(rank)]
+        strides2 = [self._next() for _ in range(rank)]
+        assert shape == shape2 and strides == strides2
+        if rank == 1:  # a vector is the [1, n] matrix
+            shape, strides = [1, shape[0]], [shape[0], 1]
+        return rt.make_desc(base.data_ptr(), shape, strides, None, _torch_dtype_code(base),
+                            "nan" if pad else "zero")
+
+    def done(self):
+        if self.i != len(self.flat):
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID,
+                                   f"{len(self.flat) - self.i} launch arguments left over for this kernel")
+
+
+def _contiguous_1d(t):
+    if t.dim() > 1 and not t.is_contiguous():
+        raise ValueError("elementwise kernels index their operands linearly: pass contiguous tensors")  # driver.py:272-274
+    return t
+
+
+# --------------------------------------------------------------------------
+# kernel name -> C entry point
+# --------------------------------------------------------------------------
+def _bind_add(lib, cur: _Cursor, consts: dict, grid, stream):
+    x, y, out = cur.tensor(), cur.tensor(), cur.tensor()
+    n = int(cur.scalar())
+    block = int(consts["BLOCK_SIZE"])
+    for t in (x, y, out):
+        _contiguous_1d(t)
+    dt = _torch_dtype_code(x)
+    if _torch_dtype_code(y) != dt or _torch_dtype_code(out) != dt:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "add_kernel: operand dtypes differ")
+    if cur.i < len(cur.flat):  # loop variant carries row_count
+        row_count = int(cur.scalar())
+        cur.done()
+        return lib.tt_add_kernel_loop(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, row_count, block, dt, grid, stream)
+    return lib.tt_add_kernel(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, block, dt, grid, stream)
+
+
+def _bind_muladd(lib, cur, consts, grid, stream):
+    x, y, z, out = (_contiguous_1d(cur.tensor()) for _ in range(4))
+    n = int(cur.scalar())
+    cur.done()
+    for t in (x, y, z, out):
+        if _torch_dtype_code(t) != rt.TT_F32:
+            raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "muladd_kernel computes in fp32")
+    return lib.tt_muladd_kernel(x.data_ptr(), y.data_ptr(), z.data_ptr(), out.data_ptr(), n,
+                                int(consts["BLOCK_SIZE"]), grid, stream)
+
+
+def _bind_sin(lib, cur, consts, grid, stream):
+    x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
+    n = int(cur.scalar())
+    cur.done()
+    if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "sin_kernel computes in fp32")
+    return lib.tt_sin_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
+
+
+def _mnk(cur: _Cursor, a: rt.tt_desc2d, b: rt.tt_desc2d):
+    """M, N, K follow the descriptors when the signature carries them; the
+    minimal variant reads them from ``desc.shape`` (kernel_matmul_tma.py:71-75).
+    An int equal to 1 is specialised to a constexpr by Triton and is then
+    absent from the launch list; the caller passes those through consts."""
+    if cur.i < len(cur.flat):
+        return int(cur.scalar()), int(cur.scalar()), int(cur.scalar())
+    return a.shape[0], b.shape[1], a.shape[1]
+
+
+def _block_consts(consts: dict, a: rt.tt_desc2d):
+    bm = int(consts.get("BLOCK_SIZE_M", consts.get("BLOCK_M", 0)) or 0)
+    bn = int(consts.get("BLOCK_SIZE_N", consts.get("BLOCK_N", 0)) or 0)
+    bk = int(consts.get("BLOCK_SIZE_K", consts.get("BLOCK_K", 0)) or 0)
+    return bm, bn, bk, int(consts.get("GROUP_SIZE_M", 1) or 1)
+
+
+def _bind_matmul_tma(lib, cur, consts, grid, stream):
+    a, b, c = cur.desc(), cur.desc(), cur.desc()
+    M, N, K = _mnk(cur, a, b)
+    fp8_scaled = "scale_a" in consts or cur.i < len(cur.flat)
+    bm, bn, bk, g = _block_consts(consts, a)
+    if fp8_scaled:
+        sa = float(consts["scale_a"]) if "scale_a" in consts else float(cur.scalar())
+        sb = float(consts["scale_b"]) if "scale_b" in consts else float(cur.scalar())
+        cur.done()
+        return lib.tt_matmul_kernel_tma_fp8_scaled(C.byref(a), C.byref(b), C.byref(c), M, N, K, sa, sb, bm, bn, bk,
+                                                   g, grid, stream)
+    cur.done()
+    return lib.tt_matmul_kernel_tma(C.byref(a), C.byref(b), C.byref(c), M, N, K, bm, bn, bk, g, grid, stream)
+
+
+_EPILOGUES = {None: None, "": None, "bias": rt.TT_EPI_BIAS_FULL, "bias_full": rt.TT_EPI_BIAS_FULL,
+              "bias_row": rt.TT_EPI_BIAS_ROW, "bias_row_gelu": rt.TT_EPI_BIAS_ROW_GELU, "gelu": rt.TT_EPI_BIAS_ROW_GELU,
+              "leaky_relu": rt.TT_EPI_LEAKY_RELU}
+
+
+def _bind_matmul_fused(lib, cur, consts, grid, stream):
+    a, b, c, bias = cur.desc(), cur.desc(), cur.desc(), cur.desc()
+    M, N, K = _mnk(cur, a, b)
+    cur.done()
+    bm, bn, bk, g = _block_consts(consts, a)
+    epi = _EPILOGUES.get(consts.get("EPILOGUE"))
+    if epi is None:
+        # the reference kernel: full [M,N] bias of the output type; a [1,N]/[N] fp32 bias selects the row form
+        full = (bias.shape[0], bias.shape[1]) == (c.shape[0], c.shape[1]) and bias.dtype == c.dtype
+        epi = rt.TT_EPI_BIAS_FULL if full else rt.TT_EPI_BIAS_ROW
+    return lib.tt_matmul_kernel_fused(C.byref(a), C.byref(b), C.byref(c), C.byref(bias), M, N, K, bm, bn, bk, g, epi,
+                                      grid, stream)
+
+
+def _bind_attn_fwd(lib, cur, consts, grid, stream):
+    sm_scale = float(consts["sm_scale"]) if "sm_scale" in consts else float(cur.scalar())
+    M = cur.tensor()
+    Z = int(consts["Z"]) if "Z" in consts else int(cur.scalar())
+    H = int(consts["H"]) if "H" in consts else int(cur.scalar())
+    q, k, v, o = cur.desc(), cur.desc(), cur.desc(), cur.desc()
+    n_ctx = int(consts["N_CTX"]) if "N_CTX" in consts else int(cur.scalar())
+    cur.done()
+    if _torch_dtype_code(M) != rt.TT_F32:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "_attn_fwd: M must be fp32")
+    if M.numel() < Z * H * n_ctx or not M.is_contiguous():
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "_attn_fwd: M must be a contiguous [Z,H,N_CTX] tensor")
+    if consts.get("FP8_OUTPUT"):
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "_attn_fwd: FP8_OUTPUT is not supported")
+    return lib.tt_attn_fwd(sm_scale, M.data_ptr(), Z, H, C.byref(q), C.byref(k), C.byref(v), C.byref(o), n_ctx,
+                           int(consts["HEAD_DIM"]), int(consts["BLOCK_M"]), int(consts["BLOCK_N"]),
+                           int(consts["STAGE"]), grid, stream)
+
+
+KERNEL_TABLE: dict[str, Callable] = {
+    "add_kernel": _bind_add,
+    "muladd_kernel": _bind_muladd,
+    "sin_kernel": _bind_sin,
+    "matmul_kernel_tma": _bind_matmul_tma,
+    "matmul_kernel_tma_fp8_scaled": _bind_matmul_tma,
+    "matmul_kernel_fused": _bind_matmul_fused,
+    "_attn_fwd": _bind_attn_fwd,
+}
+
+
+class BoundKernel:
+    """What ``load_binary`` hands back as ``function``: the kernel name and its binder."""
+
+    def __init__(self, name: str, record: dict):
+        if name not in KERNEL_TABLE:
+            raise rt.RuntimeError_(rt.RT_ERR_NOT_FOUND, f"no prebuilt kernel named {name!r}; have {sorted(KERNEL_TABLE)}")
+        self.name = name
+        self.record = record
+        self.bind = KERNEL_TABLE[name]
+
+    def __repr__(self):
+        return f"<BoundKernel {self.name}>"
+
+
+# --------------------------------------------------------------------------
+# reference classes
+# --------------------------------------------------------------------------
+class TTUtils:
+    """load_binary / get_device_properties (backend/driver.py:63-82)."""
+
+    def __init__(self, driver: "TTDriver"):
+        self.driver = driver
+
+    def load_binary(self, name, kernel, shared_mem, device_id):
+        rt.init(int(device_id or 0))
+        record = json.loads(kernel.decode() if isinstance(kernel, (bytes, bytearray)) else kernel) if kernel else {}
+        fn = BoundKernel(record.get("kernel", name), record)
+        # (module, function, n_regs, n_spills, n_max_threads); Triton checks
+        # num_warps * warp_size <= n_max_threads
+        return (rt.load(), fn, 0, 0, 1024)
+
+    def get_device_properties(self, *args):
+        p = rt.device_props()
+        return {"max_num_regs": p["max_num_regs"], "max_shared_mem": p["max_shared_mem"],
+                "multiprocessor_count": p["multiprocessor_count"], "warpSize": p["warp_size"],
+                "sm_clock_rate": p["clock_khz"], "mem_clock_rate": p["mem_clock_khz"], "mem_bus_width": p["mem_bus_bits"],
+                "arch": p["arch"], "name": p["name"]}
+
+
+class TTLauncher:
+    """``__init__(src, metadata)`` / ``__call__(gridX, gridY, gridZ, stream,
+    function, packed_metadata, launch_metadata, enter_hook, exit_hook, *args)``
+    (backend/driver.py:87-111)."""
+
+    def __init__(self, src, metadata):
+        constants = src.constants if hasattr(src, "constants") else dict()
+        arg_names = list(src.fn.arg_names)
+        arg_idx = lambda x: (arg_names.index(x), ) if isinstance(x, str) else x
+        self.constants = {arg_idx(idx): value for idx, value in constants.items()}
+        self.signature = {idx: value for idx, value in src.signature.items()}
+        self.arg_names = arg_names
+        self.keepalive: list = []
+
+    def __call__(self, gridX, gridY, gridZ, stream, function, *args):
+        kernel_metadata, launch_metadata, launch_enter_hook, launch_exit_hook = args[0], args[1], args[2], args[3]
+        del kernel_metadata  # num_warps / shared describe Triton codegen; the prebuilt kernels fix their own
+        user_args = args[4:]
+        sig_types = list(self.signature.values())
+        if len(user_args) != len(sig_types):
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID,
+                                   f"{function.name}: {len(user_args)} arguments for a {len(sig_types)}-entry signature")
+        ranks: list = []
+        flat = flatten_launch_args(sig_types, user_args, ranks)
+        # constexprs by name: explicit constexpr parameters plus ints Triton specialised away (value 1)
+        consts = {}
+        for name, ty, val in zip(self.arg_names, sig_types, user_args):
+            if ty == "constexpr":
+                consts[name] = val
+        for idx, val in self.constants.items():
+            if len(idx) == 1 and idx[0] < len(self.arg_names):
+                consts.setdefault(self.arg_names[idx[0]], val)
+        keep: list = []
+        cur = _Cursor(flat, keep, ranks)
+        lib = rt.init(0)
+        grid = rt.grid3(gridX, gridY, gridZ)
+        if launch_enter_hook is not None:
+            launch_enter_hook(launch_metadata)
+        rc = function.bind(lib, cur, consts, grid, C.c_void_p(int(stream or 0)))
+        rt.check(rc)
+        # launches are asynchronous: keep operands referenced until the next launch replaces them
+        self.keepalive = keep
+        if launch_exit_hook is not None:
+            launch_exit_hook(launch_metadata)
+
+
+class TTDeviceInterface:
+    """What ``triton.testing.do_bench`` drives (backend/driver.py:390-442):
+    ``Event(enable_timing)``, ``synchronize()``, optional hook timing.  Events
+    are hipEvents on the current torch stream."""
+
+    class HooksTimeAccessor:
+
+        def __init__(self, di):
+            self.di = di
+            self.record_idx = 0
+
+        def elapsed_time(self, end_event) -> float:
+            return sum(self.di.kernel_times[self.record_idx:end_event.record_idx]) * 1000
+
+        def record(self):
+            self.record_idx = len(self.di.kernel_times)
+
+    class DeviceEvent:
+
+        def __init__(self):
+            self.ev = rt.Event()
+
+        def record(self):
+            import torch
+            self.ev.record(torch.cuda.current_stream().cuda_stream)
+
+        def elapsed_time(self, end_event) -> float:
+            return self.ev.elapsed_time(end_event.ev)
+
+        def synchronize(self):
+            self.ev.synchronize()
+
+    def __init__(self):
+        self.kernel_times: list[float] = []
+        self.last_start = 0.0
+        self.use_hooks = False
+
+    def enable_hook_timing(self):
+        self.use_hooks = True
+        if _HAVE_TRITON:
+            import triton
+            triton.compiler.CompiledKernel.launch_enter_hook = lambda arg: self._enter_hook()
+            triton.compiler.CompiledKernel.launch_exit_hook = lambda arg: self._exit_hook()
+
+    def synchronize(self):
+        import torch
+        torch.cuda.synchronize()
+
+    def _enter_hook(self):
+        self.synchronize()
+        self.last_start = time.perf_counter()
+
+    def _exit_hook(self):
+        self.synchronize()
+        self.kernel_times.append(time.perf_counter() - self.last_start)
+
+    def Event(self, enable_timing=True):
+        if self.use_hooks:
+            return TTDeviceInterface.HooksTimeAccessor(self)
+        return TTDeviceInterface.DeviceEvent()
+
+
+class TTDriver(_DriverBase):
+    """backend/driver.py:445-535 on an MI355X."""
+
+    @staticmethod
+    def is_active():
+        try:
+            import torch
+            return bool(torch.cuda.is_available()) and rt.LIB_PATH.exists()
+        except Exception:
+            return False
+
+    def __init__(self):
+        super().__init__()
+        self.utils = TTUtils(self)
+        self.launcher_cls = TTLauncher
+
+    def get_device(self, device_id=0):
+        return device_id
+
+    def get_current_device(self):
+        import torch
+        return torch.cuda.current_device()
+
+    def set_current_device(self, device):
+        import torch
+        torch.cuda.set_device(device)
+
+    def get_current_stream(self, device_id=None):
+        import torch
+        return torch.cuda.current_stream(device_id).cuda_stream
+
+    def get_device_interface(self):
+        return TTDeviceInterface()
+
+    def get_current_target(self):
+        # same backend name as the reference (driver.py:509-512) so that
+        # TTBackend.supports_target and `--target tenstorrent:...` keep working;
+        # arch and wavefront size are the MI355X's
+        return GPUTarget("tenstorrent", "gfx950", 64)
+
+    def get_active_torch_device(self):
+        import torch
+        return torch.device("cuda", self.get_current_device())
+
+    def map_python_to_cpp_type(self, ty: str) -> str:
+        return ty
+
+    def get_benchmarker(self):
+        from triton.testing import do_bench
+        return do_bench
+
+    def get_empty_cache_for_benchmark(self):
+        import torch
+        # 512 MiB: twice the 256 MiB last-level cache, so a clear really evicts
+        return torch.empty(512 * 1024 * 1024 // 4, dtype=torch.int, device="cuda")
+
+    def clear_cache(self, cache):
+        cache.zero_()
+
+    def get_empty_device_buffer(self, size, dtype):
+        """Output allocation used by the loop/mul-add tutorials
+        (python/tutorials/01-vector-add.loop.py:70)."""
+        import torch
+        return torch.empty(size, dtype=dtype, device="cuda")
+
+
+def activate() -> TTDriver:
+    """Make this driver Triton's active one (Triton allows a single active
+    driver; on a ROCm box the stock HIP driver would otherwise win)."""
+    drv = TTDriver()
+    if _HAVE_TRITON:
+        import triton
+        triton.runtime.driver.set_active(drv)
+    return drv

@@ -1,0 +1,72 @@
+"""Build recipe: gfx950 code objects (hipcc --genco) and libttamd_rt.so.
+
+    python -m triton_tenstorrent_amd.build        # rebuild everything
+
+Every kernels/*.hip becomes one code object under build/, and the host runtime
+embeds them, so the shared library is the only file that has to travel.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+ROOT = PKG.parent
+CSRC = PKG / "csrc"
+BUILD = PKG / "build"
+LIB = PKG / "lib" / "libttamd_rt.so"
+ARCH = "gfx950"
+
+CODE_OBJECTS = ["elementwise", "gemm", "attention"]
+RT_SOURCES = ["ttamd_rt.cpp", "tt_elementwise.cpp", "tt_gemm.cpp", "tt_attention.cpp"]
+
+# -packed-fp32-ops off: the compiler must not form v_pk_*_f32 on this target
+DEVICE_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-ffp-contract=on", "-fno-fast-math", "-Wall", "-Wno-unused-function"]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found; the runtime cannot be built without ROCm")
+    return exe
+
+
+def _run(cmd: list[str]) -> None:
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
+        raise RuntimeError(f"build step failed: {cmd[0]} ... {cmd[-1]}")
+    noise = [l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip()]
+    if noise and os.environ.get("TTAMD_BUILD_VERBOSE"):
+        sys.stderr.write("\n".join(noise) + "\n")
+
+
+def build_code_object(name: str, extra: list[str] | None = None) -> Path:
+    BUILD.mkdir(exist_ok=True)
+    out = BUILD / f"{name}.hsaco"
+    _run([hipcc(), "--genco", *DEVICE_FLAGS, *(extra or []), str(CSRC / "kernels" / f"{name}.hip"), "-o", str(out)])
+    return out
+
+
+def build_runtime() -> Path:
+    LIB.parent.mkdir(exist_ok=True)
+    cmd = [hipcc(), "-shared", "-fPIC", "-O2", "-std=c++17", "-fvisibility=hidden", "-Wall",
+           f"-I{ROOT / 'include'}", f"-I{CSRC / 'rt'}", f'-DTTAMD_CO_DIR="{BUILD}"',
+           *[str(CSRC / "rt" / s) for s in RT_SOURCES], "-o", str(LIB)]
+    _run(cmd)
+    return LIB
+
+
+def build_all(jobs: int = 4) -> Path:
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(build_code_object, CODE_OBJECTS))
+    return build_runtime()
+
+
+if __name__ == "__main__":
+    print(build_all())

@@ -1,0 +1,218 @@
+// Elementwise streaming kernels for gfx950: add_kernel (fp32 / int32),
+// muladd_kernel, sin_kernel.
+//
+// Each follows the masked-block semantics of the example kernel sources
+// (python/tutorials/01-vector-add.py:29-54, 01-vector-mul-add.py:30-57,
+//  examples/01-sin-kernel.py:17-29): logical program pid owns BLOCK consecutive
+// elements, lanes at or past n are masked.  The host folds grid and BLOCK into
+// one bound n_eff = min(n, grid*BLOCK); the kernels touch exactly [0, n_eff).
+//
+// HBM-bound: 16-byte loads and stores per lane, UNROLL independent vectors in
+// flight per lane, a grid-stride loop over a grid sized to the CU count.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace {
+
+constexpr int kThreads = 256;
+
+template <typename T> struct Vec4 { typedef T type __attribute__((ext_vector_type(4))); };
+
+struct AddOp {
+  template <typename T> __device__ static T apply(T a, T b) { return a + b; }
+};
+struct AddWrapOp {  // int32: two's-complement wraparound without signed-overflow UB
+  __device__ static int apply(int a, int b) { return (int)((unsigned)a + (unsigned)b); }
+};
+
+template <typename T, typename Op, int UNROLL>
+__device__ __forceinline__ void binary_body(const T *__restrict__ x, const T *__restrict__ y,
+                                            T *__restrict__ out, uint32_t n) {
+  using V = typename Vec4<T>::type;
+  const uint32_t nvec = n >> 2;
+  const uint32_t stride = gridDim.x * kThreads;
+  const V *xv = reinterpret_cast<const V *>(x);
+  const V *yv = reinterpret_cast<const V *>(y);
+  V *ov = reinterpret_cast<V *>(out);
+  uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  // full groups of UNROLL vectors: no per-vector bounds checks
+  for (; (uint64_t)i + (uint64_t)(UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+    V a[UNROLL], b[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) b[u] = __builtin_nontemporal_load(yv + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      V r;
+      r.x = Op::apply(a[u].x, b[u].x);
+      r.y = Op::apply(a[u].y, b[u].y);
+      r.z = Op::apply(a[u].z, b[u].z);
+      r.w = Op::apply(a[u].w, b[u].w);
+      __builtin_nontemporal_store(r, ov + i + u * stride);
+    }
+  }
+  for (; i < nvec; i += stride) {
+    V a = xv[i], b = yv[i], r;
+    r.x = Op::apply(a.x, b.x);
+    r.y = Op::apply(a.y, b.y);
+    r.z = Op::apply(a.z, b.z);
+    r.w = Op::apply(a.w, b.w);
+    ov[i] = r;
+  }
+  // scalar tail: the last n % 4 elements
+  if (blockIdx.x == 0) {
+    uint32_t t = (nvec << 2) + threadIdx.x;
+    if (t < n) out[t] = Op::apply(x[t], y[t]);
+  }
+}
+
+template <typename T, typename Op>
+__device__ __forceinline__ void binary_scalar_body(const T *x, const T *y, T *out, uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
+    out[i] = Op::apply(x[i], y[i]);
+}
+
+// ---- sin ------------------------------------------------------------------
+// k = rint(x * 2/pi); r = x - k*pi/2 by a three-constant Cody-Waite reduction
+// carried out with fused multiply-adds (each k*piece product enters the fma
+// unrounded); minimax polynomials for sin and
+// cos on [-pi/4, pi/4]; quadrant select.  Valid while k*pi/2's third piece
+// still resolves the result: |x| < 2^17 here, beyond that the library routine
+// with its full Payne-Hanek reduction takes over (a wave-uniform rarity).
+__device__ __forceinline__ float sin_fast(float x) {
+  const float two_over_pi = 0.636619772367581343f;
+  const float p1 = 1.5707963705062866f;     // fp32(pi/2)
+  const float p2 = -4.371138828673793e-08f;  // fp32(pi/2 - p1)
+  const float p3 = -1.7151245100058819e-15f; // fp32(pi/2 - p1 - p2)
+  float kf = __builtin_rintf(x * two_over_pi);
+  float r = __builtin_fmaf(-kf, p1, x);
+  r = __builtin_fmaf(-kf, p2, r);
+  r = __builtin_fmaf(-kf, p3, r);
+  int q = (int)kf;
+  float r2 = r * r;
+  // sin(r) = r + r^3 * S(r^2)
+  float s = __builtin_fmaf(r2, 2.7183114939898219064e-06f, -1.98393348360966317347e-04f);
+  s = __builtin_fmaf(s, r2, 8.3333293858894631756e-03f);
+  s = __builtin_fmaf(s, r2, -1.66666666416265235595e-01f);
+  s = __builtin_fmaf(s * r2, r, r);
+  // cos(r) = 1 + r^2 * C(r^2)
+  float c = __builtin_fmaf(r2, 2.43904487962774090654e-05f, -1.38867637746099294692e-03f);
+  c = __builtin_fmaf(c, r2, 4.16666233237390631894e-02f);
+  c = __builtin_fmaf(c, r2, -4.99999997251031003120e-01f);
+  c = __builtin_fmaf(c, r2, 1.0f);
+  float v = (q & 1) ? c : s;
+  return (q & 2) ? -v : v;
+}
+
+__device__ __forceinline__ float sin_any(float x) {
+  return (__builtin_fabsf(x) < 131072.0f) ? sin_fast(x) : sinf(x);
+}
+
+template <int UNROLL>
+__device__ __forceinline__ void sin_body(const float *__restrict__ x, float *__restrict__ out,
+                                         uint32_t n) {
+  using V = Vec4<float>::type;
+  const uint32_t nvec = n >> 2;
+  const uint32_t stride = gridDim.x * kThreads;
+  const V *xv = reinterpret_cast<const V *>(x);
+  V *ov = reinterpret_cast<V *>(out);
+  uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  for (; (uint64_t)i + (uint64_t)(UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+    V a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      V r;
+      r.x = sin_any(a[u].x);
+      r.y = sin_any(a[u].y);
+      r.z = sin_any(a[u].z);
+      r.w = sin_any(a[u].w);
+      __builtin_nontemporal_store(r, ov + i + u * stride);
+    }
+  }
+  for (; i < nvec; i += stride) {
+    V a = xv[i], r;
+    r.x = sin_any(a.x);
+    r.y = sin_any(a.y);
+    r.z = sin_any(a.z);
+    r.w = sin_any(a.w);
+    ov[i] = r;
+  }
+  if (blockIdx.x == 0) {
+    uint32_t t = (nvec << 2) + threadIdx.x;
+    if (t < n) out[t] = sin_any(x[t]);
+  }
+}
+
+struct MulAdd {
+  __device__ static float apply(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+};
+
+} // namespace
+
+extern "C" {
+
+// 16-byte aligned operands
+__global__ __launch_bounds__(kThreads) void ew_add_f32(const float *x, const float *y, float *out,
+                                                       uint32_t n) {
+  binary_body<float, AddOp, 4>(x, y, out, n);
+}
+__global__ __launch_bounds__(kThreads) void ew_add_i32(const int *x, const int *y, int *out,
+                                                       uint32_t n) {
+  binary_body<int, AddWrapOp, 4>(x, y, out, n);
+}
+// any alignment (4-byte)
+__global__ __launch_bounds__(kThreads) void ew_add_f32_unaligned(const float *x, const float *y,
+                                                                 float *out, uint32_t n) {
+  binary_scalar_body<float, AddOp>(x, y, out, n);
+}
+__global__ __launch_bounds__(kThreads) void ew_add_i32_unaligned(const int *x, const int *y,
+                                                                 int *out, uint32_t n) {
+  binary_scalar_body<int, AddWrapOp>(x, y, out, n);
+}
+
+__global__ __launch_bounds__(kThreads) void ew_sin_f32(const float *x, float *out, uint32_t n) {
+  sin_body<4>(x, out, n);
+}
+__global__ __launch_bounds__(kThreads) void ew_sin_f32_unaligned(const float *x, float *out,
+                                                                 uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = sin_any(x[i]);
+}
+
+__global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restrict__ x,
+                                                          const float *__restrict__ y,
+                                                          const float *__restrict__ z,
+                                                          float *__restrict__ out, uint32_t n,
+                                                          uint32_t aligned) {
+  using V = Vec4<float>::type;
+  const uint32_t stride = gridDim.x * kThreads;
+  if (aligned) {
+    const uint32_t nvec = n >> 2;
+    const V *xv = reinterpret_cast<const V *>(x);
+    const V *yv = reinterpret_cast<const V *>(y);
+    const V *zv = reinterpret_cast<const V *>(z);
+    V *ov = reinterpret_cast<V *>(out);
+    for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
+      V a = __builtin_nontemporal_load(xv + i), b = __builtin_nontemporal_load(yv + i),
+        c = __builtin_nontemporal_load(zv + i), r;
+      r.x = MulAdd::apply(a.x, b.x, c.x);
+      r.y = MulAdd::apply(a.y, b.y, c.y);
+      r.z = MulAdd::apply(a.z, b.z, c.z);
+      r.w = MulAdd::apply(a.w, b.w, c.w);
+      __builtin_nontemporal_store(r, ov + i);
+    }
+    if (blockIdx.x == 0) {
+      uint32_t t = (nvec << 2) + threadIdx.x;
+      if (t < n) out[t] = MulAdd::apply(x[t], y[t], z[t]);
+    }
+  } else {
+    for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
+      out[i] = MulAdd::apply(x[i], y[i], z[i]);
+  }
+}
+
+} // extern "C"

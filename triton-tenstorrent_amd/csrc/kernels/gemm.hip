@@ -1,0 +1,102 @@
+// Tile-matmul kernels for gfx950: matmul_kernel_tma, matmul_kernel_fused and the
+// fp8-scaled sibling
+// (examples/matmul_tensor_descriptor/09-persistent-matmul.py:102-145,
+//  python/tutorials/09-matmul-fused.py:100-148).
+//
+// gemm_any_*   : every shape, stride, tile size (multiples of 32), partial
+//                logical grid, ragged edges with descriptor zero-padding and
+//                clipped stores.  One wavefront owns one 32x32 piece of a
+//                logical tile and walks K with v_mfma_f32_32x32x16, operands
+//                straight from global memory.  Correctness path, not a fast one.
+#include "gemm_common.h"
+
+namespace {
+
+// Operand fragment of v_mfma_f32_32x32x16_{bf16,f16}: lane l holds row (A) or
+// column (B) l%32 and the 8 consecutive k of group l/32.
+template <int IN_DT> struct Frag;
+template <> struct Frag<DT_BF16> {
+  typedef bf16x8 vec;
+  static __device__ __forceinline__ uint16_t enc(const void *p, int64_t i) { return ((const uint16_t *)p)[i]; }
+  static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Frag<DT_F16> {
+  typedef f16x8 vec;
+  static __device__ __forceinline__ uint16_t enc(const void *p, int64_t i) { return ((const uint16_t *)p)[i]; }
+  static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+// e4m3 values are exactly representable in bf16 (3 mantissa bits, narrower
+// exponent range), so the any-shape path widens them and reuses the bf16 MFMA.
+template <> struct Frag<DT_FP8> {
+  typedef bf16x8 vec;
+  static __device__ __forceinline__ uint16_t enc(const void *p, int64_t i) {
+    return (uint16_t)(f32_bits(fp8_to_f32(((const uint8_t *)p)[i])) >> 16);
+  }
+  static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <int IN_DT, int OUT_DT> __device__ __forceinline__ void gemm_any_body(const GemmArgs &g) {
+  using F = Frag<IN_DT>;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int waves_per_block = blockDim.x >> 6;
+  const int sub_n = g.BN >> 5;
+  const int spt = (g.BM >> 5) * sub_n; // 32x32 pieces per logical tile
+  const int64_t items = (int64_t)g.grid * spt;
+  const int64_t stride = (int64_t)gridDim.x * waves_per_block;
+  const int r32 = lane & 31, kg = lane >> 5;
+  for (int64_t it = (int64_t)blockIdx.x * waves_per_block + wave; it < items; it += stride) {
+    const int pid = (int)(it / spt), sub = (int)(it % spt);
+    int pid_m, pid_n;
+    tile_of_pid(pid, g.num_pid_m, g.num_pid_n, g.group_m, pid_m, pid_n);
+    const int64_t m0 = (int64_t)pid_m * g.BM + (sub / sub_n) * 32;
+    const int64_t n0 = (int64_t)pid_n * g.BN + (sub % sub_n) * 32;
+    if (m0 >= g.M || n0 >= g.N) continue; // piece lies wholly in the padding (wave-uniform)
+    const int64_t am = m0 + r32, bn = n0 + r32;
+    const bool am_ok = am < g.M, bn_ok = bn < g.N;
+    f32x16 acc = {0};
+    for (int k0 = 0; k0 < g.K; k0 += 16) {
+      union { typename F::vec v; uint16_t s[8]; } a, b;
+      const int kb = k0 + kg * 8;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = kb + j;
+        const bool k_ok = k < g.K;
+        a.s[j] = (am_ok && k_ok) ? F::enc(g.a, am * g.lda + k) : (uint16_t)0;
+        b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, (int64_t)k * g.ldb + bn) : (uint16_t)0;
+      }
+      acc = F::mfma(a.v, b.v, acc);
+    }
+    // accumulator register r of lane l is C[(r/4)*8 + (l/32)*4 + r%4][l%32]
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int64_t m = m0 + (r >> 2) * 8 + kg * 4 + (r & 3);
+      const int64_t n = n0 + r32;
+      if (m < g.M && n < g.N) {
+        float v = apply_epilogue<OUT_DT>(g, acc[r] * g.scale, m, n);
+        store_from_f32<OUT_DT>(g.c, m * g.ldc + n, v);
+      }
+    }
+  }
+}
+
+} // namespace
+
+extern "C" {
+
+#define GEMM_ANY(name, IN, OUT)                                                        \
+  __global__ __launch_bounds__(256) void name(GemmArgs g) { gemm_any_body<IN, OUT>(g); }
+
+GEMM_ANY(gemm_any_bf16_bf16, DT_BF16, DT_BF16)
+GEMM_ANY(gemm_any_f16_f16, DT_F16, DT_F16)
+GEMM_ANY(gemm_any_fp8_bf16, DT_FP8, DT_BF16)
+GEMM_ANY(gemm_any_fp8_f16, DT_FP8, DT_F16)
+GEMM_ANY(gemm_any_fp8_fp8, DT_FP8, DT_FP8)
+
+} // extern "C"

@@ -1,0 +1,19 @@
+// Argument block shared by the tile-matmul kernels and their host launcher.
+#pragma once
+#include <stdint.h>
+
+// One argument block for every tile-matmul kernel (passed by value).
+struct GemmArgs {
+  const void *a;    // [M,K] row-major, leading stride lda (elements)
+  const void *b;    // [K,N] row-major, leading stride ldb
+  void *c;          // [M,N] row-major, leading stride ldc
+  const void *bias; // [M,N] of the output type (EPI_BIAS_FULL) or fp32 [N] (row forms)
+  int64_t lda, ldb, ldc, ldbias;
+  int32_t M, N, K;
+  int32_t BM, BN, BK;       // logical tile of one program
+  int32_t group_m;          // GROUP_SIZE_M
+  int32_t grid;             // number of logical programs
+  int32_t num_pid_m, num_pid_n;
+  int32_t epi;
+  float scale;              // multiplies the accumulator before the cast
+};

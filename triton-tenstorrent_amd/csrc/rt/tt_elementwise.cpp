@@ -1,0 +1,122 @@
+// tt_add_kernel / tt_add_kernel_loop / tt_muladd_kernel / tt_sin_kernel:
+// launch validation and binding to the streaming kernels of elementwise.hip.
+#include <algorithm>
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <string>
+
+#include "tt_internal.h"
+
+namespace ttamd {
+
+int env_int(const char *name, int dflt) {
+  static std::mutex mu;
+  static std::map<std::string, int> cache;
+  std::lock_guard<std::mutex> lk(mu);
+  auto it = cache.find(name);
+  if (it != cache.end()) return it->second;
+  const char *v = getenv(name);
+  int r = (v && *v) ? atoi(v) : dflt;
+  cache[name] = r;
+  return r;
+}
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kUnroll = 4;
+
+// Elements the logical grid covers: programs 0..grid-1 own `per_program`
+// consecutive elements each, clipped by the n_elements mask.
+int check_1d(const char *who, int32_t n, int64_t per_program, const uint32_t grid[3],
+             uint32_t *n_eff) {
+  if (!grid) return fail(RT_ERR_INVALID, "%s: null grid", who);
+  if (n < 0) return fail(RT_ERR_INVALID, "%s: n_elements %d < 0", who, n);
+  if (per_program <= 0) return fail(RT_ERR_INVALID, "%s: BLOCK_SIZE must be positive", who);
+  if (grid[1] != 1 || grid[2] != 1)
+    return fail(RT_ERR_INVALID, "%s: 1-D grid expected, got (%u,%u,%u)", who, grid[0], grid[1],
+                grid[2]);
+  int64_t covered = (int64_t)grid[0] * per_program;
+  *n_eff = (uint32_t)std::min<int64_t>(n, covered);
+  return RT_OK;
+}
+
+// Persistent physical grid: enough workgroups to fill every CU, never more
+// than there are UNROLL-vector groups to stream.
+uint32_t streaming_grid(uint32_t n_eff) {
+  const rt_props *p = props();
+  int wg_per_cu = env_int("TTAMD_EW_WG_PER_CU", 8);
+  int64_t cap = (int64_t)p->multiprocessor_count * wg_per_cu;
+  int64_t need = cdiv64((int64_t)n_eff, (int64_t)kThreads * 4 * kUnroll);
+  return (uint32_t)std::max<int64_t>(1, std::min(cap, need));
+}
+
+} // namespace
+} // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" {
+
+static int add_common(const char *who, const void *x, const void *y, void *out, int32_t n,
+                      int64_t per_program, int32_t dtype, const uint32_t grid[3], void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "%s: call rt_init first", who);
+  if (dtype != TT_F32 && dtype != TT_I32)
+    return fail(RT_ERR_UNSUPPORTED, "%s: dtype %d (fp32 and int32 are supported)", who, dtype);
+  uint32_t n_eff = 0;
+  int rc = check_1d(who, n, per_program, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK; // nothing to do, nothing to touch
+  if (!x || !y || !out) return fail(RT_ERR_INVALID, "%s: null tensor pointer", who);
+  bool al = aligned16(x) && aligned16(y) && aligned16(out);
+  const char *name = dtype == TT_F32 ? (al ? "ew_add_f32" : "ew_add_f32_unaligned")
+                                     : (al ? "ew_add_i32" : "ew_add_i32_unaligned");
+  void *args[] = {&x, &y, &out, &n_eff};
+  return launch("elementwise", name, dim3(streaming_grid(n_eff)), dim3(kThreads), 0, stream, args, 4);
+}
+
+int tt_add_kernel(const void *x, const void *y, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
+                  int32_t dtype, const uint32_t grid[3], void *stream) {
+  return add_common("add_kernel", x, y, out, n_elements, BLOCK_SIZE, dtype, grid, stream);
+}
+
+int tt_add_kernel_loop(const void *x, const void *y, void *out, int32_t n_elements,
+                       int32_t row_count, int32_t BLOCK_SIZE, int32_t dtype, const uint32_t grid[3],
+                       void *stream) {
+  if (row_count < 0) return fail(RT_ERR_INVALID, "add_kernel: row_count %d < 0", row_count);
+  if (row_count == 0) return RT_OK; // every program's range is empty
+  if (BLOCK_SIZE <= 0) return fail(RT_ERR_INVALID, "add_kernel: BLOCK_SIZE must be positive");
+  return add_common("add_kernel", x, y, out, n_elements, (int64_t)BLOCK_SIZE * row_count, dtype,
+                    grid, stream);
+}
+
+int tt_muladd_kernel(const void *x, const void *y, const void *z, void *out, int32_t n_elements,
+                     int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "muladd_kernel: call rt_init first");
+  uint32_t n_eff = 0;
+  int rc = check_1d("muladd_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !y || !z || !out) return fail(RT_ERR_INVALID, "muladd_kernel: null tensor pointer");
+  uint32_t al = aligned16(x) && aligned16(y) && aligned16(z) && aligned16(out);
+  void *args[] = {&x, &y, &z, &out, &n_eff, &al};
+  return launch("elementwise", "ew_muladd_f32", dim3(streaming_grid(n_eff)), dim3(kThreads), 0,
+                stream, args, 6);
+}
+
+int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
+                  const uint32_t grid[3], void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "sin_kernel: call rt_init first");
+  uint32_t n_eff = 0;
+  int rc = check_1d("sin_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !out) return fail(RT_ERR_INVALID, "sin_kernel: null tensor pointer");
+  bool al = aligned16(x) && aligned16(out);
+  void *args[] = {&x, &out, &n_eff};
+  return launch("elementwise", al ? "ew_sin_f32" : "ew_sin_f32_unaligned",
+                dim3(streaming_grid(n_eff)), dim3(kThreads), 0, stream, args, 3);
+}
+
+} // extern "C"

@@ -1,0 +1,137 @@
+// tt_matmul_kernel_tma / tt_matmul_kernel_fused / tt_matmul_kernel_tma_fp8_scaled:
+// launch validation and kernel selection for the tile-matmul family.
+#include <algorithm>
+#include <cstring>
+
+#include "tt_internal.h"
+#include "../kernels/gemm_args.h"
+
+using namespace ttamd;
+
+namespace {
+
+int check_desc(const char *who, const char *what, const tt_desc2d *d, int64_t rows, int64_t cols) {
+  if (!d) return fail(RT_ERR_INVALID, "%s: null %s descriptor", who, what);
+  if (!d->base) return fail(RT_ERR_INVALID, "%s: %s descriptor has a null base", who, what);
+  if (dtype_size(d->dtype) == 0 || d->dtype == TT_I32)
+    return fail(RT_ERR_UNSUPPORTED, "%s: %s dtype %d", who, what, d->dtype);
+  if (d->padding_nan)
+    return fail(RT_ERR_UNSUPPORTED, "%s: %s descriptor asks for NaN padding; only zero padding exists",
+                who, what);
+  if (d->strides[1] != 1)
+    return fail(RT_ERR_INVALID, "%s: %s descriptor's last stride is %lld, must be 1", who, what,
+                (long long)d->strides[1]);
+  if (d->shape[0] != rows || d->shape[1] != cols)
+    return fail(RT_ERR_INVALID, "%s: %s descriptor is [%d,%d], the launch says [%lld,%lld]", who, what,
+                d->shape[0], d->shape[1], (long long)rows, (long long)cols);
+  if (d->strides[0] < cols)
+    return fail(RT_ERR_INVALID, "%s: %s leading stride %lld < row length %lld", who, what,
+                (long long)d->strides[0], (long long)cols);
+  if (reinterpret_cast<uintptr_t>(d->base) % dtype_size(d->dtype))
+    return fail(RT_ERR_INVALID, "%s: %s base is not aligned to its element size", who, what);
+  return RT_OK;
+}
+
+int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c,
+               const tt_desc2d *bias, int32_t M, int32_t N, int32_t K, int32_t BM, int32_t BN,
+               int32_t BK, int32_t group_m, int32_t epi, float scale, const uint32_t grid[3],
+               void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "%s: call rt_init first", who);
+  if (!grid) return fail(RT_ERR_INVALID, "%s: null grid", who);
+  if (M <= 0 || N <= 0 || K < 0) return fail(RT_ERR_INVALID, "%s: M,N,K = %d,%d,%d", who, M, N, K);
+  if (BM <= 0 || BN <= 0 || BK <= 0 || group_m <= 0)
+    return fail(RT_ERR_INVALID, "%s: BLOCK sizes and GROUP_SIZE_M must be positive", who);
+  if (BM % 32 || BN % 32)
+    return fail(RT_ERR_UNSUPPORTED, "%s: BLOCK_SIZE_M/N = %d/%d, multiples of 32 are supported", who,
+                BM, BN);
+  int rc;
+  if ((rc = check_desc(who, "a", a, M, K))) return rc;
+  if ((rc = check_desc(who, "b", b, K, N))) return rc;
+  if ((rc = check_desc(who, "c", c, M, N))) return rc;
+  if (a->dtype != b->dtype) return fail(RT_ERR_INVALID, "%s: a and b dtypes differ", who);
+  if (grid[1] != 1 || grid[2] != 1)
+    return fail(RT_ERR_INVALID, "%s: 1-D grid expected, got (%u,%u,%u)", who, grid[0], grid[1], grid[2]);
+  const int64_t num_pid_m = cdiv64(M, BM), num_pid_n = cdiv64(N, BN);
+  if ((int64_t)grid[0] > num_pid_m * num_pid_n)
+    return fail(RT_ERR_INVALID, "%s: grid %u exceeds the %lld tiles of the problem", who, grid[0],
+                (long long)(num_pid_m * num_pid_n));
+  if (grid[0] == 0) return fail(RT_ERR_INVALID, "%s: empty grid", who);
+
+  GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a->base; g.b = b->base; g.c = c->base;
+  g.lda = a->strides[0]; g.ldb = b->strides[0]; g.ldc = c->strides[0];
+  g.M = M; g.N = N; g.K = K; g.BM = BM; g.BN = BN; g.BK = BK;
+  g.group_m = group_m; g.grid = (int32_t)grid[0];
+  g.num_pid_m = (int32_t)num_pid_m; g.num_pid_n = (int32_t)num_pid_n;
+  g.epi = epi; g.scale = scale;
+  switch (epi) {
+  case TT_EPI_NONE: case TT_EPI_LEAKY_RELU: break;
+  case TT_EPI_BIAS_FULL:
+    if ((rc = check_desc(who, "bias", bias, M, N))) return rc;
+    if (bias->dtype != c->dtype)
+      return fail(RT_ERR_INVALID, "%s: the full bias must have the output dtype", who);
+    g.bias = bias->base; g.ldbias = bias->strides[0];
+    break;
+  case TT_EPI_BIAS_ROW: case TT_EPI_BIAS_ROW_GELU:
+    if (!bias || !bias->base) return fail(RT_ERR_INVALID, "%s: null bias descriptor", who);
+    if (bias->dtype != TT_F32) return fail(RT_ERR_UNSUPPORTED, "%s: the row bias must be fp32", who);
+    if (!((bias->shape[0] == 1 && bias->shape[1] == N) || (bias->shape[0] == N && bias->shape[1] == 1)))
+      return fail(RT_ERR_INVALID, "%s: row bias must have N = %d elements, got [%d,%d]", who, N,
+                  bias->shape[0], bias->shape[1]);
+    if (bias->shape[1] == 1 && bias->shape[0] != 1 && bias->strides[0] != 1)
+      return fail(RT_ERR_INVALID, "%s: row bias must be contiguous", who);
+    g.bias = bias->base;
+    break;
+  default: return fail(RT_ERR_INVALID, "%s: unknown epilogue %d", who, epi);
+  }
+
+  const char *name = nullptr;
+  const int in = a->dtype, out = c->dtype;
+  if (in == TT_BF16 && out == TT_BF16) name = "gemm_any_bf16_bf16";
+  else if (in == TT_F16 && out == TT_F16) name = "gemm_any_f16_f16";
+  else if (in == TT_FP8E4M3 && out == TT_BF16) name = "gemm_any_fp8_bf16";
+  else if (in == TT_FP8E4M3 && out == TT_F16) name = "gemm_any_fp8_f16";
+  else if (in == TT_FP8E4M3 && out == TT_FP8E4M3) name = "gemm_any_fp8_fp8";
+  else return fail(RT_ERR_UNSUPPORTED, "%s: no kernel for input dtype %d -> output dtype %d", who, in, out);
+
+  const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
+  const int64_t cap = (int64_t)props()->multiprocessor_count * 8;
+  const uint32_t blocks = (uint32_t)std::max<int64_t>(1, std::min(cap, cdiv64(items, 4)));
+  void *args[] = {&g};
+  return launch("gemm", name, dim3(blocks), dim3(256), 0, stream, args, 1);
+}
+
+} // namespace
+
+extern "C" {
+
+int tt_matmul_kernel_tma(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c, int32_t M,
+                         int32_t N, int32_t K, int32_t BLOCK_SIZE_M, int32_t BLOCK_SIZE_N,
+                         int32_t BLOCK_SIZE_K, int32_t GROUP_SIZE_M, const uint32_t grid[3],
+                         void *stream) {
+  return run_matmul("matmul_kernel_tma", a, b, c, nullptr, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
+                    BLOCK_SIZE_K, GROUP_SIZE_M, TT_EPI_NONE, 1.0f, grid, stream);
+}
+
+int tt_matmul_kernel_fused(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c,
+                           const tt_desc2d *bias, int32_t M, int32_t N, int32_t K,
+                           int32_t BLOCK_SIZE_M, int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K,
+                           int32_t GROUP_SIZE_M, int32_t epilogue, const uint32_t grid[3],
+                           void *stream) {
+  return run_matmul("matmul_kernel_fused", a, b, c, bias, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
+                    BLOCK_SIZE_K, GROUP_SIZE_M, epilogue, 1.0f, grid, stream);
+}
+
+int tt_matmul_kernel_tma_fp8_scaled(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c,
+                                    int32_t M, int32_t N, int32_t K, float scale_a, float scale_b,
+                                    int32_t BLOCK_SIZE_M, int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K,
+                                    int32_t GROUP_SIZE_M, const uint32_t grid[3], void *stream) {
+  if (a && a->dtype != TT_FP8E4M3)
+    return fail(RT_ERR_INVALID, "matmul_kernel_tma_fp8_scaled: a and b must be fp8 e4m3");
+  return run_matmul("matmul_kernel_tma_fp8_scaled", a, b, c, nullptr, M, N, K, BLOCK_SIZE_M,
+                    BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, TT_EPI_NONE, scale_a * scale_b, grid,
+                    stream);
+}
+
+} // extern "C"

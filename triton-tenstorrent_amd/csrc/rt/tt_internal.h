@@ -1,0 +1,32 @@
+// Shared between the translation units of libttamd_rt.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ttamd_rt.h"
+
+namespace ttamd {
+
+// Records the calling thread's error message and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+// Properties of the initialised device, or nullptr before rt_init.
+const rt_props *props();
+// Looks up `name` in the built-in module `module` and launches it.
+int launch(const char *module, const char *name, dim3 grid, dim3 block, uint32_t shmem,
+           void *stream, void **args, size_t nargs);
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline size_t dtype_size(int dt) {
+  switch (dt) {
+  case TT_F32: case TT_I32: return 4;
+  case TT_BF16: case TT_F16: return 2;
+  case TT_FP8E4M3: return 1;
+  default: return 0;
+  }
+}
+// Integer environment knob read once per name (tuning sweeps only).
+int env_int(const char *name, int dflt);
+
+} // namespace ttamd

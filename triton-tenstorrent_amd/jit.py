@@ -1,0 +1,148 @@
+"""``kernel[grid](*args, **constexprs)`` for the prebuilt kernels, without
+Triton's JIT in the loop.
+
+It reproduces the part of Triton's runtime that sits between a user script and
+the plugin's launcher (triton/runtime/jit.py:695-745): bind the arguments,
+specialise the signature (tensors -> ``*fp32``, ints -> ``i32`` with the value 1
+folded to ``constexpr``, floats -> ``fp32``, descriptors ->
+``tensordesc<dtype[b0,b1]>``), run the autotune config's ``pre_hook``, evaluate
+the grid callable on the meta-parameters, obtain ``function`` from
+``driver.utils.load_binary`` and call ``driver.launcher_cls(src, metadata)`` with
+``(gridX, gridY, gridZ, stream, function, packed_metadata, launch_metadata,
+enter_hook, exit_hook, *args)``.
+"""
+from __future__ import annotations
+
+import json
+from types import SimpleNamespace
+from typing import Any, Callable, Sequence
+
+from .backend.driver import BINARY_EXT, TTDriver
+from .tensor_descriptor import is_tensor_descriptor
+
+_TORCH_TYPESTR = None
+
+
+def _typestr_of_torch(dtype) -> str:
+    global _TORCH_TYPESTR
+    if _TORCH_TYPESTR is None:
+        import torch
+        _TORCH_TYPESTR = {torch.float32: "fp32", torch.int32: "i32", torch.bfloat16: "bf16", torch.float16: "fp16",
+                          torch.float8_e4m3fn: "fp8e4nv", torch.float8_e5m2: "fp8e5", torch.int64: "i64",
+                          torch.float64: "fp64", torch.int8: "i8", torch.uint8: "u8", torch.int16: "i16"}
+    return _TORCH_TYPESTR[dtype]
+
+
+def specialize(arg: Any, is_constexpr: bool) -> str:
+    """Type string of one bound argument, as Triton's specializer writes it."""
+    if is_constexpr or arg is None:
+        return "constexpr"
+    if is_tensor_descriptor(arg):
+        block = ",".join(str(int(b)) for b in arg.block_shape)
+        return f"tensordesc<{_typestr_of_torch(arg.base.dtype)}[{block}]>"
+    if hasattr(arg, "data_ptr"):
+        return "*" + _typestr_of_torch(arg.dtype)
+    if isinstance(arg, bool):
+        return "i1"
+    if isinstance(arg, int):
+        if arg == 1:
+            return "constexpr"  # Triton folds the value 1 into the specialisation
+        return "i32" if -2**31 <= arg < 2**31 else "i64"
+    if isinstance(arg, float):
+        return "fp32"
+    raise TypeError(f"Unsupported scalar type: {type(arg)}")  # backend/driver.py:295
+
+
+class Config:
+    """One autotune configuration: meta-parameters plus an optional ``pre_hook(nargs)``."""
+
+    def __init__(self, kwargs: dict, num_warps: int = 4, num_stages: int = 1, pre_hook: Callable | None = None):
+        self.kwargs, self.num_warps, self.num_stages, self.pre_hook = dict(kwargs), num_warps, num_stages, pre_hook
+
+
+_driver: TTDriver | None = None
+
+
+def active_driver() -> TTDriver:
+    global _driver
+    if _driver is None:
+        _driver = TTDriver()
+    return _driver
+
+
+class PrebuiltKernel:
+    """A kernel of the prebuilt table with a Triton-style call surface."""
+
+    launch_enter_hook: Callable | None = None
+    launch_exit_hook: Callable | None = None
+
+    def __init__(self, name: str, arg_names: Sequence[str], constexprs: Sequence[str], *,
+                 configs: Sequence[Config] | None = None, launch_metadata: Callable | None = None,
+                 defaults: dict | None = None):
+        self.name = name
+        self.arg_names = list(arg_names)
+        self.constexprs = set(constexprs)
+        self.configs = list(configs or [])
+        self.launch_metadata = launch_metadata
+        self.defaults = dict(defaults or {})
+        self.fn = SimpleNamespace(arg_names=self.arg_names, __name__=name)
+        self._cache: dict = {}
+
+    def __getitem__(self, grid):
+        return lambda *args, **kwargs: self.run(*args, grid=grid, **kwargs)
+
+    def _bind(self, args, kwargs) -> dict:
+        if len(args) > len(self.arg_names):
+            raise TypeError(f"{self.name}() takes {len(self.arg_names)} arguments, {len(args)} given")
+        bound = dict(zip(self.arg_names, args))
+        for k, v in kwargs.items():
+            if k in ("num_warps", "num_stages", "num_ctas"):
+                continue
+            if k not in self.arg_names:
+                raise TypeError(f"{self.name}() got an unexpected keyword argument {k!r}")
+            if k in bound:
+                raise TypeError(f"{self.name}() got multiple values for argument {k!r}")
+            bound[k] = v
+        config = self.configs[0] if self.configs else None
+        for src in ((config.kwargs if config else {}), self.defaults):
+            for k, v in src.items():
+                bound.setdefault(k, v)
+        missing = [n for n in self.arg_names if n not in bound]
+        if missing:
+            raise TypeError(f"{self.name}() missing arguments: {missing}")
+        return {n: bound[n] for n in self.arg_names}
+
+    def run(self, *args, grid, **kwargs):
+        bound = self._bind(args, kwargs)
+        config = self.configs[0] if self.configs else None
+        if config is not None and config.pre_hook is not None:
+            config.pre_hook(bound)
+        if callable(grid):
+            grid = grid(bound)
+        grid = tuple(int(g) for g in grid)
+        gx, gy, gz = (grid + (1, 1, 1))[:3]
+        types = [specialize(bound[n], n in self.constexprs) for n in self.arg_names]
+        drv = active_driver()
+        device = drv.get_current_device()
+        stream = drv.get_current_stream(device)
+        key = (tuple(types), device)
+        entry = self._cache.get(key)
+        if entry is None:
+            signature = dict(zip(self.arg_names, types))
+            constants = {(i, ): bound[n] for i, (n, t) in enumerate(zip(self.arg_names, types))
+                         if t == "constexpr" and not hasattr(bound[n], "data_ptr")}
+            src = SimpleNamespace(fn=self.fn, signature=signature, constants=constants, name=self.name)
+            metadata = SimpleNamespace(name=self.name, shared=0, num_warps=config.num_warps if config else 4,
+                                       num_ctas=1, cluster_dims=(1, 1, 1), target=drv.get_current_target())
+            binary = json.dumps({"kernel": self.name, "ext": BINARY_EXT}).encode()
+            _, function, _, _, _ = drv.utils.load_binary(self.name, binary, metadata.shared, device)
+            packed = (metadata.num_warps, metadata.num_ctas, metadata.shared, *metadata.cluster_dims)
+            entry = (drv.launcher_cls(src, metadata), function, packed)
+            self._cache[key] = entry
+        launcher, function, packed = entry
+        enter, exit_ = PrebuiltKernel.launch_enter_hook, PrebuiltKernel.launch_exit_hook
+        launch_md = None
+        if self.launch_metadata is not None and (enter is not None or exit_ is not None):
+            launch_md = self.launch_metadata(grid, SimpleNamespace(name=self.name), bound)
+        launcher(gx, gy, gz, stream, function, packed, launch_md, enter, exit_, *bound.values())
+        return self
