@@ -1,0 +1,216 @@
+"""Host-side logic of the plugin surface, no GPU: signature specialisation, the reference's
+argument flattening, constexpr folding, binding of kernel names to C entry points (against a
+recording stand-in for the library), and that libttamd_rt.so exports what the header declares."""
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from triton_tenstorrent_amd import jit, kernels as K, runtime as rt
+from triton_tenstorrent_amd.backend import driver as drv
+from triton_tenstorrent_amd.tensor_descriptor import TensorDescriptor
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+class FakeTensor:
+    """Looks like a CUDA tensor to the launcher; never dereferenced."""
+
+    def __init__(self, shape, dtype, ptr=0x7f0000000000):
+        self.shape, self.dtype, self._ptr = tuple(shape), dtype, ptr
+        self.is_cuda = True
+
+    def data_ptr(self):
+        return self._ptr
+
+    def dim(self):
+        return len(self.shape)
+
+    def is_contiguous(self):
+        return True
+
+    def stride(self):
+        st, acc = [], 1
+        for d in reversed(self.shape):
+            st.insert(0, acc)
+            acc *= d
+        return tuple(st)
+
+    def numel(self):
+        n = 1
+        for d in self.shape:
+            n *= d
+        return n
+
+
+class RecordingLib:
+    def __init__(self):
+        self.calls = []
+
+    def __getattr__(self, name):
+        def fn(*args):
+            self.calls.append((name, args))
+            return 0
+        return fn
+
+
+@pytest.fixture
+def fake(monkeypatch):
+    lib = RecordingLib()
+    monkeypatch.setattr(rt, "init", lambda device=0: lib)
+    monkeypatch.setattr(drv.TTDriver, "get_current_device", lambda self: 0)
+    monkeypatch.setattr(drv.TTDriver, "get_current_stream", lambda self, d=None: 0x1234)
+    for k in (K.add_kernel, K.add_kernel_loop, K.sin_kernel, K.matmul_kernel_tma, K.matmul_kernel_fused, K._attn_fwd,
+              K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel):
+        k._cache.clear()
+    return lib
+
+
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "ttamd_rt.h").read_text()
+    declared = set(re.findall(r"TTAMD_API\s+(?:const\s+char\s*\*|int)\s*(\w+)\s*\(", header))
+    assert declared == set(rt.SYMBOLS), declared ^ set(rt.SYMBOLS)
+    lib = rt.load()
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_calls_before_init_return_errors_instead_of_aborting():
+    lib = rt.load()
+    g = rt.grid3(1)
+    assert lib.tt_add_kernel(None, None, None, 4, 1024, rt.TT_F32, g, None) == rt.RT_ERR_NOT_INIT
+    assert "rt_init" in rt.last_error()
+    p = rt.rt_props()
+    assert lib.rt_device_props(C.byref(p)) == rt.RT_ERR_NOT_INIT
+    assert lib.rt_launch(None, g, g, 0, None, None, 0) == rt.RT_ERR_INVALID
+    if not torch.cuda.is_available():
+        with pytest.raises(rt.RuntimeError_):
+            rt.init(0)  # no device here: a HIP error string, not a crash
+
+
+def test_specialize_matches_tritons_type_strings():
+    x = FakeTensor((8, ), torch.float32)
+    assert jit.specialize(x, False) == "*fp32"
+    assert jit.specialize(FakeTensor((8, ), torch.bfloat16), False) == "*bf16"
+    assert jit.specialize(FakeTensor((8, ), torch.float8_e4m3fn), False) == "*fp8e4nv"
+    assert jit.specialize(98432, False) == "i32" and jit.specialize(2**31, False) == "i64"
+    assert jit.specialize(1, False) == "constexpr"       # the value 1 is folded
+    assert jit.specialize(0.5, False) == "fp32" and jit.specialize(1024, True) == "constexpr"
+    d = TensorDescriptor(FakeTensor((256, 64), torch.bfloat16), [256, 64], [64, 1], [128, 64])
+    assert jit.specialize(d, False) == "tensordesc<bf16[128,64]>"
+    with pytest.raises(TypeError):
+        jit.specialize("nope", False)
+
+
+def test_descriptor_flattening_is_the_references_ten_scalars():
+    # base, shape0, shape1, stride0, stride1, pad, shape0, shape1, stride0, stride1 (backend/driver.py:141-159)
+    t = FakeTensor((64, 2560), torch.bfloat16)
+    d = TensorDescriptor(t, [64, 2560], [2560, 1], [64, 64])
+    flat = drv.flatten_launch_args(["tensordesc<bf16[64,64]>", "i32", "constexpr"], (d, 7, 64))
+    assert flat == [t, 64, 2560, 2560, 1, 0, 64, 2560, 2560, 1, 7]
+    d.padding = "nan"
+    assert drv.flatten_launch_args(["tensordesc<bf16[64,64]>"], (d, ))[5] == 1
+    # matmul_kernel_tma: 3 descriptors + M,N,K = 33 scalars (matmul_multi_core_tma.cpp:307-339)
+    sig = ["tensordesc<bf16[64,64]>"] * 3 + ["i32"] * 3 + ["constexpr"] * 6
+    assert len(drv.flatten_launch_args(sig, (d, d, d, 64, 2560, 9728, 64, 64, 64, 1, False, False))) == 33
+
+
+def test_descriptor_asserts():
+    t = FakeTensor((64, 64), torch.bfloat16)
+    with pytest.raises(AssertionError):
+        TensorDescriptor(t, [64, 64], [64, 2], [32, 32])            # last stride
+    with pytest.raises(AssertionError):
+        TensorDescriptor(FakeTensor((64, 64), torch.bfloat16, ptr=0x1008), [64, 64], [64, 1], [32, 32])  # 16 B base
+    with pytest.raises(AssertionError):
+        TensorDescriptor(t, [64, 60], [60, 1], [32, 32])            # 16 B leading stride
+    with pytest.raises(AssertionError):
+        TensorDescriptor(t, [64, 64], [64, 1], [32, 32], padding="inf")
+
+
+def test_add_binds_and_folds_n_equal_one(fake):
+    x = FakeTensor((98432, ), torch.float32)
+    K.add_kernel[lambda meta: (K.cdiv(98432, meta["BLOCK_SIZE"]), )](x, x, x, 98432, BLOCK_SIZE=1024)
+    name, a = fake.calls[-1]
+    assert name == "tt_add_kernel" and a[3:6] == (98432, 1024, rt.TT_F32) and list(a[6]) == [97, 1, 1]
+    assert a[7].value == 0x1234
+    K.add_kernel[(1, )](x, x, x, 1, BLOCK_SIZE=1024)     # n_elements == 1 arrives as a constexpr
+    assert fake.calls[-1][1][3] == 1
+    xi = FakeTensor((10, ), torch.int32)
+    K.add_kernel[(1, )](xi, xi, xi, 10, BLOCK_SIZE=1024)
+    assert fake.calls[-1][1][5] == rt.TT_I32
+    K.add_kernel_loop[(130, )](x, x, x, 98432, 1, BLOCK_SIZE=1024)  # row_count == 1 folded too
+    assert fake.calls[-1][0] == "tt_add_kernel_loop" and fake.calls[-1][1][3:6] == (98432, 1, 1024)
+
+
+def test_matmul_binding_pre_hook_and_grid(fake):
+    a, b, c = FakeTensor((256, 128), torch.bfloat16), FakeTensor((128, 512), torch.bfloat16), FakeTensor((256, 512), torch.bfloat16)
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+    K.matmul_kernel_tma[lambda META: (K.cdiv(256, META["BLOCK_SIZE_M"]) * K.cdiv(512, META["BLOCK_SIZE_N"]), )](
+        ad, bd, cd, 256, 512, 128, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert ad.block_shape == [128, 64] and bd.block_shape == [64, 128] and cd.block_shape == [128, 128]  # pre_hook ran
+    name, args = fake.calls[-1]
+    assert name == "tt_matmul_kernel_tma" and args[3:10] == (256, 512, 128, 128, 128, 64, 8) and list(args[10]) == [8, 1, 1]
+    d = args[0]._obj
+    assert (d.shape[0], d.shape[1], d.strides[0], d.strides[1], d.dtype) == (256, 128, 128, 1, rt.TT_BF16)
+    # reference configuration by keyword
+    K.matmul_kernel_tma[(32, )](ad, bd, cd, 256, 512, 128, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64, GROUP_SIZE_M=1,
+                                FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert fake.calls[-1][1][6:10] == (64, 64, 64, 1)
+
+
+def test_fused_and_attention_binding(fake):
+    a, b, c = FakeTensor((256, 128), torch.bfloat16), FakeTensor((128, 512), torch.bfloat16), FakeTensor((256, 512), torch.bfloat16)
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+    full = TensorDescriptor.from_tensor(FakeTensor((256, 512), torch.bfloat16), [32, 32])
+    K.matmul_kernel_fused[(8, )](ad, bd, cd, full, 256, 512, 128, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert fake.calls[-1][0] == "tt_matmul_kernel_fused" and fake.calls[-1][1][11] == rt.TT_EPI_BIAS_FULL
+    row = TensorDescriptor.from_tensor(FakeTensor((1, 512), torch.float32), [1, 32])
+    K.matmul_kernel_fused[(8, )](ad, bd, cd, row, 256, 512, 128, FP8_OUTPUT=False, WARP_SPECIALIZE=False, EPILOGUE="gelu")
+    assert fake.calls[-1][1][11] == rt.TT_EPI_BIAS_ROW_GELU
+    q = FakeTensor((1, 1, 256, 64), torch.bfloat16)
+    M = FakeTensor((1, 1, 256), torch.float32)
+    dq = TensorDescriptor(q, [256, 64], [64, 1], [1, 1])
+    K._attn_fwd[(2, 1, 1)](0.125, M, 1, 1, dq, dq, dq, dq, N_CTX=256, HEAD_DIM=64, BLOCK_M=128, BLOCK_N=64, FP8_OUTPUT=False,
+                           STAGE=3, warp_specialize=False, IS_HOPPER=False)   # Z = H = 1 are folded to constexprs
+    name, args = fake.calls[-1]
+    assert name == "tt_attn_fwd" and args[2:4] == (1, 1) and args[8:13] == (256, 64, 128, 64, 3)
+    assert dq.block_shape == [128, 64]
+
+
+def test_launch_hooks_and_metadata(fake):
+    seen = []
+    jit.PrebuiltKernel.launch_enter_hook = lambda md: seen.append(("enter", md))
+    jit.PrebuiltKernel.launch_exit_hook = lambda md: seen.append(("exit", md))
+    try:
+        a, b, c = FakeTensor((128, 128), torch.bfloat16), FakeTensor((128, 128), torch.bfloat16), FakeTensor((128, 128), torch.bfloat16)
+        ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+        K.matmul_kernel_tma[(1, )](ad, bd, cd, 128, 128, 128, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    finally:
+        jit.PrebuiltKernel.launch_enter_hook = jit.PrebuiltKernel.launch_exit_hook = None
+    assert [s[0] for s in seen] == ["enter", "exit"]
+    assert seen[0][1]["flops16"] == 2.0 * 128 ** 3 and seen[0][1]["bytes"] == 2 * 3 * 128 * 128
+
+
+def test_unknown_kernel_and_bad_arguments(fake):
+    with pytest.raises(rt.RuntimeError_):
+        drv.BoundKernel("no_such_kernel", {})
+    x = FakeTensor((8, ), torch.float32)
+    with pytest.raises(TypeError):
+        K.add_kernel[(1, )](x, x, x, 8)                      # BLOCK_SIZE missing
+    with pytest.raises(TypeError):
+        K.add_kernel[(1, )](x, x, x, 8, BLOCK_SIZE=1024, bogus=3)
+    with pytest.raises(ValueError):
+        cpu = torch.zeros(8)
+        K.add_kernel[(1, )](cpu, cpu, cpu, 8, BLOCK_SIZE=1024)   # host tensor
+
+
+def test_driver_surface():
+    d = drv.TTDriver()
+    t = d.get_current_target()
+    assert (t.backend, t.arch, t.warp_size) == ("tenstorrent", "gfx950", 64)
+    assert d.map_python_to_cpp_type("*fp32") == "*fp32"
+    assert d.launcher_cls is drv.TTLauncher and isinstance(d.utils, drv.TTUtils)
+    di = d.get_device_interface()
+    assert hasattr(di, "Event") and hasattr(di, "synchronize") and hasattr(di, "enable_hook_timing")

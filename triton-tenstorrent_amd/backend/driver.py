@@ -88,9 +88,12 @@ def flatten_launch_args(sig_types: list[str], args: tuple, ranks_out: list | Non
 class _Cursor:
     """Reads the flattened argument list back in signature order."""
 
-    def __init__(self, flat: list, keep: list, ranks: list | None = None):
+    def __init__(self, flat: list, keep: list, ranks: list | None = None, consts: dict | None = None,
+                 arg_names: list | None = None):
         self.flat, self.i, self.keep = flat, 0, keep
         self.ranks = list(ranks or [])
+        self.consts = consts or {}
+        self.arg_names = arg_names or []
 
     def _next(self):
         v = self.flat[self.i]
@@ -106,8 +109,16 @@ class _Cursor:
         self.keep.append(t)
         return t
 
-    def scalar(self):
+    def scalar(self, name: str | None = None):
+        """Next launch-time scalar; a parameter that Triton specialised to a
+        constexpr (an int equal to 1) is absent from the launch list and is
+        read from the constants instead."""
+        if name is not None and name in self.consts:
+            return self.consts[name]
         return self._next()
+
+    def has(self, name: str) -> bool:
+        return name in self.arg_names
 
     def desc(self) -> rt.tt_desc2d:
         rank = self.ranks.pop(0) if self.ranks else 2
@@ -140,23 +151,24 @@ def _contiguous_1d(t):
 # --------------------------------------------------------------------------
 def _bind_add(lib, cur: _Cursor, consts: dict, grid, stream):
     x, y, out = cur.tensor(), cur.tensor(), cur.tensor()
-    n = int(cur.scalar())
+    n = int(cur.scalar("n_elements"))
     block = int(consts["BLOCK_SIZE"])
     for t in (x, y, out):
         _contiguous_1d(t)
     dt = _torch_dtype_code(x)
     if _torch_dtype_code(y) != dt or _torch_dtype_code(out) != dt:
         raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "add_kernel: operand dtypes differ")
-    if cur.i < len(cur.flat):  # loop variant carries row_count
-        row_count = int(cur.scalar())
+    if cur.has("row_count"):  # the loop variant
+        row_count = int(cur.scalar("row_count"))
         cur.done()
         return lib.tt_add_kernel_loop(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, row_count, block, dt, grid, stream)
+    cur.done()
     return lib.tt_add_kernel(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, block, dt, grid, stream)
 
 
 def _bind_muladd(lib, cur, consts, grid, stream):
     x, y, z, out = (_contiguous_1d(cur.tensor()) for _ in range(4))
-    n = int(cur.scalar())
+    n = int(cur.scalar("n_elements"))
     cur.done()
     for t in (x, y, z, out):
         if _torch_dtype_code(t) != rt.TT_F32:
@@ -167,7 +179,7 @@ def _bind_muladd(lib, cur, consts, grid, stream):
 
 def _bind_sin(lib, cur, consts, grid, stream):
     x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
-    n = int(cur.scalar())
+    n = int(cur.scalar("n_elements"))
     cur.done()
     if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "sin_kernel computes in fp32")
@@ -179,8 +191,8 @@ def _mnk(cur: _Cursor, a: rt.tt_desc2d, b: rt.tt_desc2d):
     minimal variant reads them from ``desc.shape`` (kernel_matmul_tma.py:71-75).
     An int equal to 1 is specialised to a constexpr by Triton and is then
     absent from the launch list; the caller passes those through consts."""
-    if cur.i < len(cur.flat):
-        return int(cur.scalar()), int(cur.scalar()), int(cur.scalar())
+    if cur.has("M"):
+        return int(cur.scalar("M")), int(cur.scalar("N")), int(cur.scalar("K"))
     return a.shape[0], b.shape[1], a.shape[1]
 
 
@@ -194,11 +206,9 @@ def _block_consts(consts: dict, a: rt.tt_desc2d):
 def _bind_matmul_tma(lib, cur, consts, grid, stream):
     a, b, c = cur.desc(), cur.desc(), cur.desc()
     M, N, K = _mnk(cur, a, b)
-    fp8_scaled = "scale_a" in consts or cur.i < len(cur.flat)
     bm, bn, bk, g = _block_consts(consts, a)
-    if fp8_scaled:
-        sa = float(consts["scale_a"]) if "scale_a" in consts else float(cur.scalar())
-        sb = float(consts["scale_b"]) if "scale_b" in consts else float(cur.scalar())
+    if cur.has("scale_a"):
+        sa, sb = float(cur.scalar("scale_a")), float(cur.scalar("scale_b"))
         cur.done()
         return lib.tt_matmul_kernel_tma_fp8_scaled(C.byref(a), C.byref(b), C.byref(c), M, N, K, sa, sb, bm, bn, bk,
                                                    g, grid, stream)
@@ -226,12 +236,11 @@ def _bind_matmul_fused(lib, cur, consts, grid, stream):
 
 
 def _bind_attn_fwd(lib, cur, consts, grid, stream):
-    sm_scale = float(consts["sm_scale"]) if "sm_scale" in consts else float(cur.scalar())
+    sm_scale = float(cur.scalar("sm_scale"))
     M = cur.tensor()
-    Z = int(consts["Z"]) if "Z" in consts else int(cur.scalar())
-    H = int(consts["H"]) if "H" in consts else int(cur.scalar())
+    Z, H = int(cur.scalar("Z")), int(cur.scalar("H"))
     q, k, v, o = cur.desc(), cur.desc(), cur.desc(), cur.desc()
-    n_ctx = int(consts["N_CTX"]) if "N_CTX" in consts else int(cur.scalar())
+    n_ctx = int(cur.scalar("N_CTX"))
     cur.done()
     if _torch_dtype_code(M) != rt.TT_F32:
         raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "_attn_fwd: M must be fp32")
@@ -327,7 +336,7 @@ class TTLauncher:
             if len(idx) == 1 and idx[0] < len(self.arg_names):
                 consts.setdefault(self.arg_names[idx[0]], val)
         keep: list = []
-        cur = _Cursor(flat, keep, ranks)
+        cur = _Cursor(flat, keep, ranks, consts, self.arg_names)
         lib = rt.init(0)
         grid = rt.grid3(gridX, gridY, gridZ)
         if launch_enter_hook is not None:
