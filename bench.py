@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm,add,...] [--no-cpu]
+
+One "step" is one launch of the persistent bf16 GEMM, M=N=K=8192 (BASELINE
+configs[2], the configuration the metric's TFLOP/s figure is quoted on), with
+inputs resident in HBM.  The other configurations of the metric (elementwise
+streaming, fused epilogue, fp8, attention) are measured beside it and reported
+under "extra", each with its own roofline fraction.  Kernel durations come from
+HIP events recorded on the stream the kernels are launched on.  Prints ONE JSON
+line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
+PEAK_BF16_TFLOPS = 2500.0    # dense MFMA bf16 / fp16
+PEAK_FP8_TFLOPS = 5000.0     # dense MFMA fp8
+
+
+def _events_time(fn, steps: int, warmup: int, stream: int):
+    """Run fn() warmup+steps times; returns (avg_ms over the K-step region, list of per-launch ms)."""
+    import torch
+    from triton_tenstorrent_amd import runtime as rt
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [rt.Event() for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    evs[0].record(stream)
+    for i in range(steps):
+        fn()
+        evs[i + 1].record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    per = [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)]
+    total = evs[0].elapsed_time(evs[steps])
+    return total / steps, per, wall_ms / steps
+
+
+def _roof(bound: str, achieved: float, peak: float, unit: str, traffic=None):
+    return {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": traffic}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,fused,fp8,attn,add0")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE MI355X; every kernel here shards without communication "
+              "and no multi-GPU figure is produced (--gpus must be 1)", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    import __graft_entry__ as ge
+    ge._package()
+    from triton_tenstorrent_amd import kernels as K
+    from triton_tenstorrent_amd import runtime as rt
+    from triton_tenstorrent_amd.tensor_descriptor import TensorDescriptor
+
+    if not torch.cuda.is_available():
+        print("bench.py needs the GPU (no CPU fallback exists)", file=sys.stderr)
+        return 2
+    only = set(filter(None, args.only.split(",")))
+    want = lambda name: not only or name in only
+    props = rt.device_props()
+    stream = torch.cuda.current_stream().cuda_stream
+    steps, warmup = args.steps, args.warmup
+    extra: dict = {"device": props["name"], "arch": props["arch"], "cus": props["multiprocessor_count"],
+                   "clock_mhz": props["clock_khz"] // 1000,
+                   "peaks": {"hbm_GBs": PEAK_HBM_GBS, "bf16_TFLOPs": PEAK_BF16_TFLOPS, "fp8_TFLOPs": PEAK_FP8_TFLOPS}}
+    rooflines: dict = {}
+    torch.manual_seed(0)
+
+    # ---------------- primary: persistent bf16 GEMM 8192^3 -----------------
+    M = N = Kd = 8192
+    value = ms_per_step = None
+    primary_roof = None
+    if want("gemm"):
+        a = (torch.randn(M, Kd, device="cuda") / math.sqrt(Kd)).to(torch.bfloat16)
+        b = (torch.randn(Kd, N, device="cuda") / math.sqrt(Kd)).to(torch.bfloat16)
+        c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+        grid = (K.cdiv(M, 128) * K.cdiv(N, 128), )
+
+        def gemm_step():
+            K.matmul_kernel_tma[grid](ad, bd, cd, M, N, Kd, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+
+        # barrier + synchronize on both sides of exactly K timed steps
+        avg_ms, per, wall_ms = _events_time(gemm_step, steps, warmup, stream)
+        flops = 2.0 * M * N * Kd
+        value = flops / (avg_ms * 1e-3) / 1e12
+        ms_per_step = avg_ms
+        primary_roof = _roof("mfma", value, PEAK_BF16_TFLOPS, "TFLOP/s")
+        extra["gemm_bf16_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
+                                   "ms_min": round(min(per), 4), "ms_median": round(statistics.median(per), 4),
+                                   "wall_ms_per_step": round(wall_ms, 4), "TFLOPs": round(value, 2),
+                                   "TFLOPs_best": round(flops / (min(per) * 1e-3) / 1e12, 2)}
+        # spot parity on the benchmark's own output: 64 random rows against fp64 on the host
+        rows = torch.randint(0, M, (64, ), device="cuda")
+        ref = (a[rows].double() @ b.double()).float()
+        err = (c[rows].float() - ref).abs()
+        ok = bool(torch.all(err <= 1e-2 * ref.abs() + 1e-4))
+        extra["gemm_bf16_8192"]["parity_rows_ok"] = ok
+        if not ok:
+            print("bench.py: GEMM output failed its parity spot check", file=sys.stderr)
+            return 1
+        del a, b, c, ad, bd, cd
+
+    # ---------------- elementwise streaming, N = 2^28 ----------------------
+    n_el = 1 << 28
+    if want("add"):
+        g = torch.Generator(device="cuda").manual_seed(0)
+        x = torch.randint(-2**20, 2**20, (n_el, ), dtype=torch.int32, device="cuda", generator=g)
+        y = torch.randint(-2**20, 2**20, (n_el, ), dtype=torch.int32, device="cuda", generator=g)
+        out = torch.empty_like(x)
+        egrid = (K.cdiv(n_el, 1024), )
+        avg_ms, per, _ = _events_time(lambda: K.add_kernel[egrid](x, y, out, n_el, BLOCK_SIZE=1024), steps, warmup, stream)
+        gbs = 3 * 4 * n_el / (avg_ms * 1e-3) / 1e9
+        assert torch.equal(out[:1 << 20], x[:1 << 20] + y[:1 << 20])
+        extra["add_i32_2p28"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
+                                 "GBs": round(gbs, 1)}
+        rooflines["add_i32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s")
+        del x, y, out
+    if want("sin"):
+        xs = (torch.rand(n_el, device="cuda") * 2 - 1) * (8 * math.pi)
+        outs = torch.empty_like(xs)
+        egrid = (K.cdiv(n_el, 1024), )
+        avg_ms, per, _ = _events_time(lambda: K.sin_kernel[egrid](xs, outs, n_el, BLOCK_SIZE=1024), steps, warmup, stream)
+        gbs = 2 * 4 * n_el / (avg_ms * 1e-3) / 1e9
+        extra["sin_f32_2p28"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
+                                 "GBs": round(gbs, 1),
+                                 "max_abs_err_vs_f64": float((outs[:1 << 20].double() - torch.sin(xs[:1 << 20].double())).abs().max())}
+        rooflines["sin_f32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s")
+        del xs, outs
+    if want("add0"):
+        n0 = 98432
+        x0, y0 = torch.rand(n0, device="cuda"), torch.rand(n0, device="cuda")
+        o0 = torch.empty_like(x0)
+        avg_ms, per, wall = _events_time(lambda: K.add_kernel[(97, )](x0, y0, o0, n0, BLOCK_SIZE=1024), 200, 20, stream)
+        extra["add_f32_98432"] = {"us_avg": round(avg_ms * 1e3, 2), "us_min": round(min(per) * 1e3, 2),
+                                  "host_us_per_launch": round(wall * 1e3, 2), "GBs": round(3 * 4 * n0 / (avg_ms * 1e-3) / 1e9, 1)}
+
+    # ---------------- fused epilogue: GELU(A.B + bias) ----------------------
+    if want("fused"):
+        Mf, Nf, Kf = 4096, 14336, 4096
+        a = (torch.randn(Mf, Kf, device="cuda") / math.sqrt(Kf)).to(torch.bfloat16)
+        b = (torch.randn(Kf, Nf, device="cuda") / math.sqrt(Kf)).to(torch.bfloat16)
+        bias = (torch.randn(Nf, device="cuda") * 0.02).reshape(1, Nf)
+        c = torch.empty(Mf, Nf, device="cuda", dtype=torch.bfloat16)
+        ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+        biasd = TensorDescriptor.from_tensor(bias, [1, 32])
+        grid = (K.cdiv(Mf, 128) * K.cdiv(Nf, 128), )
+        avg_ms, per, _ = _events_time(
+            lambda: K.matmul_kernel_fused[grid](ad, bd, cd, biasd, Mf, Nf, Kf, FP8_OUTPUT=False, WARP_SPECIALIZE=False,
+                                                EPILOGUE="gelu"), steps, warmup, stream)
+        tf = 2.0 * Mf * Nf * Kf / (avg_ms * 1e-3) / 1e12
+        extra["gemm_gelu_4096x14336x4096"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
+                                              "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
+        rooflines["gemm_gelu_4096x14336x4096"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s")
+        del a, b, c, bias
+    if want("fp8"):
+        xa = torch.randn(M, Kd, device="cuda")
+        qa, sa = K.quantize_fp8(xa)
+        del xa
+        xb = torch.randn(Kd, N, device="cuda")
+        qb, sb = K.quantize_fp8(xb)
+        del xb
+        c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (qa, qb, c))
+        grid = (K.cdiv(M, 128) * K.cdiv(N, 128), )
+        avg_ms, per, _ = _events_time(
+            lambda: K.matmul_kernel_tma_fp8_scaled[grid](ad, bd, cd, M, N, Kd, sa, sb, FP8_OUTPUT=False, WARP_SPECIALIZE=False),
+            max(2, steps // 4), 1, stream)
+        tf = 2.0 * M * N * Kd / (avg_ms * 1e-3) / 1e12
+        extra["gemm_fp8_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
+                                  "TFLOPs": round(tf, 2)}
+        rooflines["gemm_fp8_8192"] = _roof("mfma", tf, PEAK_FP8_TFLOPS, "TFLOP/s")
+        del qa, qb, c
+    if want("attn"):
+        Z, H, S, D = 4, 32, 4096, 128
+        q, k, v = (torch.randn(Z, H, S, D, device="cuda").to(torch.bfloat16) for _ in range(3))
+        sm = 1.0 / math.sqrt(D)
+        avg_ms, per, _ = _events_time(lambda: K.attention(q, k, v, True, sm), max(2, steps // 2), 2, stream)
+        fl = 4.0 * Z * H * S * S * D / 2  # lower triangle only
+        tf = fl / (avg_ms * 1e-3) / 1e12
+        extra["attn_fwd_causal_4x32x4096x128"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
+                                                  "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
+        rooflines["attn_fwd_causal_4x32x4096x128"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s")
+        del q, k, v
+
+    # ---------------- CPU baseline: the oracle on a bounded sample ---------
+    cpu_baseline = None
+    if not args.no_cpu:
+        from oracle import oracle as orc
+        cores = orc.num_threads()
+        rng = np.random.default_rng(0)
+        ms = 4096  # sample: the same kernel and tile shape on M=N=K=4096 (1/8 of the flops)
+        ah = orc.to_bf16((rng.standard_normal((ms, ms)) / math.sqrt(ms)).astype(np.float32))
+        bh = orc.to_bf16((rng.standard_normal((ms, ms)) / math.sqrt(ms)).astype(np.float32))
+        t0 = time.perf_counter()
+        orc.matmul(ah, bh, BM=128, BN=128, BK=64, group_m=8)
+        dt = time.perf_counter() - t0
+        cpu_baseline = {"value": round(2.0 * ms ** 3 / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                        "sample": f"oracle matmul_kernel_tma restatement (C, OpenMP, fp32 accumulate), bf16 M=N=K={ms}, "
+                                  f"128x128x64 tiles, one run, {dt:.2f} s"}
+        ne = 1 << 26
+        xh = rng.integers(-2**20, 2**20, ne).astype(np.int32)
+        yh = rng.integers(-2**20, 2**20, ne).astype(np.int32)
+        oh = np.empty_like(xh)
+        orc.add(xh, yh, oh)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            orc.add(xh, yh, oh)
+        dt = (time.perf_counter() - t0) / 3
+        extra["cpu_add_i32"] = {"GBs": round(3 * 4 * ne / dt / 1e9, 2), "cores": cores, "sample": f"N=2^26, mean of 3"}
+        xf = ((rng.random(1 << 24, dtype=np.float32) * 2 - 1) * np.float32(8 * math.pi)).astype(np.float32)
+        of = np.empty_like(xf)
+        t0 = time.perf_counter()
+        orc.sin(xf, of, libm_f32=True)
+        dt = time.perf_counter() - t0
+        extra["cpu_sin_f32"] = {"GBs": round(2 * 4 * xf.size / dt / 1e9, 3), "cores": cores, "sample": "N=2^24, libm sinf, one run"}
+
+    line = {
+        "metric": "GEMM TFLOP/s @8192^3 bf16 + elementwise GB/s, % of MI355X roofline",
+        "value": None if value is None else round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": None if ms_per_step is None else round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "persistent GEMM C=A.B, bf16 in/out, fp32 accumulate, M=N=K=8192, logical tiles 128x128x64, "
+                               "persistent grid = CU count (BASELINE configs[2]); elementwise int32 add / fp32 sin at N=2^28 "
+                               "(configs[1]), GELU-fused GEMM and fp8 GEMM (configs[3]) and causal attention (configs[4]) under 'extra'"},
+        "roofline": primary_roof,
+        "cpu_baseline": cpu_baseline,
+        "rooflines": rooflines,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -161,3 +161,86 @@ def test_matmul_errors():
         K.matmul_kernel_tma[(1, )](ad, bd, TensorDescriptor.from_tensor(c, [32, 32]), 64, 64, 64, FP8_OUTPUT=False,
                                    WARP_SPECIALIZE=False)
     assert rt.last_error() != ""
+
+
+# ---- the 256x256x64 macro-tile fast path -----------------------------------
+@pytest.mark.parametrize("M,N,K_", [(256, 256, 64), (256, 256, 128), (512, 768, 320), (1024, 256, 2048), (768, 1280, 192)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fast_path_matches_oracle(M, N, K_, dtype):
+    a, b = _ab(M, N, K_, dtype, seed=M + N + K_)
+    c = K.matmul_tma(a.cuda(), b.cuda())
+    assert rt.last_kernel_name().startswith("gemm_tile_"), rt.last_kernel_name()
+    _check(c, a, b)
+
+
+def test_fast_path_small_integers_bit_exact():
+    g = torch.Generator().manual_seed(11)
+    M, N, K_ = 512, 512, 448
+    a = torch.randint(-4, 5, (M, K_), generator=g).to(torch.bfloat16)
+    b = torch.randint(-4, 5, (K_, N), generator=g).to(torch.bfloat16)
+    c = K.matmul_tma(a.cuda(), b.cuda())
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi0"
+    assert np.array_equal(bits(c), orc.matmul(bits(a), bits(b), BM=128, BN=128, BK=64, group_m=8))
+    # a permutation matrix tells B from B^T and exposes any mis-indexed fragment
+    p = torch.zeros(512, 512)
+    p[torch.arange(512), (torch.arange(512) * 37 + 5) % 512] = 1
+    x = torch.randn(512, 512, generator=g).to(torch.bfloat16)
+    c = K.matmul_tma(x.cuda(), p.to(torch.bfloat16).cuda())
+    assert torch.equal(c.cpu(), (x.float() @ p).to(torch.bfloat16))
+    c = K.matmul_tma(p.to(torch.bfloat16).cuda(), x.cuda())
+    assert torch.equal(c.cpu(), (p @ x.float()).to(torch.bfloat16))
+
+
+def test_fast_path_strided_rows_and_epilogues():
+    M, N, K_ = 512, 512, 256
+    a, b = _ab(M, N + 64, K_ + 64, seed=12)
+    a = a.cuda()[:, :K_]                 # lda = K+64
+    b = b.cuda()[:K_ , :N]               # ldb = N+64
+    cbuf = torch.full((M, N + 64), 7.5, dtype=torch.bfloat16, device="cuda")
+    c = cbuf[:, :N]
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+    K.matmul_kernel_tma[(16, )](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi0"
+    _check(c, a.cpu(), b.cpu())
+    assert torch.all(cbuf[:, N:] == 7.5)
+    ac, bc = a.contiguous(), b.contiguous()
+    bias_full = torch.randn(M, N, generator=torch.Generator().manual_seed(13)).to(torch.bfloat16).cuda()
+    cf = K.matmul_fused(ac, bc, bias_full)
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi1"
+    assert torch.equal(cf, c + bias_full)
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(14)) * 0.02).cuda()
+    cg = K.matmul_fused(ac, bc, bias, epilogue="gelu")
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi2"
+    ref = orc.from_bf16(orc.matmul(bits(ac), bits(bc), bias=bias.cpu().numpy(), epi=orc.EPI_BIAS_ROW_GELU, acc64=True))
+    assert close_bf16(decode(cg), ref, RTOL, ATOL)
+    cl = K.matmul_fused(ac, bc, bias, epilogue="leaky_relu")
+    ref = orc.from_bf16(orc.matmul(bits(ac), bits(bc), epi=orc.EPI_LEAKY_RELU, acc64=True))
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi3" and close_bf16(decode(cl), ref, RTOL, ATOL)
+    cr = K.matmul_fused(ac, bc, bias, epilogue="bias_row")
+    ref = orc.from_bf16(orc.matmul(bits(ac), bits(bc), bias=bias.cpu().numpy(), epi=orc.EPI_BIAS_ROW, acc64=True))
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi4" and close_bf16(decode(cr), ref, RTOL, ATOL)
+
+
+def test_full_size_8192_properties():
+    """BASELINE's 8192^3: checked through size-independent properties -- B = I gives C = A
+    bit for bit, linearity in A, and sampled rows against fp64 on the host."""
+    n = 8192
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = (torch.randn(n, n, device="cuda", generator=g) / n ** 0.5).to(torch.bfloat16)
+    eye = torch.eye(n, device="cuda", dtype=torch.bfloat16)
+    c = K.matmul_tma(a, eye)
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi0"
+    assert torch.equal(c, a)
+    assert torch.equal(K.matmul_tma(eye, a), a)
+    del eye
+    b = (torch.randn(n, n, device="cuda", generator=g) / n ** 0.5).to(torch.bfloat16)
+    c = K.matmul_tma(a, b)
+    rows = torch.tensor([0, 1, 255, 256, 4095, 4096, 8191, 5000, 77], device="cuda")
+    ref = (a[rows].double() @ b.double()).float()
+    err = (c[rows].float() - ref).abs()
+    assert bool(torch.all(err <= RTOL * ref.abs() + ATOL))
+    cols = torch.tensor([0, 31, 32, 255, 256, 8191, 6007], device="cuda")
+    ref = (a.double() @ b[:, cols].double()).float()
+    assert bool(torch.all((c[:, cols].float() - ref).abs() <= RTOL * ref.abs() + ATOL))
+    # scaling A by 2 scales C by 2 exactly (powers of two commute with every rounding)
+    assert torch.equal(K.matmul_tma(a * 2, b), c * 2)

@@ -107,7 +107,10 @@ __device__ __forceinline__ float sin_fast(float x) {
 }
 
 __device__ __forceinline__ float sin_any(float x) {
-  return (__builtin_fabsf(x) < 131072.0f) ? sin_fast(x) : sinf(x);
+  const float ax = __builtin_fabsf(x);
+  // below 2^-12 sin(x) rounds to x itself; returning x also keeps the sign of -0.0
+  float v = (ax < 131072.0f) ? sin_fast(x) : sinf(x);
+  return ax < 2.44140625e-4f ? x : v;
 }
 
 template <int UNROLL>

@@ -125,3 +125,21 @@ __device__ __forceinline__ float apply_epilogue(const GemmArgs &g, float acc, in
   default: return acc;
   }
 }
+
+// Same, with the epilogue fixed at compile time (one kernel per epilogue keeps
+// the unrolled fast-path epilogue free of per-element switches).
+template <int OUT_DT, int EPI>
+__device__ __forceinline__ float apply_epilogue_ct(const GemmArgs &g, float acc, int64_t m, int64_t n) {
+  if constexpr (EPI == EPI_BIAS_FULL) {
+    float cv = round_through<OUT_DT>(acc);
+    return cv + load_as_f32<OUT_DT>(g.bias, m * g.ldbias + n);
+  } else if constexpr (EPI == EPI_BIAS_ROW_GELU) {
+    return gelu_erf(acc + ((const float *)g.bias)[n]);
+  } else if constexpr (EPI == EPI_BIAS_ROW) {
+    return acc + ((const float *)g.bias)[n];
+  } else if constexpr (EPI == EPI_LEAKY_RELU) {
+    return acc >= 0.0f ? acc : 0.01f * acc;
+  } else {
+    return acc;
+  }
+}

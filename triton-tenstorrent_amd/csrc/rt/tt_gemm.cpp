@@ -1,6 +1,7 @@
 // tt_matmul_kernel_tma / tt_matmul_kernel_fused / tt_matmul_kernel_tma_fp8_scaled:
 // launch validation and kernel selection for the tile-matmul family.
 #include <algorithm>
+#include <cstdio>
 #include <cstring>
 
 #include "tt_internal.h"
@@ -94,6 +95,22 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   else if (in == TT_FP8E4M3 && out == TT_F16) name = "gemm_any_fp8_f16";
   else if (in == TT_FP8E4M3 && out == TT_FP8E4M3) name = "gemm_any_fp8_fp8";
   else return fail(RT_ERR_UNSUPPORTED, "%s: no kernel for input dtype %d -> output dtype %d", who, in, out);
+
+  // Fast path: whole 256x256x64 macro tiles, 16-byte aligned rows, and a grid that covers
+  // the problem (then the assignment of output to programs does not show in the result).
+  const bool full_grid = (int64_t)grid[0] == num_pid_m * num_pid_n;
+  const bool half_io = (in == TT_BF16 && out == TT_BF16) || (in == TT_F16 && out == TT_F16);
+  const bool fast_shape = M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && K >= 64;
+  const bool fast_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 8 == 0 &&
+                          g.ldb % 8 == 0 && g.ldc % 8 == 0;
+  if (full_grid && half_io && fast_shape && fast_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+    char fast_name[64];
+    snprintf(fast_name, sizeof(fast_name), "gemm_tile_%s_epi%d", in == TT_BF16 ? "bf16" : "f16", epi);
+    const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+    const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    void *fargs[] = {&g};
+    return launch("gemm", fast_name, dim3(wgs), dim3(256), 0, stream, fargs, 1);
+  }
 
   const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
   const int64_t cap = (int64_t)props()->multiprocessor_count * 8;
