@@ -26,7 +26,7 @@ RT_SOURCES = ["ttamd_rt.cpp", "tt_elementwise.cpp", "tt_gemm.cpp", "tt_attention
 
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 on this target
 DEVICE_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                "-ffp-contract=on", "-fno-fast-math", "-Wall", "-Wno-unused-function"]
+                "-ffp-contract=on", "-fno-fast-math", "-Wall", "-Wno-unused-function", "-Wno-inline-asm"]
 
 
 def hipcc() -> str:

@@ -16,4 +16,5 @@ struct GemmArgs {
   int32_t num_pid_m, num_pid_n;
   int32_t epi;
   float scale;              // multiplies the accumulator before the cast
+  unsigned long long *probe; // diagnostic: workgroup 0 stores {core-clock cycles, 100 MHz ticks} of its run, or null
 };

@@ -1,24 +1,28 @@
 // gemm_tile_*: the fast tile-matmul path for gfx950.
 //
 // Requirements (checked by the host): M and N multiples of 256, K a multiple of
-// 64, 16-byte aligned bases and leading strides, and a logical grid that covers
+// 128, 16-byte aligned bases and leading strides, and a logical grid that covers
 // every tile -- then which physical tile computes which part of C does not show
 // in the result (up to fp32 summation order).
 //
-// One workgroup (4 wavefronts, 2x2) computes a 256x256 macro tile, walking K in
-// steps of 64 through two LDS stages (A 256x64 + B 64x256 = 64 KiB per stage).
-// Each wavefront owns 128x128: 4x4 v_mfma_f32_32x32x16 accumulators (256
-// registers), so one wavefront per SIMD.  The grid is persistent, one workgroup
-// per CU, striding over the macro tiles in an XCD-aware order.
+// One workgroup (4 wavefronts, 2x2) computes a 256x256 macro tile.  Each
+// wavefront owns 128x128 of it: 4x4 v_mfma_f32_32x32x16 accumulators (256
+// registers), hence one wavefront per SIMD.  The grid is persistent, one
+// workgroup per CU, striding over the macro tiles in an XCD-aware order.
 //
-// Data path: global -> LDS directly (global_load_lds_dwordx4, no register
-// staging), issued one whole K-step ahead; LDS -> registers one 16-deep
-// sub-step ahead of the MFMAs that consume them, so a single wavefront keeps
-// its matrix pipe busy without help from a second one.
+// K is walked in steps of 32 through a ring of four LDS stages (A 256x32 +
+// B 32x256 = 32 KiB per stage).  Data goes global -> LDS directly
+// (global_load_lds_dwordx4, no register staging) three steps ahead of its use,
+// and the ring runs on across tile boundaries, so the first steps of the next
+// tile are already in flight while the current tile's epilogue stores C.  LDS ->
+// registers runs one 16-deep sub-step ahead of the MFMAs that consume it.  A
+// single wavefront thus keeps its matrix pipe fed without a second one to hide
+// behind: every stall that matters (HBM/L2 latency, LDS latency) is covered by
+// distance in the software pipeline.
 //
-// LDS layout (16-byte chunks, XOR-swizzled so that the row-wise A reads and the
-// transposing B reads are both bank-conflict free):
-//   A: row m = 128 B = 8 chunks;  logical chunk c sits at c ^ ((m>>1)&7)
+// LDS layout per stage (16-byte chunks, XOR-swizzled so that the row-wise A
+// reads and the transposing B reads are both bank-conflict free):
+//   A: row m = 64 B = 4 chunks;   logical chunk c sits at c ^ ((m>>2)&3)
 //   B: row k = 512 B = 32 chunks; logical chunk c sits at c ^ ((k&3)<<2)
 // A direct-to-LDS load writes lane l's 16 bytes at (wave-uniform base) + 16*l,
 // so thread t owns byte 16*t of every 4 KiB slab and the swizzle is applied to
@@ -30,14 +34,18 @@
 // contiguous: ds_read_b64_tr_b16 transposes a 4x16 block of 16-bit values
 // across each group of 16 lanes on the way out of LDS.
 #pragma once
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace fast {
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int A_BYTES = BM * BK * 2;        // 32 KiB
-constexpr int B_BYTES = BK * BN * 2;        // 32 KiB
-constexpr int STAGE = A_BYTES + B_BYTES;    // 64 KiB
+constexpr int BM = 256, BN = 256, BK = 32;
+constexpr int R = 4;                        // ring depth
+constexpr int A_BYTES = BM * BK * 2;        // 16 KiB
+constexpr int B_BYTES = BK * BN * 2;        // 16 KiB
+constexpr int STAGE = A_BYTES + B_BYTES;    // 32 KiB
+constexpr int DMA_PER_STEP = 8;             // direct-to-LDS loads per thread and step
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
@@ -74,13 +82,14 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int &tm
   tn = (id % in_group) / gsz;
 }
 
-// scheduling hints: one group of `n` instructions of a class, in program order
-#define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
-#define SCHED_DSRD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
-#define SCHED_VMEM(n) __builtin_amdgcn_sched_group_barrier(0x010, n, 0)
+#define FENCE() __builtin_amdgcn_sched_barrier(0)
+
+struct Ring {
+  uint8_t *s[R];
+};
 
 template <int IN_DT, int OUT_DT, int EPI>
-__device__ __forceinline__ void body(const GemmArgs &g, uint8_t *lds0, uint8_t *lds1) {
+__device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   using X = MFMA<IN_DT>;
   using vec = typename X::vec;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -88,27 +97,28 @@ __device__ __forceinline__ void body(const GemmArgs &g, uint8_t *lds0, uint8_t *
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = g.M / BM, tiles_n = g.N / BN;
   const int total = tiles_m * tiles_n;
-  const int nk = g.K / BK;
+  const int nk = g.K / BK; // steps per tile, a multiple of R
 
   // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
-  // A slab i (32 rows): row = i*32 + (t>>3), chunk position t&7 holds logical chunk (t&7)^((row>>1)&7)
-  const int a_row = tid >> 3;
-  const int a_chunk = (tid & 7) ^ ((a_row >> 1) & 7);
+  // A slab i (64 rows): row = i*64 + (t>>2), chunk position t&3 holds logical chunk (t&3)^((row>>2)&3)
+  const int a_row = tid >> 2;
+  const int a_chunk = (tid & 3) ^ ((a_row >> 2) & 3);
   // B slab i (8 k-rows): k = i*8 + (t>>5), chunk position t&31 holds logical chunk (t&31)^((k&3)<<2)
   const int b_k = tid >> 5;
   const int b_chunk = (tid & 31) ^ ((b_k & 3) << 2);
   const uint32_t a_voff = (uint32_t)(((int64_t)a_row * g.lda + a_chunk * 8) * 2); // bytes, per thread
   const uint32_t b_voff = (uint32_t)(((int64_t)b_k * g.ldb + b_chunk * 8) * 2);
-  const int64_t a_slab = 32 * g.lda * 2, b_slab = 8 * g.ldb * 2;                   // bytes, uniform
+  const int64_t a_slab = 64 * g.lda * 2, b_slab = 8 * g.ldb * 2;                   // bytes, uniform
+  const int64_t b_kstep = (int64_t)BK * g.ldb * 2;
   const int lds_wave = wave * 1024;
 
   // ---- LDS -> fragments ----
   const int l32 = lane & 31, hi = lane >> 5;
-  const int a_base = (wm * 128 + l32) * 128;
-  const int a_x = (lane >> 1) & 7;
-  int a_pos[4];
+  const int a_base = (wm * 128 + l32) * 64;
+  const int a_x = (l32 >> 2) & 3;
+  int a_pos[2]; // sub-step s: logical chunk 2s + hi
 #pragma unroll
-  for (int s = 0; s < 4; ++s) a_pos[s] = a_base + (((s * 2 + hi) ^ a_x) << 4);
+  for (int s = 0; s < 2; ++s) a_pos[s] = a_base + (((s * 2 + hi) ^ a_x) << 4);
   const int G4 = lane >> 4, i16 = lane & 15, q = i16 >> 2;
   const int b_base = A_BYTES + (((G4 >> 1) * 8 + q) * 512) + ((wn * 16 + (G4 & 1) * 2 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
@@ -118,104 +128,149 @@ __device__ __forceinline__ void body(const GemmArgs &g, uint8_t *lds0, uint8_t *
 
   const uint8_t *A = (const uint8_t *)g.a;
   const uint8_t *B = (const uint8_t *)g.b;
+  const long long probe_c0 = g.probe ? clock64() : 0, probe_w0 = g.probe ? wall_clock64() : 0;
 
-  for (int t = blockIdx.x; t < total; t += gridDim.x) {
+  // Fragment registers: two sets (even / odd sub-steps).  B fragments are kept as their
+  // two transposed halves (k 0-3 and k 4-7 of the lane's group).
+  struct Frags {
+    vec a[4];
+    union { s16x4 h[2]; vec v; } b[4];
+  };
+  Frags f0, f1;
+  f32x16 acc[4][4]; // [m-tile][n-tile]
+
+  // The 12 LDS reads of one sub-step, in the order the MFMAs will want them:
+  // b0.lo b0.hi a0 b1.lo b1.hi b2.lo b2.hi b3.lo b3.hi a1 a2 a3
+  auto rd = [&](Frags &f, const uint8_t *stage, int s, int r) {
+    switch (r) {
+    case 2: f.a[0] = *(const vec *)(stage + a_pos[s]); break;
+    case 9: f.a[1] = *(const vec *)(stage + a_pos[s] + 2048); break;
+    case 10: f.a[2] = *(const vec *)(stage + a_pos[s] + 4096); break;
+    case 11: f.a[3] = *(const vec *)(stage + a_pos[s] + 6144); break;
+    default: {
+      const int rr = r < 2 ? r : r - 1; // 0..7 over the b reads
+      const int j = rr >> 1, h = rr & 1;
+      f.b[j].h[h] =
+          __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(stage + b_pos[j] + s * 8192 + h * 2048));
+    }
+    }
+  };
+  // MFMA number n (0..15) of a sub-step, m-tile major: needs a[n/4], b[n%4]
+  auto mm = [&](Frags &f, int n) {
+    const int i = n >> 2, j = n & 3;
+    acc[i][j] = X::run(f.b[j].v, f.a[i], acc[i][j]);
+  };
+  // One direct-to-LDS copy: lane l's 16 bytes land at dst_slab + wave*1024 + 16*l.
+  // Written as assembly on purpose: the compiler's own bookkeeping of such copies is
+  // conservative (it drains every outstanding one before an LDS read it cannot prove
+  // unrelated), which would flatten the multi-step prefetch.  Completion is tracked by
+  // hand instead: copies retire in issue order, and each step's barrier waits with
+  // s_waitcnt vmcnt(n) for exactly the copies that the following reads depend on.
+  auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+    const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(src_uniform)
+                 : "memory", "m0");
+  };
+
+  // The stream of steps this workgroup executes: tile after tile, nk steps each.
+  // a_cur/b_cur point at the current tile's A rows / B columns, a_nxt/b_nxt at the next
+  // tile's (or the current one again when there is none: a harmless refetch).
+  const uint8_t *a_cur, *b_cur, *a_nxt, *b_nxt;
+  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp) {
+    int tm, tn;
+    tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
+    ap = A + (int64_t)tm * BM * g.lda * 2;
+    bp = B + (int64_t)tn * BN * 2;
+  };
+  // copies of step kk (kk may run past nk into the next tile) into ring stage I
+  auto dma_pair = [&](int kk, uint8_t *stage, int i) { // i = 0..3: two of the eight loads
+    const bool over = kk >= nk;
+    const int k = over ? kk - nk : kk;
+    const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * (BK * 2);
+    const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
+    if (i < 2) {
+      dma_one(ap + (2 * i) * a_slab, a_voff, stage + (2 * i) * 4096);
+      dma_one(ap + (2 * i + 1) * a_slab, a_voff, stage + (2 * i + 1) * 4096);
+    } else {
+      dma_one(bp + (2 * i - 4) * b_slab, b_voff, stage + A_BYTES + (2 * i - 4) * 4096);
+      dma_one(bp + (2 * i - 3) * b_slab, b_voff, stage + A_BYTES + (2 * i - 3) * 4096);
+    }
+  };
+
+  // One step (K += 32) on ring stage I.
+  //   entry: f0 holds sub-step 0 of stage I; copies for the next R-1 steps are in flight
+  //   exit : f0 holds sub-step 0 of stage I+1; the copy of step k+R into stage I is in flight
+  auto step = [&](auto I_, int k) {
+    constexpr int I = decltype(I_)::value;
+    uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
+    // sub-step 0: MFMAs on f0, sub-step 1's fragments ride along (two reads per MFMA)
+#pragma unroll
+    for (int n = 0; n < 16; ++n) {
+      if (n < 6) {
+        rd(f1, cur, 1, 2 * n);
+        rd(f1, cur, 1, 2 * n + 1);
+      }
+      mm(f0, n);
+      FENCE();
+    }
+    // All of this wave's reads of stage I have returned, and so has its share of the
+    // copy into stage I+1 (the R-2 younger copies may still be in flight).  After the
+    // barrier that holds for every wave: I+1 may be read, I may be overwritten.
+    static_assert(DMA_PER_STEP * (R - 2) == 16, "the wait below is written for 16 younger copies");
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    FENCE();
+    // sub-step 1: MFMAs on f1; first the copy of step k+R into the freed stage (two loads
+    // per MFMA), then the next stage's sub-step 0 fragments
+#pragma unroll
+    for (int n = 0; n < 16; ++n) {
+      if (n < 4) dma_pair(k + R, cur, n);
+      if (n >= 4 && n < 10) {
+        rd(f0, nxt, 0, 2 * (n - 4));
+        rd(f0, nxt, 0, 2 * (n - 4) + 1);
+      }
+      mm(f1, n);
+      FENCE();
+    }
+  };
+
+  // ---- fill the ring: steps 0..R-1 of the first tile ----
+  int t = blockIdx.x;
+  if (t >= total) return;
+  tile_bases(t, a_cur, b_cur);
+  tile_bases(t + gridDim.x < total ? t + gridDim.x : t, a_nxt, b_nxt);
+#pragma unroll
+  for (int s = 0; s < R; ++s)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_pair(s, ring.s[s], i);
+  static_assert(DMA_PER_STEP * (R - 1) == 24, "the wait below is written for 24 younger copies");
+  asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+  for (int r = 0; r < 12; ++r) rd(f0, ring.s[0], 0, r);
+
+  for (; t < total; t += gridDim.x) {
     int tm, tn;
     tile_of(t, tiles_m, tiles_n, tm, tn);
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
-    const uint8_t *a_tile = A + m0 * g.lda * 2; // + kt*128 per K-step
-    const uint8_t *b_tile = B + n0 * 2;         // + kt*64*ldb*2 per K-step
-    const int64_t b_kstep = (int64_t)BK * g.ldb * 2;
-
-    // direct-to-LDS copy of K-step kt (clamped: past the end it refetches the last one
-    // into a stage nobody reads again, which keeps the loop body branch-free)
-    auto dma = [&](int kt, uint8_t *stage) {
-      kt = min(kt, nk - 1);
-      const uint8_t *ap = a_tile + (int64_t)kt * (BK * 2);
-      const uint8_t *bp = b_tile + (int64_t)kt * b_kstep;
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        __builtin_amdgcn_global_load_lds((global_void *)(ap + i * a_slab + a_voff),
-                                         (lds_void *)(stage + i * 4096 + lds_wave), 16, 0, 0);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        __builtin_amdgcn_global_load_lds((global_void *)(bp + i * b_slab + b_voff),
-                                         (lds_void *)(stage + A_BYTES + i * 4096 + lds_wave), 16, 0, 0);
-    };
-    auto read_a = [&](const uint8_t *stage, int s, vec (&f)[4]) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) f[i] = *(const vec *)(stage + a_pos[s] + i * 4096);
-    };
-    auto read_b = [&](const uint8_t *stage, int s, vec (&f)[4]) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint8_t *p = stage + b_pos[j] + s * 8192;
-        union { s16x4 h[2]; vec v; } u;
-        u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p));
-        u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 2048));
-        f[j] = u.v;
-      }
-    };
-
-    f32x16 acc[4][4]; // [m-tile][n-tile]
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
-    auto mma = [&](vec (&fa)[4], vec (&fb)[4], int i0, int i1) {
-#pragma unroll
-      for (int i = i0; i < i1; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = X::run(fb[j], fa[i], acc[i][j]);
-    };
 
-    vec fa0[4], fb0[4], fa1[4], fb1[4];
-
-    // One K-step on stage `cur`; `nxt` is being filled with K-step kt+1 meanwhile.
-    // Entry: fa0/fb0 hold sub-step 0 of `cur`.  Exit: fa0/fb0 hold sub-step 0 of `nxt`.
-    auto kstep = [&](int kt, uint8_t *cur, uint8_t *nxt) {
-      read_a(cur, 1, fa1); read_b(cur, 1, fb1);
-      mma(fa0, fb0, 0, 4);
-      for (int r = 0; r < 12; ++r) { SCHED_MFMA(1); SCHED_DSRD(1); }
-      SCHED_MFMA(4);
-
-      read_a(cur, 2, fa0); read_b(cur, 2, fb0);
-      mma(fa1, fb1, 0, 4);
-      for (int r = 0; r < 12; ++r) { SCHED_MFMA(1); SCHED_DSRD(1); }
-      SCHED_MFMA(4);
-
-      read_a(cur, 3, fa1); read_b(cur, 3, fb1);
-      mma(fa0, fb0, 0, 3);
-      for (int r = 0; r < 12; ++r) { SCHED_MFMA(1); SCHED_DSRD(1); }
-      // every wave has its last fragments of `cur` and the copy into `nxt` has landed:
-      // after the barrier `nxt` may be read and `cur` may be overwritten
-      __syncthreads();
-      dma(kt + 2, cur);
-      mma(fa0, fb0, 3, 4);
-
-      read_a(nxt, 0, fa0); read_b(nxt, 0, fb0);
-      mma(fa1, fb1, 0, 4);
-      // the 16 copies go out first (they have the longest way to go), two per MFMA
-      for (int r = 0; r < 4; ++r) { SCHED_MFMA(1); SCHED_VMEM(2); }
-      for (int r = 0; r < 4; ++r) { SCHED_MFMA(1); SCHED_VMEM(2); SCHED_DSRD(1); }
-      for (int r = 0; r < 8; ++r) { SCHED_MFMA(1); SCHED_DSRD(1); }
-      SCHED_MFMA(4);
-    };
-
-    __syncthreads(); // the previous tile's fragment reads are done before the stages are refilled
-    dma(0, lds0);
-    dma(1, lds1);
-    __builtin_amdgcn_s_waitcnt(0x4F70); // vmcnt(16): K-step 0 has landed, K-step 1 still in flight
-    __builtin_amdgcn_s_barrier();
-    read_a(lds0, 0, fa0); read_b(lds0, 0, fb0);
-
-    int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-      kstep(kt, lds0, lds1);
-      kstep(kt + 1, lds1, lds0);
+    for (int k = 0; k < nk; k += R) {
+      step(std::integral_constant<int, 0>{}, k);
+      step(std::integral_constant<int, 1>{}, k + 1);
+      step(std::integral_constant<int, 2>{}, k + 2);
+      step(std::integral_constant<int, 3>{}, k + 3);
     }
-    if (kt < nk) kstep(kt, lds0, lds1);
-    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): drain the clamped refetches before the stages are reused
+    // the ring already holds the next tile's first steps; move the tile window on
+    a_cur = a_nxt;
+    b_cur = b_nxt;
+    {
+      const int t2 = t + 2 * (int)gridDim.x;
+      tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt);
+    }
 
     // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
     //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
@@ -241,6 +296,11 @@ __device__ __forceinline__ void body(const GemmArgs &g, uint8_t *lds0, uint8_t *
       }
     }
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the trailing refetches must land before the LDS is released
+  if (g.probe && blockIdx.x == 0 && tid == 0) {
+    g.probe[0] = (unsigned long long)(clock64() - probe_c0);
+    g.probe[1] = (unsigned long long)(wall_clock64() - probe_w0);
+  }
 }
 
 } // namespace fast
@@ -251,7 +311,10 @@ extern "C" {
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
-    fast::body<IN, OUT, EPI>(g, lds0, lds1);                                                        \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
+    fast::body<IN, OUT, EPI>(g, ring);                                                              \
   }
 #define GEMM_TILE_ALL_EPI(prefix, IN, OUT)             \
   GEMM_TILE(prefix##_epi0, IN, OUT, EPI_NONE)           \

@@ -100,7 +100,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   // the problem (then the assignment of output to programs does not show in the result).
   const bool full_grid = (int64_t)grid[0] == num_pid_m * num_pid_n;
   const bool half_io = (in == TT_BF16 && out == TT_BF16) || (in == TT_F16 && out == TT_F16);
-  const bool fast_shape = M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && K >= 64;
+  const bool fast_shape = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
   const bool fast_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 8 == 0 &&
                           g.ldb % 8 == 0 && g.ldc % 8 == 0;
   if (full_grid && half_io && fast_shape && fast_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
@@ -108,8 +108,22 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     snprintf(fast_name, sizeof(fast_name), "gemm_tile_%s_epi%d", in == TT_BF16 ? "bf16" : "f16", epi);
     const int64_t tiles = (int64_t)(M / 256) * (N / 256);
     const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
+    // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
+    static unsigned long long *probe_buf = nullptr;
+    const bool probe = env_int("TTAMD_GEMM_CLOCK_PROBE", 0) != 0;
+    if (probe && !probe_buf && hipMalloc((void **)&probe_buf, 16) != hipSuccess) probe_buf = nullptr;
+    g.probe = probe ? probe_buf : nullptr;
     void *fargs[] = {&g};
-    return launch("gemm", fast_name, dim3(wgs), dim3(256), 0, stream, fargs, 1);
+    int lrc = launch("gemm", fast_name, dim3(wgs), dim3(256), 0, stream, fargs, 1);
+    if (lrc == 0 && g.probe) {
+      unsigned long long h[2] = {0, 0};
+      if (hipStreamSynchronize((hipStream_t)stream) == hipSuccess &&
+          hipMemcpy(h, probe_buf, 16, hipMemcpyDeviceToHost) == hipSuccess && h[1])
+        fprintf(stderr, "[ttamd] %s: workgroup 0 ran %llu core cycles in %.1f us -> %.3f GHz\n", fast_name, h[0],
+                h[1] / 100.0, h[0] / (h[1] * 10.0));
+    }
+    return lrc;
   }
 
   const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
