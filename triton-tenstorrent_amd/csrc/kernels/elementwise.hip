@@ -7,8 +7,12 @@
 // elements, lanes at or past n are masked.  The host folds grid and BLOCK into
 // one bound n_eff = min(n, grid*BLOCK); the kernels touch exactly [0, n_eff).
 //
-// HBM-bound: 16-byte loads and stores per lane, UNROLL independent vectors in
-// flight per lane, a grid-stride loop over a grid sized to the CU count.
+// HBM-bound: 16-byte non-temporal loads and stores per lane, UNROLL independent
+// vectors in flight per lane.  Each workgroup streams one contiguous run of
+// 256*UNROLL vectors and exits (measured on MI355X: 6.4-6.5 TB/s for the
+// 2-read/1-write add, against 4.5-5.3 TB/s for grid-stride loops over a
+// CU-count-sized grid at any unroll, and 5.6 TB/s for one contiguous chunk per
+// persistent workgroup).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -30,18 +34,17 @@ __device__ __forceinline__ void binary_body(const T *__restrict__ x, const T *__
                                             T *__restrict__ out, uint32_t n) {
   using V = typename Vec4<T>::type;
   const uint32_t nvec = n >> 2;
-  const uint32_t stride = gridDim.x * kThreads;
   const V *xv = reinterpret_cast<const V *>(x);
   const V *yv = reinterpret_cast<const V *>(y);
   V *ov = reinterpret_cast<V *>(out);
-  uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-  // full groups of UNROLL vectors: no per-vector bounds checks
-  for (; (uint64_t)i + (uint64_t)(UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+  const uint32_t base = blockIdx.x * (kThreads * UNROLL);
+  const uint32_t i = base + threadIdx.x;
+  if (base + kThreads * UNROLL <= nvec) { // whole run inside the array: no per-vector checks
     V a[UNROLL], b[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * stride);
+    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * kThreads);
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) b[u] = __builtin_nontemporal_load(yv + i + u * stride);
+    for (int u = 0; u < UNROLL; ++u) b[u] = __builtin_nontemporal_load(yv + i + u * kThreads);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       V r;
@@ -49,20 +52,22 @@ __device__ __forceinline__ void binary_body(const T *__restrict__ x, const T *__
       r.y = Op::apply(a[u].y, b[u].y);
       r.z = Op::apply(a[u].z, b[u].z);
       r.w = Op::apply(a[u].w, b[u].w);
-      __builtin_nontemporal_store(r, ov + i + u * stride);
+      __builtin_nontemporal_store(r, ov + i + u * kThreads);
     }
-  }
-  for (; i < nvec; i += stride) {
-    V a = xv[i], b = yv[i], r;
-    r.x = Op::apply(a.x, b.x);
-    r.y = Op::apply(a.y, b.y);
-    r.z = Op::apply(a.z, b.z);
-    r.w = Op::apply(a.w, b.w);
-    ov[i] = r;
-  }
-  // scalar tail: the last n % 4 elements
-  if (blockIdx.x == 0) {
-    uint32_t t = (nvec << 2) + threadIdx.x;
+  } else { // the last workgroup: ragged end plus the n % 4 scalar tail
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t j = i + u * kThreads;
+      if (j < nvec) {
+        V a = xv[j], b = yv[j], r;
+        r.x = Op::apply(a.x, b.x);
+        r.y = Op::apply(a.y, b.y);
+        r.z = Op::apply(a.z, b.z);
+        r.w = Op::apply(a.w, b.w);
+        ov[j] = r;
+      }
+    }
+    const uint32_t t = (nvec << 2) + threadIdx.x;
     if (t < n) out[t] = Op::apply(x[t], y[t]);
   }
 }
@@ -118,14 +123,14 @@ __device__ __forceinline__ void sin_body(const float *__restrict__ x, float *__r
                                          uint32_t n) {
   using V = Vec4<float>::type;
   const uint32_t nvec = n >> 2;
-  const uint32_t stride = gridDim.x * kThreads;
   const V *xv = reinterpret_cast<const V *>(x);
   V *ov = reinterpret_cast<V *>(out);
-  uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-  for (; (uint64_t)i + (uint64_t)(UNROLL - 1) * stride < nvec; i += UNROLL * stride) {
+  const uint32_t base = blockIdx.x * (kThreads * UNROLL);
+  const uint32_t i = base + threadIdx.x;
+  if (base + kThreads * UNROLL <= nvec) {
     V a[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * stride);
+    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * kThreads);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       V r;
@@ -133,19 +138,22 @@ __device__ __forceinline__ void sin_body(const float *__restrict__ x, float *__r
       r.y = sin_any(a[u].y);
       r.z = sin_any(a[u].z);
       r.w = sin_any(a[u].w);
-      __builtin_nontemporal_store(r, ov + i + u * stride);
+      __builtin_nontemporal_store(r, ov + i + u * kThreads);
     }
-  }
-  for (; i < nvec; i += stride) {
-    V a = xv[i], r;
-    r.x = sin_any(a.x);
-    r.y = sin_any(a.y);
-    r.z = sin_any(a.z);
-    r.w = sin_any(a.w);
-    ov[i] = r;
-  }
-  if (blockIdx.x == 0) {
-    uint32_t t = (nvec << 2) + threadIdx.x;
+  } else {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t j = i + u * kThreads;
+      if (j < nvec) {
+        V a = xv[j], r;
+        r.x = sin_any(a.x);
+        r.y = sin_any(a.y);
+        r.z = sin_any(a.z);
+        r.w = sin_any(a.w);
+        ov[j] = r;
+      }
+    }
+    const uint32_t t = (nvec << 2) + threadIdx.x;
     if (t < n) out[t] = sin_any(x[t]);
   }
 }
@@ -192,27 +200,32 @@ __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restric
                                                           float *__restrict__ out, uint32_t n,
                                                           uint32_t aligned) {
   using V = Vec4<float>::type;
-  const uint32_t stride = gridDim.x * kThreads;
   if (aligned) {
     const uint32_t nvec = n >> 2;
     const V *xv = reinterpret_cast<const V *>(x);
     const V *yv = reinterpret_cast<const V *>(y);
     const V *zv = reinterpret_cast<const V *>(z);
     V *ov = reinterpret_cast<V *>(out);
-    for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < nvec; i += stride) {
-      V a = __builtin_nontemporal_load(xv + i), b = __builtin_nontemporal_load(yv + i),
-        c = __builtin_nontemporal_load(zv + i), r;
-      r.x = MulAdd::apply(a.x, b.x, c.x);
-      r.y = MulAdd::apply(a.y, b.y, c.y);
-      r.z = MulAdd::apply(a.z, b.z, c.z);
-      r.w = MulAdd::apply(a.w, b.w, c.w);
-      __builtin_nontemporal_store(r, ov + i);
+    const uint32_t base = blockIdx.x * (kThreads * 4);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t i = base + threadIdx.x + u * kThreads;
+      if (i < nvec) {
+        V a = __builtin_nontemporal_load(xv + i), b = __builtin_nontemporal_load(yv + i),
+          c = __builtin_nontemporal_load(zv + i), r;
+        r.x = MulAdd::apply(a.x, b.x, c.x);
+        r.y = MulAdd::apply(a.y, b.y, c.y);
+        r.z = MulAdd::apply(a.z, b.z, c.z);
+        r.w = MulAdd::apply(a.w, b.w, c.w);
+        __builtin_nontemporal_store(r, ov + i);
+      }
     }
-    if (blockIdx.x == 0) {
-      uint32_t t = (nvec << 2) + threadIdx.x;
+    if (nvec >= base && nvec < base + kThreads * 4) { // the last workgroup also takes the n % 4 tail
+      const uint32_t t = (nvec << 2) + threadIdx.x;
       if (t < n) out[t] = MulAdd::apply(x[t], y[t], z[t]);
     }
   } else {
+    const uint32_t stride = gridDim.x * kThreads;
     for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
       out[i] = MulAdd::apply(x[i], y[i], z[i]);
   }

@@ -42,14 +42,18 @@ int check_1d(const char *who, int32_t n, int64_t per_program, const uint32_t gri
   return RT_OK;
 }
 
-// Persistent physical grid: enough workgroups to fill every CU, never more
-// than there are UNROLL-vector groups to stream.
-uint32_t streaming_grid(uint32_t n_eff) {
+// One workgroup per run of kThreads*kUnroll vectors (plus one for a ragged end / scalar
+// tail); the unaligned kernels use a grid-stride loop over a grid sized to the CU count.
+uint32_t streaming_grid(uint32_t n_eff, bool aligned) {
+  if (aligned) {
+    const uint32_t nvec = n_eff >> 2, per_wg = kThreads * kUnroll;
+    uint32_t wgs = nvec / per_wg;
+    if (wgs * per_wg < nvec || (n_eff & 3u) || wgs == 0) ++wgs; // ragged end or scalar tail
+    return wgs;
+  }
   const rt_props *p = props();
-  int wg_per_cu = env_int("TTAMD_EW_WG_PER_CU", 8);
-  int64_t cap = (int64_t)p->multiprocessor_count * wg_per_cu;
-  int64_t need = cdiv64((int64_t)n_eff, (int64_t)kThreads * 4 * kUnroll);
-  return (uint32_t)std::max<int64_t>(1, std::min(cap, need));
+  int64_t cap = (int64_t)p->multiprocessor_count * env_int("TTAMD_EW_WG_PER_CU", 8);
+  return (uint32_t)std::max<int64_t>(1, std::min(cap, cdiv64((int64_t)n_eff, kThreads)));
 }
 
 } // namespace
@@ -73,7 +77,7 @@ static int add_common(const char *who, const void *x, const void *y, void *out, 
   const char *name = dtype == TT_F32 ? (al ? "ew_add_f32" : "ew_add_f32_unaligned")
                                      : (al ? "ew_add_i32" : "ew_add_i32_unaligned");
   void *args[] = {&x, &y, &out, &n_eff};
-  return launch("elementwise", name, dim3(streaming_grid(n_eff)), dim3(kThreads), 0, stream, args, 4);
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 4);
 }
 
 int tt_add_kernel(const void *x, const void *y, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
@@ -101,7 +105,7 @@ int tt_muladd_kernel(const void *x, const void *y, const void *z, void *out, int
   if (!x || !y || !z || !out) return fail(RT_ERR_INVALID, "muladd_kernel: null tensor pointer");
   uint32_t al = aligned16(x) && aligned16(y) && aligned16(z) && aligned16(out);
   void *args[] = {&x, &y, &z, &out, &n_eff, &al};
-  return launch("elementwise", "ew_muladd_f32", dim3(streaming_grid(n_eff)), dim3(kThreads), 0,
+  return launch("elementwise", "ew_muladd_f32", dim3(streaming_grid(n_eff, al != 0)), dim3(kThreads), 0,
                 stream, args, 6);
 }
 
@@ -116,7 +120,7 @@ int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SI
   bool al = aligned16(x) && aligned16(out);
   void *args[] = {&x, &out, &n_eff};
   return launch("elementwise", al ? "ew_sin_f32" : "ew_sin_f32_unaligned",
-                dim3(streaming_grid(n_eff)), dim3(kThreads), 0, stream, args, 3);
+                dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 3);
 }
 
 } // extern "C"
