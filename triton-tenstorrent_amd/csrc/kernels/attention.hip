@@ -167,3 +167,247 @@ ATTN_ANY(128)
 ATTN_ANY(256)
 
 } // extern "C"
+
+// ===========================================================================
+// attn_tile_d{64,128}: the fast path (N_CTX a multiple of 256, 16-byte aligned
+// contiguous rows, full grid).
+//
+// One workgroup = 8 wavefronts = 256 query rows of one (batch, head); K and V are
+// streamed through LDS in blocks of 64 keys, double buffered, shared by all eight
+// wavefronts; two wavefronts per SIMD, so one's softmax (VALU, exp2) overlaps the
+// other's MFMAs.  The per-wavefront math is the transposed scheme described at the
+// top of this file, with K fragments read row-wise (ds_read_b128) and V^T fragments
+// read through the transposing ds_read_b64_tr_b16.
+//
+// LDS tiles are [key][d] with 16-byte chunks XOR-swizzled:
+//   K: logical chunk c of row r sits at c ^ ((r / rows_per_256B) & (chunks-1))
+//   V: logical chunk c of row r sits at c ^ (vswz(r) << 2)   (4-row x 64-byte reads)
+// Global -> LDS copies are direct (global_load_lds_dwordx4): thread t writes byte
+// 16*t of each 8 KiB slab, the swizzle is applied to the global address.
+//
+// Workgroup order: a 1-D grid; ids are dealt round-robin to the 8 XCDs by the
+// dispatcher, so id -> (xcd, slot) -> head = xcd*heads_per_xcd + slot/qblocks keeps
+// every head's K/V inside one XCD's L2; within a head the late (heavy under the
+// causal mask) query blocks go first.
+// ===========================================================================
+namespace fastattn {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+typedef __attribute__((address_space(3))) void lds_void;
+
+constexpr int WAVES = 8, BM = WAVES * 32, BN = 64;
+
+template <int D>
+__device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *lds1) {
+  constexpr int DK = D / 16;            // k-steps of S^T
+  constexpr int DT = D / 32;            // 32-row tiles of O^T
+  constexpr int ROW = D * 2;            // bytes per K/V row
+  constexpr int CH = D / 8;             // 16-byte chunks per row
+  constexpr int RPB = 256 / ROW;        // rows per 256 bytes (1 for D=128, 2 for D=64)
+  constexpr int TILE = BN * ROW;        // bytes of one K (or V) tile
+  constexpr int SLAB = 512 * 16;        // bytes one pass of the 512 threads copies
+  constexpr int NSLAB = TILE / SLAB;    // 2 for D=128, 1 for D=64
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, hi = lane >> 5;
+
+  // ---- which (head, query block) ----
+  const int qblocks = a.rows / BM;
+  const int total = qblocks * a.heads;
+  int id = blockIdx.x;
+  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+  const int head = id / qblocks;
+  const int qblk = qblocks - 1 - (id % qblocks);
+  const int q0 = qblk * BM;
+  const int qw = q0 + wave * 32;        // this wavefront's first query
+  const int my_q = qw + c32;
+  const int64_t base = (int64_t)head * a.n_ctx;
+  const float qk_scale = a.sm_scale * 1.44269504f;
+  const int n_end = a.causal ? q0 + BM : a.n_ctx;
+  const int nblk = n_end / BN;
+
+  // ---- global -> LDS copy constants: thread t owns byte 16*t of each slab ----
+  // slab i covers rows i*(SLAB/ROW) ..; row = i*(SLAB/ROW) + t/CH, position t%CH
+  const int crow = tid / CH, cpos = tid % CH;
+  const int k_chunk = cpos ^ ((crow / RPB) & (CH - 1));
+  const int v_swz = (D == 128) ? (crow & 3) : ((crow >> 1) & 1);
+  const int v_chunk = cpos ^ (v_swz << 2);
+  const uint32_t k_voff = (uint32_t)(((int64_t)crow * a.ldk + k_chunk * 8) * 2);
+  const uint32_t v_voff = (uint32_t)(((int64_t)crow * a.ldv + v_chunk * 8) * 2);
+  const int lds_wave = wave * 1024;
+  const uint8_t *kg = (const uint8_t *)(a.k + base * a.ldk);
+  const uint8_t *vg = (const uint8_t *)(a.v + base * a.ldv);
+  auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst) {
+    const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst + lds_wave);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(src_uniform)
+                 : "memory", "m0");
+  };
+  auto dma_block = [&](int blk, uint8_t *stage) { // K tile then V tile of key block blk
+    const int64_t row0 = (int64_t)blk * BN;
+#pragma unroll
+    for (int i = 0; i < NSLAB; ++i)
+      dma_one(kg + (row0 + i * (SLAB / ROW)) * a.ldk * 2, k_voff, stage + i * SLAB);
+#pragma unroll
+    for (int i = 0; i < NSLAB; ++i)
+      dma_one(vg + (row0 + i * (SLAB / ROW)) * a.ldv * 2, v_voff, stage + TILE + i * SLAB);
+  };
+
+  // ---- fragment read constants ----
+  // K (A operand of S^T): lane = key row c32 of a 32-key tile, chunk 2s+hi of its row
+  const int k_rowoff = c32 * ROW;
+  const int k_x = (c32 / RPB) & (CH - 1);
+  // V^T (A operand of O^T) through transposing reads: see the B operand of the GEMM
+  const int G4 = lane >> 4, i16 = lane & 15, qd = i16 >> 2;
+  // key row within a 16-key step: h2*8 + hi*4 + qd ; d chunk (4 elems): dt*32 + (G4&1)*16 + (i16&3)*4
+  const int v_key = hi * 4 + qd; // + h2*8 + step*16
+  const int v_cc = (G4 & 1) * 2 + ((i16 >> 1) & 1); // 16-byte chunk within the 64-byte d-tile window
+  const int v_half = (i16 & 1) << 3;
+
+  // ---- Q fragments (B operand of S^T), straight from global ----
+  union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; };
+  Frag qf[DK];
+  {
+    const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
+#pragma unroll
+    for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+  }
+  f32x16 acc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) acc[t] = (f32x16){0};
+  float m_i = -__builtin_inff(), l_i = 1.0f;
+
+  dma_block(0, lds0);
+  for (int b = 0; b < nblk; ++b) {
+    uint8_t *cur = (b & 1) ? lds1 : lds0;
+    uint8_t *nxt = (b & 1) ? lds0 : lds1;
+    // block b has landed; every wave is done with the other stage
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (b + 1 < nblk) dma_block(b + 1, nxt);
+    const int n0 = b * BN;
+    if (a.causal && n0 > qw + 31) continue; // wholly above this wavefront's diagonal (wave-uniform)
+
+    // ---- S^T = K . Q^T : two 32-key tiles ----
+    f32x16 st[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      st[kt] = (f32x16){0};
+      const uint8_t *kb = cur + kt * 32 * ROW + k_rowoff;
+#pragma unroll
+      for (int s = 0; s < DK; ++s) {
+        Frag kf;
+        kf.v = *(const bf16x8 *)(kb + (((2 * s + hi) ^ k_x) << 4));
+        st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[s].v, st[kt], 0, 0, 0);
+      }
+    }
+    // ---- online softmax (per lane = per query; keys run over registers and the hi half) ----
+    const bool on_band = a.causal && (n0 + BN - 1 > qw);
+    float rmax = -__builtin_inff();
+    float m_ij;
+    if (on_band) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = n0 + kt * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+          st[kt][r] = st[kt][r] * qk_scale + (my_q >= key ? 0.0f : -1.0e6f);
+          rmax = fmaxf(rmax, st[kt][r]);
+        }
+      rmax = xor32_max(rmax);
+      m_ij = fmaxf(m_i, rmax);
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[kt][r] -= m_ij;
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) rmax = fmaxf(rmax, st[kt][r]);
+      rmax = xor32_max(rmax);
+      m_ij = fmaxf(m_i, rmax * qk_scale);
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[kt][r] = st[kt][r] * qk_scale - m_ij;
+    }
+    float l_ij = 0.0f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        st[kt][r] = __builtin_amdgcn_exp2f(st[kt][r]);
+        l_ij += st[kt][r];
+      }
+    l_ij = xor32_sum(l_ij);
+    const float alpha = __builtin_amdgcn_exp2f(m_i - m_ij);
+    // alpha == 1 for every query of the wavefront once the running maxima have settled:
+    // multiplying by 1.0f is the identity, so the rescale can be skipped exactly
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[t][r] *= alpha;
+    }
+    l_i = l_i * alpha + l_ij;
+    m_i = m_ij;
+    // ---- P^T fragments: 16-key step k4 uses registers 8*(k4&1).. of st[k4>>1] ----
+    Frag pf[4];
+#pragma unroll
+    for (int k4 = 0; k4 < 4; ++k4)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) pf[k4].u[j] = f32_to_bf16(st[k4 >> 1][(k4 & 1) * 8 + j]);
+    // ---- O^T += V^T . P^T ----
+    const uint8_t *vb = cur + TILE;
+#pragma unroll
+    for (int k4 = 0; k4 < 4; ++k4) {
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+        Frag vf;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const int key = k4 * 16 + h2 * 8 + v_key; // row in the tile
+          const int swz = (D == 128) ? (key & 3) : ((key >> 1) & 1);
+          const int chunk = (t * 4 + v_cc) ^ (swz << 2);
+          vf.h[h2] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + key * ROW + (chunk << 4) + v_half));
+        }
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[k4].v, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // ---- epilogue ----
+  if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
+  const float inv_l = 1.0f / l_i;
+  uint16_t *orow = a.o + (base + my_q) * a.ldo;
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const int d = t * 32 + r4 * 8 + hi * 4;
+      uint16_t o4[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o4[j] = f32_to_bf16(acc[t][r4 * 4 + j] / l_i);
+      (void)inv_l;
+      typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+      u32x2_t pk = {(uint32_t)o4[0] | ((uint32_t)o4[1] << 16), (uint32_t)o4[2] | ((uint32_t)o4[3] << 16)};
+      *(u32x2_t *)(orow + d) = pk;
+    }
+}
+
+} // namespace fastattn
+
+extern "C" {
+
+#define ATTN_TILE(D)                                                                       \
+  __global__ __launch_bounds__(512) void attn_tile_d##D(AttnArgs a) {                      \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[2 * 64 * D * 2];                \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
+    fastattn::body<D>(a, lds0, lds1);                                                      \
+  }
+ATTN_TILE(64)
+ATTN_TILE(128)
+
+} // extern "C"
