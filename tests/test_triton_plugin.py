@@ -1,0 +1,112 @@
+"""The plugin surface under real Triton: target registration, option parsing, the stage pipeline
+on the host (no GPU needed to compile: nothing is generated for the device), and -- on the GPU --
+launching ``@triton.jit`` kernels through Triton's own JIT onto the prebuilt kernels."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+triton = pytest.importorskip("triton")
+
+from triton.backends.compiler import GPUTarget  # noqa: E402
+
+from triton_tenstorrent_amd.backend import compiler as ttc  # noqa: E402
+from triton_tenstorrent_amd.backend import driver as ttd  # noqa: E402
+
+TARGET = GPUTarget("tenstorrent", "gfx950", 64)
+
+
+def test_backend_surface():
+    assert ttc.TTBackend.supports_target(TARGET)
+    assert not ttc.TTBackend.supports_target(GPUTarget("hip", "gfx950", 64))
+    b = ttc.TTBackend(TARGET)
+    assert b.get_target_name(None) == "tenstorrent" and b.binary_ext == ttd.BINARY_EXT
+    o = b.parse_options({"num_warps": 8, "bogus": 1, "num_stages": None})
+    assert (o.num_warps, o.num_stages, o.arch, o.allowed_dot_input_precisions) == (8, 1, "gfx950", ("ieee", ))
+    assert len(o.hash()) == 64 and o.hash() != b.parse_options({}).hash()
+    md = type("M", (), dict(num_warps=4, num_ctas=1, shared=0, cluster_dims=(1, 1, 1)))
+    assert b.pack_metadata(md) == (4, 1, 0, 1, 1, 1)
+    assert b.get_codegen_implementation(o)["min_dot_size"](None, None) == (1, 1, 1)
+    assert ["tt.divisibility", 8] in ttc.TTBackend.parse_attr("D")     # the reference's 8, not upstream's 16
+    assert b.hash() == "0.1-gfx950"
+    stages = {}
+    b.add_stages(stages, o, triton.backends.compiler.Language.TRITON)
+    assert list(stages) == ["ttir", ttd.BINARY_EXT]
+    with pytest.raises(NotImplementedError):
+        b.add_stages({}, o, triton.backends.compiler.Language.GLUON)
+    with pytest.raises(ValueError):
+        b.add_stages({}, b.parse_options({"ttmlir_target": "d2m"}), triton.backends.compiler.Language.TRITON)
+    # every field the Triton front end reads from a backend's options exists
+    for f in ("supported_fp8_dtypes", "deprecated_fp8_dot_operand_dtypes", "default_dot_input_precision",
+              "max_num_imprecise_acc_default", "launch_cooperative_grid", "extern_libs", "sanitize_overflow",
+              "enable_fp_fusion", "num_ctas", "num_stages", "num_warps", "debug", "arch"):
+        assert hasattr(o, f)
+
+
+def _compile(fn, signature, constexprs):
+    from triton.backends import Backend, backends
+    from triton.compiler import ASTSource
+    backends["tenstorrent"] = Backend(compiler=ttc.TTBackend, driver=ttd.TTDriver)
+    try:
+        src = ASTSource(fn=fn, signature=signature, constexprs=constexprs)
+        return triton.compile(src, target=TARGET)
+    finally:
+        backends.pop("tenstorrent", None)
+
+
+def test_compile_on_host_binds_by_name(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton_tenstorrent_amd.examples import triton_kernels as tk
+    k = _compile(tk.add_kernel, {"x_ptr": "*fp32", "y_ptr": "*fp32", "output_ptr": "*fp32", "n_elements": "i32",
+                                 "BLOCK_SIZE": "constexpr"}, {"BLOCK_SIZE": 1024})
+    assert k.name == "add_kernel" and k.metadata.shared == 0
+    assert json.loads(k.kernel)["kernel"] == "add_kernel"
+    assert "tt.func public @add_kernel" in k.asm["ttir"]
+    assert k.packed_metadata[:3] == (4, 1, 0)
+
+    @triton.jit
+    def unknown_kernel(x_ptr, n):
+        tl_pid = triton.language.program_id(0)
+        triton.language.store(x_ptr + tl_pid, n)
+
+    with pytest.raises(Exception, match="no prebuilt gfx950 implementation"):
+        _compile(unknown_kernel, {"x_ptr": "*i32", "n": "i32"}, {})
+
+
+@pytest.mark.gpu
+def test_triton_jit_launches_prebuilt_kernels(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton.tools.tensor_descriptor import TensorDescriptor
+    from oracle import oracle as orc
+    from triton_tenstorrent_amd import runtime as rt
+    from triton_tenstorrent_amd.examples import triton_kernels as tk
+    ttc.register()
+    try:
+        n = 98432
+        x, y = torch.rand(n, device="cuda"), torch.rand(n, device="cuda")
+        out = torch.empty_like(x)
+        tk.add_kernel[lambda meta: (triton.cdiv(n, meta["BLOCK_SIZE"]), )](x, y, out, n, BLOCK_SIZE=1024)
+        assert rt.last_kernel_name() == "ew_add_f32"
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), orc.add(x.cpu().numpy(), y.cpu().numpy()).view(np.uint32))
+        s = torch.empty_like(x)
+        tk.sin_kernel[(triton.cdiv(n, 1024), )](x, s, n, BLOCK_SIZE=1024)
+        assert np.max(np.abs(s.cpu().numpy() - orc.sin(x.cpu().numpy()))) <= 2e-6
+        M = N = Kd = 512
+        a = (torch.randn(M, Kd, device="cuda") / 16).to(torch.bfloat16)
+        b = torch.randn(Kd, N, device="cuda").to(torch.bfloat16)
+        c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+        ad, bd, cd = (TensorDescriptor.from_tensor(a, [128, 64]), TensorDescriptor.from_tensor(b, [64, 128]),
+                      TensorDescriptor.from_tensor(c, [128, 128]))
+        tk.matmul_kernel_tma[(16, )](ad, bd, cd, M, N, Kd, BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64,
+                                     GROUP_SIZE_M=8, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+        assert rt.last_kernel_name().startswith("gemm_tile_bf16")
+        ref = (a.double() @ b.double()).float()
+        assert torch.all((c.float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4)
+        # do_bench drives the device interface of the active driver
+        ms = triton.testing.do_bench(lambda: tk.add_kernel[(97, )](x, y, out, n, BLOCK_SIZE=1024), warmup=5, rep=20)
+        assert 0 < ms < 10
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None  # back to the stock driver, lazily
