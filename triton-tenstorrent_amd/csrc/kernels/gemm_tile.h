@@ -142,6 +142,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // The 12 LDS reads of one sub-step, in the order the MFMAs will want them:
   // b0.lo b0.hi a0 b1.lo b1.hi b2.lo b2.hi b3.lo b3.hi a1 a2 a3
   auto rd = [&](Frags &f, const uint8_t *stage, int s, int r) {
+#ifdef EXP_NO_LDSREAD
+    if (g.K > 0) return;
+#endif
     switch (r) {
     case 2: f.a[0] = *(const vec *)(stage + a_pos[s]); break;
     case 9: f.a[1] = *(const vec *)(stage + a_pos[s] + 2048); break;
@@ -167,6 +170,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // hand instead: copies retire in issue order, and each step's barrier waits with
   // s_waitcnt vmcnt(n) for exactly the copies that the following reads depend on.
   auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+#ifdef EXP_NO_DMA
+    if (g.K > 0) return;
+#endif
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
@@ -181,55 +187,71 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp) {
     int tm, tn;
     tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
+#ifdef EXP_SAME_TILE
+    tm = tn = 0;
+#endif
+#ifdef EXP_XCD_TILE
+    tm = blockIdx.x % 8; tn = 0;
+#endif
     ap = A + (int64_t)tm * BM * g.lda * 2;
     bp = B + (int64_t)tn * BN * 2;
   };
-  // copies of step kk (kk may run past nk into the next tile) into ring stage I
-  auto dma_pair = [&](int kk, uint8_t *stage, int i) { // i = 0..3: two of the eight loads
+  // copy number i (0..3: A slabs, 4..7: B slabs) of step kk into `stage`; kk may run past
+  // nk into the next tile
+  auto dma_single = [&](int kk, uint8_t *stage, int i) {
     const bool over = kk >= nk;
     const int k = over ? kk - nk : kk;
-    const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * (BK * 2);
-    const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
-    if (i < 2) {
-      dma_one(ap + (2 * i) * a_slab, a_voff, stage + (2 * i) * 4096);
-      dma_one(ap + (2 * i + 1) * a_slab, a_voff, stage + (2 * i + 1) * 4096);
+#ifdef EXP_ONLY_A
+    if (i >= 4 && g.K > 0) return;
+#endif
+#ifdef EXP_ONLY_B
+    if (i < 4 && g.K > 0) return;
+#endif
+    if (i < 4) {
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * (BK * 2);
+      dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
-      dma_one(bp + (2 * i - 4) * b_slab, b_voff, stage + A_BYTES + (2 * i - 4) * 4096);
-      dma_one(bp + (2 * i - 3) * b_slab, b_voff, stage + A_BYTES + (2 * i - 3) * 4096);
+      const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
+      dma_one(bp + (i - 4) * b_slab, b_voff, stage + A_BYTES + (i - 4) * 4096);
     }
   };
 
   // One step (K += 32) on ring stage I.
   //   entry: f0 holds sub-step 0 of stage I; copies for the next R-1 steps are in flight
-  //   exit : f0 holds sub-step 0 of stage I+1; the copy of step k+R into stage I is in flight
+  //   exit : f0 holds sub-step 0 of stage I+1
+  // The eight copies that refill a stage are spread thinly, one per four MFMAs, over the
+  // step period that follows the barrier which frees it (second half of this step, first
+  // half of the next): a wavefront that issues copies back to back stalls behind the
+  // memory pipeline's input queue, and its MFMAs stall with it.
   auto step = [&](auto I_, int k) {
     constexpr int I = decltype(I_)::value;
-    uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
-    // sub-step 0: MFMAs on f0, sub-step 1's fragments ride along (two reads per MFMA)
+    uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R], *prv = ring.s[(I + R - 1) % R];
+    // sub-step 0: MFMAs on f0; sub-step 1's fragments ride along (two reads per MFMA);
+    // second half of the refill of the stage freed one step ago
 #pragma unroll
     for (int n = 0; n < 16; ++n) {
       if (n < 6) {
         rd(f1, cur, 1, 2 * n);
         rd(f1, cur, 1, 2 * n + 1);
       }
+      if ((n & 3) == 1) dma_single(k - 1 + R, prv, 4 + (n >> 2));
       mm(f0, n);
       FENCE();
     }
     // All of this wave's reads of stage I have returned, and so has its share of the
-    // copy into stage I+1 (the R-2 younger copies may still be in flight).  After the
+    // copy into stage I+1 (the 16 younger copies may still be in flight).  After the
     // barrier that holds for every wave: I+1 may be read, I may be overwritten.
-    static_assert(DMA_PER_STEP * (R - 2) == 16, "the wait below is written for 16 younger copies");
     asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     FENCE();
-    // sub-step 1: MFMAs on f1; first the copy of step k+R into the freed stage (two loads
-    // per MFMA), then the next stage's sub-step 0 fragments
+    // sub-step 1: MFMAs on f1; the next stage's sub-step 0 fragments; first half of the
+    // refill of stage I with step k+R
 #pragma unroll
     for (int n = 0; n < 16; ++n) {
-      if (n < 4) dma_pair(k + R, cur, n);
-      if (n >= 4 && n < 10) {
-        rd(f0, nxt, 0, 2 * (n - 4));
-        rd(f0, nxt, 0, 2 * (n - 4) + 1);
+      if (n < 6) {
+        rd(f0, nxt, 0, 2 * n);
+        rd(f0, nxt, 0, 2 * n + 1);
       }
+      if ((n & 3) == 1) dma_single(k + R, cur, n >> 2);
       mm(f1, n);
       FENCE();
     }
@@ -240,12 +262,13 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   if (t >= total) return;
   tile_bases(t, a_cur, b_cur);
   tile_bases(t + gridDim.x < total ? t + gridDim.x : t, a_nxt, b_nxt);
+  // steps 0..R-2 whole, and the first half of step R-1 (step 0's first sub-step issues the rest)
 #pragma unroll
   for (int s = 0; s < R; ++s)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma_pair(s, ring.s[s], i);
-  static_assert(DMA_PER_STEP * (R - 1) == 24, "the wait below is written for 24 younger copies");
-  asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    for (int i = 0; i < (s == R - 1 ? 4 : 8); ++i) dma_single(s, ring.s[s], i);
+  static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume 8 copies per step and 4 stages");
+  asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
 #pragma unroll
   for (int r = 0; r < 12; ++r) rd(f0, ring.s[0], 0, r);
 
