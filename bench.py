@@ -189,7 +189,7 @@ def main() -> int:
         grid = (K.cdiv(M, 128) * K.cdiv(N, 128), )
         avg_ms, per, _ = _events_time(
             lambda: K.matmul_kernel_tma_fp8_scaled[grid](ad, bd, cd, M, N, Kd, sa, sb, FP8_OUTPUT=False, WARP_SPECIALIZE=False),
-            max(2, steps // 4), 1, stream)
+            steps, warmup, stream)
         tf = 2.0 * M * N * Kd / (avg_ms * 1e-3) / 1e12
         extra["gemm_fp8_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
                                   "TFLOPs": round(tf, 2)}
@@ -199,7 +199,7 @@ def main() -> int:
         Z, H, S, D = 4, 32, 4096, 128
         q, k, v = (torch.randn(Z, H, S, D, device="cuda").to(torch.bfloat16) for _ in range(3))
         sm = 1.0 / math.sqrt(D)
-        avg_ms, per, _ = _events_time(lambda: K.attention(q, k, v, True, sm), max(2, steps // 2), 2, stream)
+        avg_ms, per, _ = _events_time(lambda: K.attention(q, k, v, True, sm), steps, warmup, stream)
         fl = 4.0 * Z * H * S * S * D / 2  # lower triangle only
         tf = fl / (avg_ms * 1e-3) / 1e12
         extra["attn_fwd_causal_4x32x4096x128"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),

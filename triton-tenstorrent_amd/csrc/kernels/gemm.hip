@@ -102,3 +102,4 @@ GEMM_ANY(gemm_any_fp8_fp8, DT_FP8, DT_FP8)
 } // extern "C"
 
 #include "gemm_tile.h"
+#include "gemm_tile_fp8.h"

@@ -1,0 +1,226 @@
+// gemm_tile_fp8_*: fast path of the fp8 (OCP e4m3) tile matmul with per-tensor scales,
+// C = half(acc * scale_a * scale_b).
+//
+// Same organisation as the bf16 fast path (gemm_tile.h): 256x256 macro tile per workgroup
+// of 4 wavefronts, 128x128 per wavefront, a ring of four 32 KiB LDS stages filled by
+// direct-to-LDS copies three steps ahead, persistent XCD-aware grid, transposed product so
+// that the epilogue stores 4 consecutive n per lane.  What differs:
+//   * one step is K = 64 (64 one-byte elements per A row = the same 64 bytes as 32 bf16),
+//     consumed by ONE v_mfma_scale_f32_32x32x64_f8f6f4 per accumulator (block scales fixed
+//     at 1.0 = E8M0 0x7f; the per-tensor scales are applied in the epilogue);
+//   * a lane's operand is 32 bytes: k = 32*(lane/32) .. +31.  A rows are k-contiguous: two
+//     ds_read_b128.  B is [K,N] with n contiguous: ds_read_b64_tr_b8 transposes an 8x16
+//     block of bytes across 16 lanes (result lane i, byte j = source lane 2j + i/8, byte
+//     i%8), four of them per fragment;
+//   * LDS layout: A rows of 64 B, logical chunk c at c ^ ((m>>2)&3); B rows of 256 B,
+//     logical chunk c at c ^ ((k&7)<<1) (8 k-rows x 2 chunks land on 16 distinct bank
+//     groups).
+// Requirements: M, N multiples of 256, K a multiple of 256, 16-byte aligned rows, full grid.
+#pragma once
+#include <type_traits>
+
+#include "gemm_tile.h"
+
+namespace fast8 {
+
+constexpr int BM = 256, BN = 256, BK = 64, R = 4;
+constexpr int A_BYTES = BM * BK;       // 16 KiB
+constexpr int B_BYTES = BK * BN;       // 16 KiB
+constexpr int STAGE = A_BYTES + B_BYTES;
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+typedef __attribute__((address_space(3))) void lds_void;
+
+template <int OUT_DT>
+__device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  const int total = tiles_m * tiles_n;
+  const int nk = g.K / BK; // steps per tile, a multiple of R
+
+  // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
+  // A slab i (64 rows of 64 B): row = i*64 + (t>>2), position t&3 holds chunk (t&3)^((row>>2)&3)
+  const int a_row = tid >> 2;
+  const int a_chunk = (tid & 3) ^ ((a_row >> 2) & 3);
+  // B slab i (16 k-rows of 256 B): k = i*16 + (t>>4), position t&15 holds chunk (t&15)^((k&7)<<1)
+  const int b_k = tid >> 4;
+  const int b_chunk = (tid & 15) ^ ((b_k & 7) << 1);
+  const uint32_t a_voff = (uint32_t)((int64_t)a_row * g.lda + a_chunk * 16);
+  const uint32_t b_voff = (uint32_t)((int64_t)b_k * g.ldb + b_chunk * 16);
+  const int64_t a_slab = 64 * g.lda, b_slab = 16 * g.ldb;
+  const int64_t b_kstep = (int64_t)BK * g.ldb;
+  const int lds_wave = wave * 1024;
+
+  // ---- LDS -> fragments ----
+  const int l32 = lane & 31, hi = lane >> 5;
+  const int a_base = (wm * 128 + l32) * 64;
+  const int a_x = (l32 >> 2) & 3;
+  int a_pos[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) a_pos[h] = a_base + (((2 * hi + h) ^ a_x) << 4);
+  const int G4 = lane >> 4, i16 = lane & 15, rj = i16 >> 1;
+  int b_pos[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    b_pos[j] = A_BYTES + (hi * 32 + rj) * 256 + ((((wn * 8 + j * 2) ^ (rj << 1)) | (G4 & 1)) << 4) + ((i16 & 1) << 3);
+
+  const uint8_t *A = (const uint8_t *)g.a;
+  const uint8_t *B = (const uint8_t *)g.b;
+
+  struct Frags {
+    union { i32x4 q[2]; i32x8 v; } a[4];
+    union { i32x2 d[4]; i32x8 v; } b[4];
+  };
+  Frags f0, f1;
+  f32x16 acc[4][4];
+
+  // the 24 LDS reads of one step in the order the MFMAs want them:
+  // b0 (4 reads) a0 (2) b1 (4) b2 (4) b3 (4) a1 (2) a2 (2) a3 (2)
+  auto rd = [&](Frags &f, const uint8_t *stage, int r) {
+    auto rb = [&](int j, int q) {
+      f.b[j].d[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2 *)(stage + b_pos[j] + q * 2048));
+    };
+    auto ra = [&](int i, int h) { f.a[i].q[h] = *(const i32x4 *)(stage + a_pos[h] + i * 2048); };
+    if (r < 4) rb(0, r);
+    else if (r < 6) ra(0, r - 4);
+    else if (r < 18) rb(1 + (r - 6) / 4, (r - 6) % 4);
+    else ra(1 + (r - 18) / 2, (r - 18) % 2);
+  };
+  auto mm = [&](Frags &f, int n) {
+    const int i = n >> 2, j = n & 3;
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j].v, f.a[i].v, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                 0x7f7f7f7f);
+  };
+  auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+    const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0v), "v"(voff), "s"(src_uniform)
+                 : "memory", "m0");
+  };
+  const uint8_t *a_cur, *b_cur, *a_nxt, *b_nxt;
+  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp) {
+    int tm, tn;
+    fast::tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
+    ap = A + (int64_t)tm * BM * g.lda;
+    bp = B + (int64_t)tn * BN;
+  };
+  auto dma_single = [&](int kk, uint8_t *stage, int i) {
+    const bool over = kk >= nk;
+    const int k = over ? kk - nk : kk;
+    if (i < 4) {
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * BK;
+      dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
+    } else {
+      const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
+      dma_one(bp + (i - 4) * b_slab, b_voff, stage + A_BYTES + (i - 4) * 4096);
+    }
+  };
+
+  // One step (K += 64) on ring stage I: 16 MFMAs on `c` (read from stage I during the previous
+  // step), the next stage's fragments into `p`, and the refill of stage I itself with step k+R.
+  auto step = [&](auto I_, int k, Frags &c, Frags &p) {
+    constexpr int I = decltype(I_)::value;
+    uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
+    mm(c, 0);
+    FENCE();
+    // every wave's reads of stage I have returned (they fed `c`), and this wave's share of the
+    // copy into stage I+1 has landed (the 16 younger copies may still be in flight); after the
+    // barrier that holds for all waves: I+1 may be read, I may be overwritten
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    FENCE();
+#pragma unroll
+    for (int n = 1; n < 16; ++n) {
+      if (n <= 12) {
+        rd(p, nxt, 2 * (n - 1));
+        rd(p, nxt, 2 * (n - 1) + 1);
+      }
+      if (n & 1) dma_single(k + R, cur, n >> 1); // one copy per two MFMAs: thin enough not to stall issue
+      mm(c, n);
+      FENCE();
+    }
+  };
+
+  int t = blockIdx.x;
+  if (t >= total) return;
+  tile_bases(t, a_cur, b_cur);
+  tile_bases(t + gridDim.x < total ? t + gridDim.x : t, a_nxt, b_nxt);
+  // fill the ring with steps 0..R-1
+#pragma unroll
+  for (int s = 0; s < R; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_single(s, ring.s[s], i);
+  asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
+#pragma unroll
+  for (int r = 0; r < 24; ++r) rd(f0, ring.s[0], r);
+
+  for (; t < total; t += gridDim.x) {
+    int tm, tn;
+    fast::tile_of(t, tiles_m, tiles_n, tm, tn);
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
+    for (int k = 0; k < nk; k += R) {
+      step(std::integral_constant<int, 0>{}, k, f0, f1);
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0);
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1);
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0);
+    }
+    a_cur = a_nxt;
+    b_cur = b_nxt;
+    {
+      const int t2 = t + 2 * (int)gridDim.x;
+      tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt);
+    }
+    // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
+    //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
+    const int64_t m = m0 + wm * 128 + l32;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int64_t mi = m + i * 32;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
+          uint16_t o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float v = acc[i][j][r4 * 4 + e] * g.scale;
+            if constexpr (OUT_DT == DT_BF16) o[e] = f32_to_bf16(v);
+            else o[e] = f32_to_f16(v);
+          }
+          u32x2 pk = {(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
+          *(u32x2 *)((uint16_t *)g.c + mi * g.ldc + n) = pk;
+        }
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+} // namespace fast8
+
+extern "C" {
+
+#define GEMM_TILE_FP8(name, OUT)                                                                    \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast8::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast8::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                    \
+    fast8::body<OUT>(g, ring);                                                                       \
+  }
+
+GEMM_TILE_FP8(gemm_tile_fp8_bf16, DT_BF16)
+GEMM_TILE_FP8(gemm_tile_fp8_f16, DT_F16)
+
+} // extern "C"

@@ -126,6 +126,19 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     return lrc;
   }
 
+  // fp8 fast path: e4m3 in, bf16/fp16 out, scale in the epilogue, K in steps of 64 through a 4-stage ring
+  const bool fp8_io = in == TT_FP8E4M3 && (out == TT_BF16 || out == TT_F16) && epi == TT_EPI_NONE;
+  const bool fp8_shape = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
+  const bool fp8_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 16 == 0 && g.ldb % 16 == 0 &&
+                         g.ldc % 4 == 0;
+  if (full_grid && fp8_io && fp8_shape && fp8_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+    const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+    const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    void *fargs[] = {&g};
+    return launch("gemm", out == TT_BF16 ? "gemm_tile_fp8_bf16" : "gemm_tile_fp8_f16", dim3(wgs), dim3(256), 0, stream,
+                  fargs, 1);
+  }
+
   const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
   const int64_t cap = (int64_t)props()->multiprocessor_count * 8;
   const uint32_t blocks = (uint32_t)std::max<int64_t>(1, std::min(cap, cdiv64(items, 4)));
