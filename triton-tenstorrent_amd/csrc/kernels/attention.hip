@@ -34,6 +34,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   r = ((u & 0x7fffffffu) > 0x7f800000u) ? (u | 0x00400000u) : r;
   return (uint16_t)(r >> 16);
 }
+// two fp32 -> packed bf16 pair (lo in bits 0-15) with one v_cvt_pk_bf16_f32: round to nearest even
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 __device__ __forceinline__ float xor32_max(float v) {
   return fmaxf(v, __shfl_xor(v, 32, 64));
 }
@@ -267,7 +274,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   const int v_half = (i16 & 1) << 3;
 
   // ---- Q fragments (B operand of S^T), straight from global ----
-  union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; };
+  union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; uint32_t w[4]; };
   Frag qf[DK];
   {
     const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
@@ -358,7 +365,8 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
 #pragma unroll
     for (int k4 = 0; k4 < 4; ++k4)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) pf[k4].u[j] = f32_to_bf16(st[k4 >> 1][(k4 & 1) * 8 + j]);
+      for (int j = 0; j < 4; ++j)
+        pf[k4].w[j] = pack_bf16x2(st[k4 >> 1][(k4 & 1) * 8 + 2 * j], st[k4 >> 1][(k4 & 1) * 8 + 2 * j + 1]);
     // ---- O^T += V^T . P^T ----
     const uint8_t *vb = cur + TILE;
 #pragma unroll
@@ -380,19 +388,15 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // ---- epilogue ----
   if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
-  const float inv_l = 1.0f / l_i;
   uint16_t *orow = a.o + (base + my_q) * a.ldo;
 #pragma unroll
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
       const int d = t * 32 + r4 * 8 + hi * 4;
-      uint16_t o4[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) o4[j] = f32_to_bf16(acc[t][r4 * 4 + j] / l_i);
-      (void)inv_l;
       typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-      u32x2_t pk = {(uint32_t)o4[0] | ((uint32_t)o4[1] << 16), (uint32_t)o4[2] | ((uint32_t)o4[3] << 16)};
+      u32x2_t pk = {pack_bf16x2(acc[t][r4 * 4 + 0] / l_i, acc[t][r4 * 4 + 1] / l_i),
+                    pack_bf16x2(acc[t][r4 * 4 + 2] / l_i, acc[t][r4 * 4 + 3] / l_i)};
       *(u32x2_t *)(orow + d) = pk;
     }
 }

@@ -40,6 +40,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
   r = ((u & 0x7fffffffu) > 0x7f800000u) ? (u | 0x00400000u) : r;
   return (uint16_t)(r >> 16);
 }
+// two fp32 -> packed bf16 pair (lo in bits 0-15) with one v_cvt_pk_bf16_f32: round to nearest even
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 __device__ __forceinline__ float f16_to_f32(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }

@@ -190,14 +190,16 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
-          uint16_t o[4];
+          float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float v = acc[i][j][r4 * 4 + e] * g.scale;
-            if constexpr (OUT_DT == DT_BF16) o[e] = f32_to_bf16(v);
-            else o[e] = f32_to_f16(v);
+          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][r4 * 4 + e] * g.scale;
+          u32x2 pk;
+          if constexpr (OUT_DT == DT_BF16) {
+            pk = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          } else {
+            pk = (u32x2){(uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16),
+                         (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
           }
-          u32x2 pk = {(uint32_t)o[0] | ((uint32_t)o[1] << 16), (uint32_t)o[2] | ((uint32_t)o[3] << 16)};
           *(u32x2 *)((uint16_t *)g.c + mi * g.ldc + n) = pk;
         }
       }
