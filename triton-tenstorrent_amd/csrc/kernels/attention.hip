@@ -41,10 +41,25 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   f32x2_t v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
-__device__ __forceinline__ float xor32_max(float v) {
-  return fmaxf(v, __shfl_xor(v, 32, 64));
+// Reductions across the two wavefront halves.  v_permlane32_swap exchanges the high half of
+// its first register with the low half of its second: fed v twice it leaves the low half's
+// value in every lane of the first and the high half's in every lane of the second.  Written
+// as asm because the compiler's builtin folds the second result into the first; the s_nop
+// covers the two wait states the instruction needs after a VALU write of its operands.
+struct Halves { float lo, hi; };
+__device__ __forceinline__ Halves halves_of(float v) {
+  Halves r = {v, v};
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(r.lo), "+v"(r.hi));
+  return r;
 }
-__device__ __forceinline__ float xor32_sum(float v) { return v + __shfl_xor(v, 32, 64); }
+__device__ __forceinline__ float xor32_max(float v) {
+  const Halves r = halves_of(v);
+  return fmaxf(r.lo, r.hi);
+}
+__device__ __forceinline__ float xor32_sum(float v) {
+  const Halves r = halves_of(v);
+  return r.lo + r.hi;
+}
 
 // Any HEAD_DIM in {16,32,64,128,256}; operands straight from global memory.
 template <int D> __device__ __forceinline__ void attn_any_body(const AttnArgs &a) {
