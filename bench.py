@@ -50,9 +50,23 @@ def _events_time(fn, steps: int, warmup: int, stream: int):
     return total / steps, per, wall_ms / steps
 
 
-def _roof(bound: str, achieved: float, peak: float, unit: str, traffic=None):
+# HBM-side bytes per launch, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file (KiB per
+# dispatch, FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0: what the same counters read for the int32 add, a
+# plain copy-like kernel of known size).  Not measured live: the counters need the profiler around the process.
+# profiles/bench_all_kernels_rocprofv3.md holds the raw readings and the commands.
+MEASURED_TRAFFIC_BYTES = {
+    "gemm_tile_bf16_epi0": int((2 * 811274 + 175491) * 1024),
+    "gemm_tile_bf16_epi2": int((2 * 386043 + 127622) * 1024),
+    "gemm_tile_fp8_bf16": int((2 * 403355 + 182167) * 1024),
+    "attn_tile_d128": int((2 * 197832 + 133120) * 1024),
+    "ew_add_i32": int((2 * 1048594 + 1048576) * 1024),
+    "ew_sin_f32": int((2 * 524419 + 1048598) * 1024),
+}
+
+
+def _roof(bound: str, achieved: float, peak: float, unit: str, kernel: str = ""):
     return {"bound": bound, "achieved": round(achieved, 3), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": traffic}
+            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(kernel)}
 
 
 def main() -> int:
@@ -109,7 +123,7 @@ def main() -> int:
         flops = 2.0 * M * N * Kd
         value = flops / (avg_ms * 1e-3) / 1e12
         ms_per_step = avg_ms
-        primary_roof = _roof("mfma", value, PEAK_BF16_TFLOPS, "TFLOP/s")
+        primary_roof = _roof("mfma", value, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_tile_bf16_epi0")
         extra["gemm_bf16_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
                                    "ms_min": round(min(per), 4), "ms_median": round(statistics.median(per), 4),
                                    "wall_ms_per_step": round(wall_ms, 4), "TFLOPs": round(value, 2),
@@ -138,7 +152,7 @@ def main() -> int:
         assert torch.equal(out[:1 << 20], x[:1 << 20] + y[:1 << 20])
         extra["add_i32_2p28"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
                                  "GBs": round(gbs, 1)}
-        rooflines["add_i32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s")
+        rooflines["add_i32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s", "ew_add_i32")
         del x, y, out
     if want("sin"):
         xs = (torch.rand(n_el, device="cuda") * 2 - 1) * (8 * math.pi)
@@ -149,7 +163,7 @@ def main() -> int:
         extra["sin_f32_2p28"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
                                  "GBs": round(gbs, 1),
                                  "max_abs_err_vs_f64": float((outs[:1 << 20].double() - torch.sin(xs[:1 << 20].double())).abs().max())}
-        rooflines["sin_f32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s")
+        rooflines["sin_f32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s", "ew_sin_f32")
         del xs, outs
     if want("add0"):
         n0 = 98432
@@ -175,7 +189,7 @@ def main() -> int:
         tf = 2.0 * Mf * Nf * Kf / (avg_ms * 1e-3) / 1e12
         extra["gemm_gelu_4096x14336x4096"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
                                               "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
-        rooflines["gemm_gelu_4096x14336x4096"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s")
+        rooflines["gemm_gelu_4096x14336x4096"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_tile_bf16_epi2")
         del a, b, c, bias
     if want("fp8"):
         xa = torch.randn(M, Kd, device="cuda")
@@ -193,7 +207,7 @@ def main() -> int:
         tf = 2.0 * M * N * Kd / (avg_ms * 1e-3) / 1e12
         extra["gemm_fp8_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
                                   "TFLOPs": round(tf, 2)}
-        rooflines["gemm_fp8_8192"] = _roof("mfma", tf, PEAK_FP8_TFLOPS, "TFLOP/s")
+        rooflines["gemm_fp8_8192"] = _roof("mfma", tf, PEAK_FP8_TFLOPS, "TFLOP/s", "gemm_tile_fp8_bf16")
         del qa, qb, c
     if want("attn"):
         Z, H, S, D = 4, 32, 4096, 128
@@ -204,7 +218,7 @@ def main() -> int:
         tf = fl / (avg_ms * 1e-3) / 1e12
         extra["attn_fwd_causal_4x32x4096x128"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
                                                   "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
-        rooflines["attn_fwd_causal_4x32x4096x128"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s")
+        rooflines["attn_fwd_causal_4x32x4096x128"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "attn_tile_d128")
         del q, k, v
 
     # ---------------- CPU baseline: the oracle on a bounded sample ---------
