@@ -74,7 +74,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,fused,fp8,attn,add0")
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,fused,fp8,tiled,attn,add0")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -209,6 +209,19 @@ def main() -> int:
                                   "TFLOPs": round(tf, 2)}
         rooflines["gemm_fp8_8192"] = _roof("mfma", tf, PEAK_FP8_TFLOPS, "TFLOP/s", "gemm_tile_fp8_bf16")
         del qa, qb, c
+    if want("tiled"):
+        # the pointer-based matmul_kernel on tile-major fp16 buffers, 32x32x32 tiles, same 8192^3 problem
+        at = K.tilize((torch.randn(M, Kd, device="cuda") / math.sqrt(Kd)).to(torch.float16), 32, 32)
+        bt = K.tilize((torch.randn(Kd, N, device="cuda") / math.sqrt(Kd)).to(torch.float16), 32, 32)
+        ct = torch.empty(M * N, device="cuda", dtype=torch.float16)
+        grid = (K.cdiv(M, 32) * K.cdiv(N, 32), )
+        avg_ms, per, _ = _events_time(lambda: K.matmul_kernel[grid](at, bt, ct, M, N, Kd, Kd, 1, N, 1, N, 1), steps, warmup,
+                                      stream)
+        tf = 2.0 * M * N * Kd / (avg_ms * 1e-3) / 1e12
+        extra["gemm_tiled_f16_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
+                                        "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
+        rooflines["gemm_tiled_f16_8192"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_tiled_f16_epi0")
+        del at, bt, ct
     if want("attn"):
         Z, H, S, D = 4, 32, 4096, 128
         q, k, v = (torch.randn(Z, H, S, D, device="cuda").to(torch.bfloat16) for _ in range(3))

@@ -211,6 +211,23 @@ TTAMD_API int tt_matmul_kernel_tma_fp8_scaled(const tt_desc2d *a, const tt_desc2
                                     int32_t GROUP_SIZE_M, const uint32_t grid[3],
                                     void *stream);
 
+/* matmul_kernel(a_ptr, b_ptr, c_ptr, M, N, K, stride_am, stride_ak, stride_bk,
+ *               stride_bn, stride_cm, stride_cn, BLOCK_SIZE_M, BLOCK_SIZE_N,
+ *               BLOCK_SIZE_K, GROUP_SIZE_M, ACTIVATION)
+ * examples/matmul/03-matrix-multiplication.py:242-391 (wrapper :403-421): the
+ * pointer-based kernel.  a, b and c are TILE-MAJOR buffers with tiles of
+ * BLOCK_M x BLOCK_K, BLOCK_K x BLOCK_N and BLOCK_M x BLOCK_N elements, row-major
+ * inside a tile, tiles in row-major order (:326-337, 349-357, 377-385); ragged
+ * edges need the buffers padded to whole tiles.  The strides are checked to be
+ * positive, as the kernel asserts, and otherwise unused, as in the kernel.
+ * in_dtype is TT_F16 or TT_BF16; c is always fp16 (:374).  leaky_relu != 0
+ * applies ACTIVATION == "leaky_relu" to the fp32 accumulator (:370-373, 396-397). */
+TTAMD_API int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t M, int32_t N,
+                     int32_t K, int64_t stride_am, int64_t stride_ak, int64_t stride_bk,
+                     int64_t stride_bn, int64_t stride_cm, int64_t stride_cn, int32_t BLOCK_SIZE_M,
+                     int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K, int32_t GROUP_SIZE_M,
+                     int32_t leaky_relu, int32_t in_dtype, const uint32_t grid[3], void *stream);
+
 /* _attn_fwd(sm_scale, M, Z, H, desc_q, desc_k, desc_v, desc_o, N_CTX, HEAD_DIM,
  *           BLOCK_M, BLOCK_N, FP8_OUTPUT, STAGE, warp_specialize, IS_HOPPER)
  * examples/fused-attn/06-fused-attention.py:143-215.  bf16 descriptors of shape

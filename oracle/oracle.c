@@ -22,6 +22,9 @@
  *   orc_sin_f32    : float64 libm sin rounded once to fp32
  *   orc_matmul_*   : textbook sum_k a*b vs numpy float64 on exactly
  *       representable inputs, B = I, tile-order independence
+ *   orc_matmul_tiled: its tile-major index maps against a brute-force python
+ *       loop; bit-equal to orc_matmul on the re-tiled operands, ragged shapes
+ *       included; the reference's own 32x64 @ 64x32 fp16 self-check (atol 1e-2)
  *   orc_attn_fwd   : textbook softmax attention in float64, row-0 closed form,
  *       uniform-K running mean, base-2 log-sum-exp identity
  *   GELU epilogue, fp8 scaled GEMM: NOT in the reference; "parity unpinned" by
@@ -432,6 +435,94 @@ ORC_API int orc_matmul(const void *a, int64_t lda, const void *b, int64_t ldb, v
             v = acc;
           }
           store_elem(c, (om + i) * ldc + on + j, out_dt, v);
+        }
+      }
+    }
+    free(accf); free(accd); free(at); free(bt);
+  }
+  return 0;
+}
+
+/*
+ * matmul_kernel, the pointer-based kernel on tile-major operands
+ * (examples/matmul/03-matrix-multiplication.py:242-391; leaky_relu :396-397).
+ * TILE_M/N/K are the BLOCK sizes (:262-264).  Element (m,k) of A lives at
+ *   ((m / TILE_M) * num_tiles_k + k / TILE_K) * TILE_M*TILE_K + (m % TILE_M) * TILE_K + k % TILE_K   (:326-337)
+ * element (k,n) of B at
+ *   ((k / TILE_K) * num_tiles_n + n / TILE_N) * TILE_K*TILE_N + (k % TILE_K) * TILE_N + n % TILE_N   (:349-357)
+ * and element (m,n) of C at the same form with (TILE_M, TILE_N, num_tiles_n)                        (:377-385).
+ * Row and column indices are wrapped (offs_m % M, offs_n % N, :308-309), loads are
+ * masked on k < K only (:340-342, 359-361), the store on m < M and n < N (:387-388).
+ * acc is fp32 (:320), the activation acts on it before the cast (:370-374), and the
+ * result is always cast to fp16 (:374).  The strides in the signature are not used
+ * by the kernel (:251-253) and are not taken here.  Program order as orc_matmul.
+ */
+ORC_API int orc_matmul_tiled(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K,
+                             int32_t BM, int32_t BN, int32_t BK, int32_t group_m, int32_t grid,
+                             int in_dt, int leaky_relu, int acc64, int nthreads) {
+  if (BM <= 0 || BN <= 0 || BK <= 0 || group_m <= 0 || M <= 0 || N <= 0) return -1;
+  int num_pid_m = (M + BM - 1) / BM, num_pid_n = (N + BN - 1) / BN;
+  if (grid > num_pid_m * num_pid_n) return -2;
+  nthreads = pick_threads(nthreads);
+  const int64_t ntk = (K + BK - 1) / BK, ntn = num_pid_n;
+#pragma omp parallel num_threads(nthreads)
+  {
+#ifdef _OPENMP
+    int w = omp_get_thread_num(), nw = omp_get_num_threads();
+#else
+    int w = 0, nw = 1;
+#endif
+    float *accf = (float *)malloc(sizeof(float) * (size_t)BM * BN);
+    double *accd = acc64 ? (double *)malloc(sizeof(double) * (size_t)BM * BN) : NULL;
+    float *at = (float *)malloc(sizeof(float) * (size_t)BM * BK);
+    float *bt = (float *)malloc(sizeof(float) * (size_t)BK * BN);
+    int64_t bs, be;
+    orc_block_range(grid, nw, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int pid_m, pid_n;
+      orc_tile_of_pid((int)pid, num_pid_m, num_pid_n, group_m, &pid_m, &pid_n);
+      int64_t om = (int64_t)pid_m * BM, on = (int64_t)pid_n * BN;
+      for (int i = 0; i < BM * BN; ++i) accf[i] = 0.0f;
+      if (acc64) for (int i = 0; i < BM * BN; ++i) accd[i] = 0.0;
+      for (int64_t kt = 0; kt < ntk; ++kt) {
+        for (int i = 0; i < BM; ++i) {
+          int64_t m = (om + i) % M;
+          for (int k = 0; k < BK; ++k) {
+            int64_t kk = kt * BK + k;
+            int64_t off = ((m / BM) * ntk + kk / BK) * ((int64_t)BM * BK) + (m % BM) * BK + kk % BK;
+            at[i * BK + k] = kk < K ? load_elem(a, off, in_dt) : 0.0f;
+          }
+        }
+        for (int k = 0; k < BK; ++k) {
+          int64_t kk = kt * BK + k;
+          for (int j = 0; j < BN; ++j) {
+            int64_t n = (on + j) % N;
+            int64_t off = ((kk / BK) * ntn + n / BN) * ((int64_t)BK * BN) + (kk % BK) * BN + n % BN;
+            bt[k * BN + j] = kk < K ? load_elem(b, off, in_dt) : 0.0f;
+          }
+        }
+        for (int i = 0; i < BM; ++i)
+          for (int k = 0; k < BK; ++k) {
+            float av = at[i * BK + k];
+            const float *brow = bt + (size_t)k * BN;
+            if (!acc64) {
+              float *arow = accf + (size_t)i * BN;
+              for (int j = 0; j < BN; ++j) arow[j] += av * brow[j];
+            } else {
+              double *arow = accd + (size_t)i * BN;
+              for (int j = 0; j < BN; ++j) arow[j] += (double)av * (double)brow[j];
+            }
+          }
+      }
+      for (int i = 0; i < BM; ++i) {
+        if (om + i >= M) break;
+        for (int j = 0; j < BN; ++j) {
+          if (on + j >= N) break;
+          float acc = acc64 ? (float)accd[(size_t)i * BN + j] : accf[(size_t)i * BN + j];
+          if (leaky_relu) acc = acc >= 0.0f ? acc : 0.01f * acc;
+          int64_t m = om + i, n = on + j;
+          int64_t off = ((m / BM) * ntn + n / BN) * ((int64_t)BM * BN) + (m % BM) * BN + n % BN;
+          store_elem(c, off, ORC_F16, acc);
         }
       }
     }

@@ -67,6 +67,8 @@ def lib() -> C.CDLL:
         L.orc_matmul.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, i32, i32, i32,
                                  i32, i32, C.c_int, C.c_int, C.c_int, f32, C.c_int, C.c_int]
         L.orc_matmul.restype = C.c_int
+        L.orc_matmul_tiled.argtypes = [vp, vp, vp] + [i32] * 8 + [C.c_int] * 4
+        L.orc_matmul_tiled.restype = C.c_int
         L.orc_attn_fwd.argtypes = [f32, vp, i32, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                    i32, C.c_int]
         L.orc_attn_fwd.restype = C.c_int
@@ -205,6 +207,40 @@ def matmul(a: np.ndarray, b: np.ndarray, *, in_dt: int = BF16, out_dt: int = BF1
                           BK, group_m, grid, in_dt, out_dt, epi, scale, int(acc64), nthreads)
     if rc != 0:
         raise ValueError(f"orc_matmul rejected the launch (code {rc})")
+    return out
+
+
+def tilize(x: np.ndarray, TR: int, TC: int) -> np.ndarray:
+    """Row-major [R,C] -> the tile-major buffer matmul_kernel addresses
+    (03-matrix-multiplication.py:326-337): tiles of TR x TC, row-major inside a tile,
+    tiles in row-major order; ragged edges are zero-filled."""
+    R, C = x.shape
+    tr, tc = cdiv(R, TR), cdiv(C, TC)
+    pad = np.zeros((tr * TR, tc * TC), dtype=x.dtype)
+    pad[:R, :C] = x
+    return np.ascontiguousarray(pad.reshape(tr, TR, tc, TC).transpose(0, 2, 1, 3)).reshape(-1)
+
+
+def untilize(flat: np.ndarray, R: int, C: int, TR: int, TC: int) -> np.ndarray:
+    """Inverse of :func:`tilize` (drops the padding)."""
+    tr, tc = cdiv(R, TR), cdiv(C, TC)
+    return np.ascontiguousarray(flat.reshape(tr, tc, TR, TC).transpose(0, 2, 1, 3).reshape(tr * TR, tc * TC)[:R, :C])
+
+
+def matmul_tiled(a_tiled: np.ndarray, b_tiled: np.ndarray, M: int, N: int, K: int, *, in_dt: int = F16,
+                 BM: int = 32, BN: int = 32, BK: int = 32, group_m: int = 1, grid: int | None = None,
+                 leaky_relu: bool = False, acc64: bool = False, out: np.ndarray | None = None,
+                 nthreads: int = 0) -> np.ndarray:
+    """matmul_kernel (03-matrix-multiplication.py:242-391) on tile-major buffers;
+    returns the tile-major fp16 C buffer (uint16 patterns)."""
+    assert a_tiled.size >= cdiv(M, BM) * cdiv(K, BK) * BM * BK and b_tiled.size >= cdiv(K, BK) * cdiv(N, BN) * BK * BN
+    grid = cdiv(M, BM) * cdiv(N, BN) if grid is None else grid
+    if out is None:
+        out = np.zeros(cdiv(M, BM) * cdiv(N, BN) * BM * BN, dtype=np.uint16)
+    rc = lib().orc_matmul_tiled(_p(a_tiled), _p(b_tiled), _p(out), M, N, K, BM, BN, BK, group_m, grid, in_dt,
+                                int(leaky_relu), int(acc64), nthreads)
+    if rc != 0:
+        raise ValueError(f"orc_matmul_tiled rejected the launch (code {rc})")
     return out
 
 

@@ -1,0 +1,152 @@
+"""matmul_kernel on tile-major buffers (examples/matmul/03-matrix-multiplication.py:242-391) through
+the launcher and the C ABI, against the oracle's restatement."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from triton_tenstorrent_amd import kernels as K
+from triton_tenstorrent_amd import runtime as rt
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(shape, seed, dtype=torch.float16):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.rand(shape, generator=g) - 0.5).to(dtype)
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _f16(buf_u16):
+    return buf_u16.view(np.float16).astype(np.float32)
+
+
+def _close(got, ref):
+    # the tile-matmul bar: |err| <= 1e-2*|ref| + 1e-4 against the fp64-accumulating oracle
+    return np.all(np.abs(got - ref) <= 1e-2 * np.abs(ref) + 1e-4)
+
+
+@pytest.mark.parametrize("M,N,K_,cfg", [
+    (32, 32, 64, {}),                                               # the reference's self-check shape
+    (70, 45, 50, {}),                                               # ragged in all three
+    (128, 192, 96, {"BLOCK_SIZE_M": 64, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 4}),
+    (33, 31, 17, {"BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 16}),
+])
+@pytest.mark.parametrize("act", ["", "leaky_relu"])
+def test_tiled_matmul_vs_oracle(M, N, K_, cfg, act):
+    c = {**K.MATMUL_POINTER_CONFIG, **cfg}
+    BM, BN, BK = c["BLOCK_SIZE_M"], c["BLOCK_SIZE_N"], c["BLOCK_SIZE_K"]
+    a, b = _rand((M, K_), 1), _rand((K_, N), 2)
+    at, bt = K.tilize(a, BM, BK), K.tilize(b, BK, BN)
+    assert np.array_equal(_bits(at), orc.tilize(_bits(a), BM, BK))          # same tiling as the oracle's
+    ct = K.matmul_tiled(at.cuda(), bt.cuda(), M, N, K_, activation=act, **cfg)
+    assert rt.last_kernel_name() == "gemm_anytiled_f16_f16"
+    ref = orc.matmul_tiled(_bits(at), _bits(bt), M, N, K_, in_dt=orc.F16, BM=BM, BN=BN, BK=BK,
+                           group_m=c["GROUP_SIZE_M"], leaky_relu=bool(act), acc64=True)
+    got = _bits(ct.cpu())
+    gm, rm = orc.untilize(got, M, N, BM, BN), orc.untilize(ref, M, N, BM, BN)
+    assert _close(_f16(gm), _f16(rm))
+    # the reference's own bar for this kernel: atol 1e-2 against a plain matmul (:438)
+    want = a.double() @ b.double()
+    want = torch.where(want >= 0, want, 0.01 * want) if act else want
+    assert np.max(np.abs(_f16(gm) - want.numpy())) <= 1e-2
+    assert torch.equal(K.untilize(ct.cpu(), M, N, BM, BN).view(torch.int16), torch.from_numpy(gm.view(np.int16)))
+
+
+def test_tiled_matmul_small_integers_are_exact_and_padding_is_untouched():
+    M, N, K_ = 70, 45, 50
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(-4, 5, (M, K_), generator=g).to(torch.float16)
+    b = torch.randint(-4, 5, (K_, N), generator=g).to(torch.float16)
+    ct = K.matmul_tiled(K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, K_)
+    assert torch.equal(K.untilize(ct.cpu(), M, N, 32, 32).float(), a.float() @ b.float())
+    # masked store (:387-388): elements of the padded C tiles beyond M, N are never written
+    c = torch.full((3 * 2 * 1024, ), float("nan"), dtype=torch.float16, device="cuda")
+    grid = (6, )
+    K.matmul_kernel[grid](K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), c, M, N, K_, K_, 1, N, 1, N, 1)
+    full = c.cpu().reshape(3, 2, 32, 32).permute(0, 2, 1, 3).reshape(96, 64)
+    assert not torch.isnan(full[:M, :N]).any() and torch.isnan(full[M:, :]).all() and torch.isnan(full[:, N:]).all()
+
+
+def test_tiled_matmul_bf16_inputs_give_fp16():
+    M, N, K_ = 64, 96, 128
+    a, b = _rand((M, K_), 4, torch.bfloat16), _rand((K_, N), 5, torch.bfloat16)
+    ct = K.matmul_tiled(K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, K_)
+    assert ct.dtype == torch.float16 and rt.last_kernel_name() == "gemm_anytiled_bf16_f16"
+    ref = orc.matmul_tiled(_bits(K.tilize(a, 32, 32)), _bits(K.tilize(b, 32, 32)), M, N, K_, in_dt=orc.BF16, acc64=True)
+    assert _close(_f16(_bits(ct.cpu())), _f16(ref))
+
+
+def test_partial_grid_and_errors():
+    M = N = 64
+    a, b = _rand((M, 32), 6), _rand((32, N), 7)
+    c = torch.full((4 * 1024, ), float("nan"), dtype=torch.float16, device="cuda")
+    K.matmul_kernel[(3, )](K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), c, M, N, 32, 32, 1, N, 1, N, 1)
+    assert torch.isnan(c[3 * 1024:]).all() and not torch.isnan(c[:3 * 1024]).any()
+    with pytest.raises(rt.InvalidLaunch):
+        K.matmul_kernel[(5, )](K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), c, M, N, 32, 32, 1, N, 1, N, 1)
+    with pytest.raises(rt.InvalidLaunch):   # the kernel asserts positive strides
+        K.matmul_kernel[(4, )](K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), c, M, N, 32, 0, 1, N, 1, N, 1)
+    with pytest.raises(rt.Unsupported):
+        K.matmul_tiled(K.tilize(a, 48, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, 32, BLOCK_SIZE_M=48)
+
+
+@pytest.mark.parametrize("act", ["", "leaky_relu"])
+def test_fast_path_tiled(act):
+    M, N, K_ = 512, 768, 256
+    a, b = _rand((M, K_), 8), _rand((K_, N), 9)
+    at, bt = K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda()
+    ct = K.matmul_tiled(at, bt, M, N, K_, activation=act)
+    assert rt.last_kernel_name() == ("gemm_tiled_f16_epi3" if act else "gemm_tiled_f16_epi0")
+    ref = orc.matmul_tiled(_bits(at.cpu()), _bits(bt.cpu()), M, N, K_, leaky_relu=bool(act), acc64=True)
+    assert _close(_f16(_bits(ct.cpu())), _f16(ref))
+    # and the reference wrapper on whole tiles: tensors handed over as they lie in memory
+    c2 = K.matmul(at.reshape(M, K_), bt.reshape(K_, N), activation=act)
+    assert torch.equal(c2.reshape(-1), ct)
+
+
+def test_fast_path_tiled_small_integers_exact_and_equal_to_any_path():
+    M, N, K_ = 256, 512, 384
+    g = torch.Generator().manual_seed(10)
+    a = torch.randint(-3, 4, (M, K_), generator=g).to(torch.float16)
+    b = torch.randint(-3, 4, (K_, N), generator=g).to(torch.float16)
+    at, bt = K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda()
+    ct = K.matmul_tiled(at, bt, M, N, K_)
+    assert rt.last_kernel_name() == "gemm_tiled_f16_epi0"
+    assert torch.equal(K.untilize(ct.cpu(), M, N, 32, 32).float(), a.float() @ b.float())
+    # one program short of the full grid takes the any-shape kernel; with GROUP_SIZE_M = 1 program p writes
+    # tile p of the tile-major result, so all tiles but the last must agree bit for bit
+    tiles = (M // 32) * (N // 32)
+    ca = torch.zeros_like(ct)
+    K.matmul_kernel[(tiles - 1, )](at, bt, ca, M, N, K_, K_, 1, N, 1, N, 1)
+    assert rt.last_kernel_name() == "gemm_anytiled_f16_f16"
+    assert torch.equal(ca[:(tiles - 1) * 1024], ct[:(tiles - 1) * 1024]) and not ca[(tiles - 1) * 1024:].any()
+
+
+def test_full_size_tiled_identity_and_scaling():
+    # 8192^3 through size-independent properties: B = I gives C = A bit for bit; 2A gives 2C
+    n = 8192
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a = ((torch.rand((n, n), device="cuda", generator=g) - 0.5) / 8).to(torch.float16)
+    at = K.tilize(a, 32, 32)
+    eye_t = K.tilize(torch.eye(n, device="cuda", dtype=torch.float16), 32, 32)
+    c = K.matmul_tiled(at, eye_t, n, n, n)
+    assert rt.last_kernel_name() == "gemm_tiled_f16_epi0"
+    assert torch.equal(c, at)
+    del eye_t
+    b = ((torch.rand((n, n), device="cuda", generator=g) - 0.5) / 8).to(torch.float16)
+    bt = K.tilize(b, 32, 32)
+    c1 = K.matmul_tiled(at, bt, n, n, n)
+    c2 = K.matmul_tiled(at * 2, bt, n, n, n)
+    # exact wherever c1 is clear of fp16's subnormal range (a value that rounded UP to 2^-14 counts as inside it);
+    # below, doubling the input keeps a bit that the rounded c1 lost
+    normal = c1.abs() >= 2.0 ** -13
+    assert torch.equal(c2[normal], c1[normal] * 2)
+    assert torch.all((c2[~normal].float() - 2 * c1[~normal].float()).abs() <= 2.0 ** -24)
+    rows = torch.randint(0, n, (32, ), device="cuda")
+    ref = (a[rows].double() @ b.double()).float()
+    got = K.untilize(c1, n, n, 32, 32)[rows].float()
+    assert torch.all((got - ref).abs() <= 1e-2 * ref.abs() + 1e-4)

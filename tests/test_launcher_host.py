@@ -63,7 +63,7 @@ def fake(monkeypatch):
     monkeypatch.setattr(drv.TTDriver, "get_current_device", lambda self: 0)
     monkeypatch.setattr(drv.TTDriver, "get_current_stream", lambda self, d=None: 0x1234)
     for k in (K.add_kernel, K.add_kernel_loop, K.sin_kernel, K.matmul_kernel_tma, K.matmul_kernel_fused, K._attn_fwd,
-              K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel):
+              K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel):
         k._cache.clear()
     return lib
 
@@ -214,3 +214,39 @@ def test_driver_surface():
     assert d.launcher_cls is drv.TTLauncher and isinstance(d.utils, drv.TTUtils)
     di = d.get_device_interface()
     assert hasattr(di, "Event") and hasattr(di, "synchronize") and hasattr(di, "enable_hook_timing")
+
+
+def test_pointer_matmul_binds_with_unit_strides_folded(fake):
+    # matmul_kernel(a,b,c, M,N,K, six strides, constexprs): the unit strides arrive as constexprs
+    # (03-matrix-multiplication.py:403-421 passes a.stride(1) == 1)
+    a, b, c = FakeTensor((64, 96), torch.float16), FakeTensor((96, 32), torch.float16), FakeTensor((64, 32), torch.float16)
+    launch = K.matmul_kernel[lambda META: (K.cdiv(64, META["BLOCK_SIZE_M"]) * K.cdiv(32, META["BLOCK_SIZE_N"]), )]
+    launch(a, b, c, 64, 32, 96, 96, 1, 32, 1, 32, 1, ACTIVATION="leaky_relu")
+    name, args = fake.calls[-1]
+    assert name == "tt_matmul_kernel"
+    assert args[3:6] == (64, 32, 96) and args[6:12] == (96, 1, 32, 1, 32, 1)
+    assert args[12:16] == (32, 32, 32, 1) and args[16] == 1 and args[17] == rt.TT_F16
+    assert list(args[18]) == [2, 1, 1]
+    launch(a, b, c, 64, 32, 96, 96, 1, 32, 1, 32, 1)
+    assert fake.calls[-1][1][16] == 0
+    with pytest.raises(rt.Unsupported):
+        launch(a, b, c, 64, 32, 96, 96, 1, 32, 1, 32, 1, ACTIVATION="relu")
+    with pytest.raises(rt.InvalidLaunch):      # c must be fp16
+        launch(a, b, FakeTensor((64, 32), torch.bfloat16), 64, 32, 96, 96, 1, 32, 1, 32, 1)
+    with pytest.raises(rt.InvalidLaunch):      # ragged M needs a buffer padded to whole tiles
+        launch(FakeTensor((60, 96), torch.float16), b, c, 60, 32, 96, 96, 1, 32, 1, 32, 1)
+
+
+def test_packaging_declares_the_triton_backends_entry_point():
+    # Triton 3.6 finds out-of-tree backends in the "triton.backends" entry-point group; the value must be a
+    # package with compiler.py and driver.py (triton/backends/__init__.py)
+    import importlib
+    import tomli
+    meta = tomli.loads((ROOT / "pyproject.toml").read_text())
+    ep = meta["project"]["entry-points"]["triton.backends"]
+    assert list(ep) == ["tenstorrent"]
+    pkg = importlib.import_module(ep["tenstorrent"])
+    comp, drv_mod = importlib.import_module(pkg.__name__ + ".compiler"), importlib.import_module(pkg.__name__ + ".driver")
+    assert hasattr(comp, "TTBackend") and hasattr(drv_mod, "TTDriver")
+    assert meta["tool"]["setuptools"]["package-dir"]["triton_tenstorrent_amd"] == "triton-tenstorrent_amd"
+    assert (ROOT / "triton-tenstorrent_amd" / "backend" / "name.conf").exists()

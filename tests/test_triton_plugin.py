@@ -65,6 +65,16 @@ def test_compile_on_host_binds_by_name(tmp_path, monkeypatch):
     assert "tt.func public @add_kernel" in k.asm["ttir"]
     assert k.packed_metadata[:3] == (4, 1, 0)
 
+    # the pointer-based matmul_kernel: its unit strides are constexprs, as Triton's specialiser makes them
+    sig = {"a_ptr": "*fp16", "b_ptr": "*fp16", "c_ptr": "*fp16", "M": "i32", "N": "i32", "K": "i32", "stride_am": "i32",
+           "stride_ak": "constexpr", "stride_bk": "i32", "stride_bn": "constexpr", "stride_cm": "i32",
+           "stride_cn": "constexpr", "BLOCK_SIZE_M": "constexpr", "BLOCK_SIZE_N": "constexpr",
+           "BLOCK_SIZE_K": "constexpr", "GROUP_SIZE_M": "constexpr", "ACTIVATION": "constexpr"}
+    k = _compile(tk.matmul_kernel, sig, {"stride_ak": 1, "stride_bn": 1, "stride_cn": 1, "BLOCK_SIZE_M": 32,
+                                         "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 1,
+                                         "ACTIVATION": "leaky_relu"})
+    assert k.name == "matmul_kernel" and "tt.dot" in k.asm["ttir"]
+
     @triton.jit
     def unknown_kernel(x_ptr, n):
         tl_pid = triton.language.program_id(0)
@@ -103,6 +113,19 @@ def test_triton_jit_launches_prebuilt_kernels(tmp_path, monkeypatch):
         assert rt.last_kernel_name().startswith("gemm_tile_bf16")
         ref = (a.double() @ b.double()).float()
         assert torch.all((c.float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4)
+        # the pointer-based kernel on tile-major fp16 buffers; its unit strides reach the launcher as constexprs
+        from triton_tenstorrent_amd import kernels as K
+        M, N, Kd = 256, 512, 128
+        ah = (torch.rand(M, Kd, device="cuda") - 0.5).to(torch.float16)
+        bh = (torch.rand(Kd, N, device="cuda") - 0.5).to(torch.float16)
+        ct = torch.empty(M * N, device="cuda", dtype=torch.float16)
+        tk.matmul_kernel[(M // 32 * (N // 32), )](K.tilize(ah, 32, 32), K.tilize(bh, 32, 32), ct, M, N, Kd, Kd, 1, N, 1,
+                                                  N, 1, BLOCK_SIZE_M=32, BLOCK_SIZE_N=32, BLOCK_SIZE_K=32,
+                                                  GROUP_SIZE_M=1, ACTIVATION="leaky_relu")
+        assert rt.last_kernel_name() == "gemm_tiled_f16_epi3"
+        ref = ah.double() @ bh.double()
+        ref = torch.where(ref >= 0, ref, 0.01 * ref).float()
+        assert torch.all((K.untilize(ct, M, N, 32, 32).float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4)
         # do_bench drives the device interface of the active driver
         ms = triton.testing.do_bench(lambda: tk.add_kernel[(97, )](x, y, out, n, BLOCK_SIZE=1024), warmup=5, rep=20)
         assert 0 < ms < 10

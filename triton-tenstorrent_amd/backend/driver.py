@@ -235,6 +235,32 @@ def _bind_matmul_fused(lib, cur, consts, grid, stream):
                                       grid, stream)
 
 
+def _bind_matmul(lib, cur, consts, grid, stream):
+    """matmul_kernel (examples/matmul/03-matrix-multiplication.py:242-260): three pointers, M, N, K and six
+    strides, of which the unit ones arrive as constexprs (Triton folds an int equal to 1)."""
+    a, b, c = cur.tensor(), cur.tensor(), cur.tensor()
+    M, N, K = (int(cur.scalar(n)) for n in ("M", "N", "K"))
+    strides = [int(cur.scalar(n)) for n in ("stride_am", "stride_ak", "stride_bk", "stride_bn", "stride_cm", "stride_cn")]
+    cur.done()
+    bm, bn, bk, g = _block_consts(consts, None)
+    act = consts.get("ACTIVATION", "") or ""
+    if act not in ("", "leaky_relu"):
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"matmul_kernel: ACTIVATION {act!r}; '' and 'leaky_relu' exist")
+    dt = _torch_dtype_code(a)
+    if _torch_dtype_code(b) != dt:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "matmul_kernel: a and b dtypes differ")
+    if _torch_dtype_code(c) != rt.TT_F16:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "matmul_kernel: c must be fp16 (the kernel casts to tl.float16)")
+    need = (-(-M // bm) * -(-K // bk) * bm * bk, -(-K // bk) * -(-N // bn) * bk * bn,
+            -(-M // bm) * -(-N // bn) * bm * bn) if min(bm, bn, bk) > 0 else (0, 0, 0)
+    for name, t, n in zip("abc", (a, b, c), need):
+        if not t.is_contiguous() or t.numel() < n:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"matmul_kernel: {name} must be a contiguous tile-major buffer of "
+                                   f"at least {n} elements, got {t.numel()}")
+    return lib.tt_matmul_kernel(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, *strides, bm, bn, bk, g,
+                                int(act == "leaky_relu"), dt, grid, stream)
+
+
 def _bind_attn_fwd(lib, cur, consts, grid, stream):
     sm_scale = float(cur.scalar("sm_scale"))
     M = cur.tensor()
@@ -260,6 +286,7 @@ KERNEL_TABLE: dict[str, Callable] = {
     "matmul_kernel_tma": _bind_matmul_tma,
     "matmul_kernel_tma_fp8_scaled": _bind_matmul_tma,
     "matmul_kernel_fused": _bind_matmul_fused,
+    "matmul_kernel": _bind_matmul,
     "_attn_fwd": _bind_attn_fwd,
 }
 

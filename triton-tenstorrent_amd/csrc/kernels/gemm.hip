@@ -1,7 +1,8 @@
-// Tile-matmul kernels for gfx950: matmul_kernel_tma, matmul_kernel_fused and the
-// fp8-scaled sibling
+// Tile-matmul kernels for gfx950: matmul_kernel_tma, matmul_kernel_fused, the
+// fp8-scaled sibling and the pointer-based matmul_kernel on tile-major buffers
 // (examples/matmul_tensor_descriptor/09-persistent-matmul.py:102-145,
-//  python/tutorials/09-matmul-fused.py:100-148).
+//  python/tutorials/09-matmul-fused.py:100-148,
+//  examples/matmul/03-matrix-multiplication.py:242-391).
 //
 // gemm_any_*   : every shape, stride, tile size (multiples of 32), partial
 //                logical grid, ragged edges with descriptor zero-padding and
@@ -41,7 +42,14 @@ template <> struct Frag<DT_FP8> {
   }
 };
 
-template <int IN_DT, int OUT_DT> __device__ __forceinline__ void gemm_any_body(const GemmArgs &g) {
+// Element offset of (r, c) in a tile-major buffer: tiles of TR x TC, row-major inside a tile,
+// ntc tiles per tile row (03-matrix-multiplication.py:326-337).
+__device__ __forceinline__ int64_t tiled_off(int64_t r, int64_t c, int TR, int TC, int64_t ntc) {
+  return ((r / TR) * ntc + c / TC) * ((int64_t)TR * TC) + (r % TR) * TC + c % TC;
+}
+
+template <int IN_DT, int OUT_DT, bool TILED = false>
+__device__ __forceinline__ void gemm_any_body(const GemmArgs &g) {
   using F = Frag<IN_DT>;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -51,6 +59,7 @@ template <int IN_DT, int OUT_DT> __device__ __forceinline__ void gemm_any_body(c
   const int64_t items = (int64_t)g.grid * spt;
   const int64_t stride = (int64_t)gridDim.x * waves_per_block;
   const int r32 = lane & 31, kg = lane >> 5;
+  const int64_t ntk = (g.K + g.BK - 1) / g.BK, ntn = g.num_pid_n; // tile-major only
   for (int64_t it = (int64_t)blockIdx.x * waves_per_block + wave; it < items; it += stride) {
     const int pid = (int)(it / spt), sub = (int)(it % spt);
     int pid_m, pid_n;
@@ -68,8 +77,13 @@ template <int IN_DT, int OUT_DT> __device__ __forceinline__ void gemm_any_body(c
       for (int j = 0; j < 8; ++j) {
         const int k = kb + j;
         const bool k_ok = k < g.K;
-        a.s[j] = (am_ok && k_ok) ? F::enc(g.a, am * g.lda + k) : (uint16_t)0;
-        b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, (int64_t)k * g.ldb + bn) : (uint16_t)0;
+        if constexpr (TILED) {
+          a.s[j] = (am_ok && k_ok) ? F::enc(g.a, tiled_off(am, k, g.BM, g.BK, ntk)) : (uint16_t)0;
+          b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, tiled_off(k, bn, g.BK, g.BN, ntn)) : (uint16_t)0;
+        } else {
+          a.s[j] = (am_ok && k_ok) ? F::enc(g.a, am * g.lda + k) : (uint16_t)0;
+          b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, (int64_t)k * g.ldb + bn) : (uint16_t)0;
+        }
       }
       acc = F::mfma(a.v, b.v, acc);
     }
@@ -80,7 +94,7 @@ template <int IN_DT, int OUT_DT> __device__ __forceinline__ void gemm_any_body(c
       const int64_t n = n0 + r32;
       if (m < g.M && n < g.N) {
         float v = apply_epilogue<OUT_DT>(g, acc[r] * g.scale, m, n);
-        store_from_f32<OUT_DT>(g.c, m * g.ldc + n, v);
+        store_from_f32<OUT_DT>(g.c, TILED ? tiled_off(m, n, g.BM, g.BN, ntn) : m * g.ldc + n, v);
       }
     }
   }
@@ -98,6 +112,11 @@ GEMM_ANY(gemm_any_f16_f16, DT_F16, DT_F16)
 GEMM_ANY(gemm_any_fp8_bf16, DT_FP8, DT_BF16)
 GEMM_ANY(gemm_any_fp8_f16, DT_FP8, DT_F16)
 GEMM_ANY(gemm_any_fp8_fp8, DT_FP8, DT_FP8)
+
+// matmul_kernel: tile-major operands, fp16 result whatever the input type
+// (03-matrix-multiplication.py:374)
+__global__ __launch_bounds__(256) void gemm_anytiled_f16_f16(GemmArgs g) { gemm_any_body<DT_F16, DT_F16, true>(g); }
+__global__ __launch_bounds__(256) void gemm_anytiled_bf16_f16(GemmArgs g) { gemm_any_body<DT_BF16, DT_F16, true>(g); }
 
 } // extern "C"
 

@@ -16,5 +16,6 @@ struct GemmArgs {
   int32_t num_pid_m, num_pid_n;
   int32_t epi;
   float scale;              // multiplies the accumulator before the cast
+  int32_t tiled;            // operands are tile-major buffers with tiles BM x BK, BK x BN, BM x BN (ld* unused)
   unsigned long long *probe; // diagnostic: workgroup 0 stores {core-clock cycles, 100 MHz ticks} of its run, or null
 };

@@ -88,7 +88,12 @@ struct Ring {
   uint8_t *s[R];
 };
 
-template <int IN_DT, int OUT_DT, int EPI>
+// TILED: operands are the tile-major buffers of the pointer-based matmul_kernel with 32x32x32
+// tiles (examples/matmul/03-matrix-multiplication.py:326-385).  A 32x32 tile is 2 KiB
+// contiguous, i.e. exactly 32 of this kernel's 64-byte LDS rows, so only the global addresses
+// of the copies and of the result change: a thread's offset inside a slab, the distance
+// between slabs and between K steps.  LDS layout, fragments and MFMA schedule are the same.
+template <int IN_DT, int OUT_DT, int EPI, bool TILED = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   using X = MFMA<IN_DT>;
   using vec = typename X::vec;
@@ -106,10 +111,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // B slab i (8 k-rows): k = i*8 + (t>>5), chunk position t&31 holds logical chunk (t&31)^((k&3)<<2)
   const int b_k = tid >> 5;
   const int b_chunk = (tid & 31) ^ ((b_k & 3) << 2);
-  const uint32_t a_voff = (uint32_t)(((int64_t)a_row * g.lda + a_chunk * 8) * 2); // bytes, per thread
-  const uint32_t b_voff = (uint32_t)(((int64_t)b_k * g.ldb + b_chunk * 8) * 2);
-  const int64_t a_slab = 64 * g.lda * 2, b_slab = 8 * g.ldb * 2;                   // bytes, uniform
-  const int64_t b_kstep = (int64_t)BK * g.ldb * 2;
+  // row-major:  A(m,k) at m*lda + k,  B(k,n) at k*ldb + n
+  // tile-major: A(m,k) at ((m/32)*ntk + k/32)*1024 + (m%32)*32 + k%32,
+  //             B(k,n) at ((k/32)*ntn + n/32)*1024 + (k%32)*32 + n%32          (elements)
+  const int64_t ntk = g.K / 32, ntn = g.N / 32;
+  const uint32_t a_voff = TILED ? (uint32_t)((((int64_t)(a_row >> 5) * ntk << 10) + (a_row & 31) * 32 + a_chunk * 8) * 2)
+                                : (uint32_t)(((int64_t)a_row * g.lda + a_chunk * 8) * 2); // bytes, per thread
+  const uint32_t b_voff = TILED ? (uint32_t)((((b_chunk >> 2) << 10) + b_k * 32 + (b_chunk & 3) * 8) * 2)
+                                : (uint32_t)(((int64_t)b_k * g.ldb + b_chunk * 8) * 2);
+  const int64_t a_slab = TILED ? 2 * ntk * 2048 : 64 * g.lda * 2;                  // bytes, uniform
+  const int64_t b_slab = TILED ? 8 * 32 * 2 : 8 * g.ldb * 2;
+  const int64_t a_kstep = TILED ? 2048 : BK * 2;
+  const int64_t b_kstep = TILED ? ntn * 2048 : (int64_t)BK * g.ldb * 2;
   const int lds_wave = wave * 1024;
 
   // ---- LDS -> fragments ----
@@ -193,8 +206,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #ifdef EXP_XCD_TILE
     tm = blockIdx.x % 8; tn = 0;
 #endif
-    ap = A + (int64_t)tm * BM * g.lda * 2;
-    bp = B + (int64_t)tn * BN * 2;
+    ap = A + (TILED ? (int64_t)tm * (BM / 32) * ntk * 2048 : (int64_t)tm * BM * g.lda * 2);
+    bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
   };
   // copy number i (0..3: A slabs, 4..7: B slabs) of step kk into `stage`; kk may run past
   // nk into the next tile
@@ -208,7 +221,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if (i < 4 && g.K > 0) return;
 #endif
     if (i < 4) {
-      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * (BK * 2);
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
@@ -316,7 +329,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
             pk = (u32x2){(uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16),
                          (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
           }
-          *(u32x2 *)((uint16_t *)g.c + mi * g.ldc + n) = pk;
+          const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
+          *(u32x2 *)((uint16_t *)g.c + coff) = pk;
         }
       }
     }
@@ -350,5 +364,18 @@ extern "C" {
 
 GEMM_TILE_ALL_EPI(gemm_tile_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
+
+// matmul_kernel on tile-major fp16 buffers, plain and with leaky_relu
+#define GEMM_TILED(name, EPI)                                                                      \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
+    fast::body<DT_F16, DT_F16, EPI, true>(g, ring);                                                 \
+  }
+GEMM_TILED(gemm_tiled_f16_epi0, EPI_NONE)
+GEMM_TILED(gemm_tiled_f16_epi3, EPI_LEAKY_RELU)
 
 } // extern "C"

@@ -1,4 +1,4 @@
-// tt_matmul_kernel_tma / tt_matmul_kernel_fused / tt_matmul_kernel_tma_fp8_scaled:
+// tt_matmul_kernel_tma / tt_matmul_kernel_fused / tt_matmul_kernel_tma_fp8_scaled / tt_matmul_kernel:
 // launch validation and kernel selection for the tile-matmul family.
 #include <algorithm>
 #include <cstdio>
@@ -176,6 +176,65 @@ int tt_matmul_kernel_tma_fp8_scaled(const tt_desc2d *a, const tt_desc2d *b, cons
   return run_matmul("matmul_kernel_tma_fp8_scaled", a, b, c, nullptr, M, N, K, BLOCK_SIZE_M,
                     BLOCK_SIZE_N, BLOCK_SIZE_K, GROUP_SIZE_M, TT_EPI_NONE, scale_a * scale_b, grid,
                     stream);
+}
+
+int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t M, int32_t N, int32_t K,
+                     int64_t stride_am, int64_t stride_ak, int64_t stride_bk, int64_t stride_bn,
+                     int64_t stride_cm, int64_t stride_cn, int32_t BLOCK_SIZE_M, int32_t BLOCK_SIZE_N,
+                     int32_t BLOCK_SIZE_K, int32_t GROUP_SIZE_M, int32_t leaky_relu, int32_t in_dtype,
+                     const uint32_t grid[3], void *stream) {
+  const char *who = "matmul_kernel";
+  if (!props()) return fail(RT_ERR_NOT_INIT, "%s: call rt_init first", who);
+  if (!grid) return fail(RT_ERR_INVALID, "%s: null grid", who);
+  if (!a_ptr || !b_ptr || !c_ptr) return fail(RT_ERR_INVALID, "%s: null operand", who);
+  if (M <= 0 || N <= 0 || K < 0) return fail(RT_ERR_INVALID, "%s: M,N,K = %d,%d,%d", who, M, N, K);
+  const int32_t BM = BLOCK_SIZE_M, BN = BLOCK_SIZE_N, BK = BLOCK_SIZE_K;
+  if (BM <= 0 || BN <= 0 || BK <= 0 || GROUP_SIZE_M <= 0)
+    return fail(RT_ERR_INVALID, "%s: BLOCK sizes and GROUP_SIZE_M must be positive", who);
+  if (BM % 32 || BN % 32)
+    return fail(RT_ERR_UNSUPPORTED, "%s: BLOCK_SIZE_M/N = %d/%d, multiples of 32 are supported", who, BM, BN);
+  // the kernel asserts positive strides (tl.assume, :292-297) and then does not use them
+  if (stride_am <= 0 || stride_ak <= 0 || stride_bk <= 0 || stride_bn <= 0 || stride_cm <= 0 || stride_cn <= 0)
+    return fail(RT_ERR_INVALID, "%s: strides must be positive", who);
+  if (in_dtype != TT_F16 && in_dtype != TT_BF16)
+    return fail(RT_ERR_UNSUPPORTED, "%s: input dtype %d; fp16 and bf16 are supported", who, in_dtype);
+  if ((reinterpret_cast<uintptr_t>(a_ptr) | reinterpret_cast<uintptr_t>(b_ptr) | reinterpret_cast<uintptr_t>(c_ptr)) & 1)
+    return fail(RT_ERR_INVALID, "%s: operands must be 2-byte aligned", who);
+  if (grid[1] != 1 || grid[2] != 1)
+    return fail(RT_ERR_INVALID, "%s: 1-D grid expected, got (%u,%u,%u)", who, grid[0], grid[1], grid[2]);
+  const int64_t num_pid_m = cdiv64(M, BM), num_pid_n = cdiv64(N, BN);
+  if (grid[0] == 0) return fail(RT_ERR_INVALID, "%s: empty grid", who);
+  if ((int64_t)grid[0] > num_pid_m * num_pid_n)
+    return fail(RT_ERR_INVALID, "%s: grid %u exceeds the %lld tiles of the problem", who, grid[0],
+                (long long)(num_pid_m * num_pid_n));
+
+  GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  g.a = a_ptr; g.b = b_ptr; g.c = c_ptr;
+  g.M = M; g.N = N; g.K = K; g.BM = BM; g.BN = BN; g.BK = BK;
+  g.group_m = GROUP_SIZE_M; g.grid = (int32_t)grid[0];
+  g.num_pid_m = (int32_t)num_pid_m; g.num_pid_n = (int32_t)num_pid_n;
+  g.epi = leaky_relu ? TT_EPI_LEAKY_RELU : TT_EPI_NONE;
+  g.scale = 1.0f;
+  g.tiled = 1;
+  void *args[] = {&g};
+
+  // Fast path: 32x32x32 tiles (the reference's configuration), whole 256x256x128 macro
+  // tiles, fp16, 16-byte aligned buffers, a grid that covers the problem.
+  const bool full_grid = (int64_t)grid[0] == num_pid_m * num_pid_n;
+  if (full_grid && in_dtype == TT_F16 && BM == 32 && BN == 32 && BK == 32 && M % 256 == 0 && N % 256 == 0 &&
+      K % 128 == 0 && K >= 128 && aligned16(a_ptr) && aligned16(b_ptr) && aligned16(c_ptr) &&
+      !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+    const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+    const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    return launch("gemm", leaky_relu ? "gemm_tiled_f16_epi3" : "gemm_tiled_f16_epi0", dim3(wgs), dim3(256), 0, stream,
+                  args, 1);
+  }
+  const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
+  const int64_t cap = (int64_t)props()->multiprocessor_count * 8;
+  const uint32_t blocks = (uint32_t)std::max<int64_t>(1, std::min(cap, cdiv64(items, 4)));
+  return launch("gemm", in_dtype == TT_F16 ? "gemm_anytiled_f16_f16" : "gemm_anytiled_bf16_f16", dim3(blocks), dim3(256),
+                0, stream, args, 1);
 }
 
 } // extern "C"

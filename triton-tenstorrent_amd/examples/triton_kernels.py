@@ -1,7 +1,8 @@
 """The example kernels written as ordinary ``@triton.jit`` functions, with the
 names and signatures of the reference's tutorials
 (python/tutorials/01-vector-add.py:29, examples/01-sin-kernel.py:17,
-examples/matmul_tensor_descriptor/09-persistent-matmul.py:102).
+examples/matmul_tensor_descriptor/09-persistent-matmul.py:102,
+examples/matmul/03-matrix-multiplication.py:242).
 
 With ``backend.compiler.register()`` in effect Triton's JIT parses these on the
 host, the backend binds each by name to its prebuilt gfx950 kernel and the
@@ -48,3 +49,35 @@ def matmul_kernel_tma(a_desc, b_desc, c_desc, M, N, K, BLOCK_SIZE_M: tl.constexp
         b = b_desc.load([k * BLOCK_SIZE_K, pid_n * BLOCK_SIZE_N])
         acc = tl.dot(a, b, acc)
     c_desc.store([pid_m * BLOCK_SIZE_M, pid_n * BLOCK_SIZE_N], acc.to(tl.bfloat16))
+
+
+@triton.jit
+def matmul_kernel(a_ptr, b_ptr, c_ptr, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm, stride_cn,
+                  BLOCK_SIZE_M: tl.constexpr, BLOCK_SIZE_N: tl.constexpr, BLOCK_SIZE_K: tl.constexpr,
+                  GROUP_SIZE_M: tl.constexpr, ACTIVATION: tl.constexpr):
+    # tile-major operands: tile (i, j) of a matrix with nt tiles per tile row starts at (i*nt + j) * tile elements
+    pid = tl.program_id(axis=0)
+    num_pid_m = tl.cdiv(M, BLOCK_SIZE_M)
+    num_pid_n = tl.cdiv(N, BLOCK_SIZE_N)
+    width = GROUP_SIZE_M * num_pid_n
+    first_pid_m = (pid // width) * GROUP_SIZE_M
+    rows = min(num_pid_m - first_pid_m, GROUP_SIZE_M)
+    pid_m = first_pid_m + (pid % rows)
+    pid_n = (pid % width) // rows
+    num_k = tl.cdiv(K, BLOCK_SIZE_K)
+    im = tl.arange(0, BLOCK_SIZE_M)
+    jn = tl.arange(0, BLOCK_SIZE_N)
+    kk = tl.arange(0, BLOCK_SIZE_K)
+    acc = tl.zeros((BLOCK_SIZE_M, BLOCK_SIZE_N), dtype=tl.float32)
+    for kt in range(num_k):
+        live = kt * BLOCK_SIZE_K + kk < K
+        a_tile = a_ptr + (pid_m * num_k + kt) * (BLOCK_SIZE_M * BLOCK_SIZE_K)
+        b_tile = b_ptr + (kt * num_pid_n + pid_n) * (BLOCK_SIZE_K * BLOCK_SIZE_N)
+        a = tl.load(a_tile + im[:, None] * BLOCK_SIZE_K + kk[None, :], mask=live[None, :], other=0.0)
+        b = tl.load(b_tile + kk[:, None] * BLOCK_SIZE_N + jn[None, :], mask=live[:, None], other=0.0)
+        acc = tl.dot(a, b, acc)
+    if ACTIVATION == "leaky_relu":
+        acc = tl.where(acc >= 0, acc, 0.01 * acc)
+    c_tile = c_ptr + (pid_m * num_pid_n + pid_n) * (BLOCK_SIZE_M * BLOCK_SIZE_N)
+    keep = (pid_m * BLOCK_SIZE_M + im[:, None] < M) & (pid_n * BLOCK_SIZE_N + jn[None, :] < N)
+    tl.store(c_tile + im[:, None] * BLOCK_SIZE_N + jn[None, :], acc.to(tl.float16), mask=keep)

@@ -4,7 +4,8 @@ Kernel objects take the arguments of the reference's ``@triton.jit`` functions
 in the same order; host wrappers mirror the reference's own
 (``add`` 01-vector-add.py:62-78, ``sin`` 01-sin-kernel.py:32-37, ``matmul_tma``
 09-persistent-matmul.py:148-176, fused ``matmul_tma`` 09-matmul-fused.py:151-181,
-``_attention.forward`` 06-fused-attention.py:224-273).
+``_attention.forward`` 06-fused-attention.py:224-273, pointer ``matmul``
+03-matrix-multiplication.py:403-421).
 """
 from __future__ import annotations
 
@@ -189,6 +190,64 @@ def _host_descriptor_pre_hook(nargs):
 
 
 _ATTN_CONSTEXPRS = ["HEAD_DIM", "BLOCK_M", "BLOCK_N", "FP8_OUTPUT", "STAGE", "warp_specialize", "IS_HOPPER"]
+# ---- pointer-based matmul_kernel on tile-major buffers ----------------------
+# the reference's configuration for this backend (03-matrix-multiplication.py:213-218)
+MATMUL_POINTER_CONFIG = {"BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 1}
+_MMP_CONSTEXPRS = ["BLOCK_SIZE_M", "BLOCK_SIZE_N", "BLOCK_SIZE_K", "GROUP_SIZE_M", "ACTIVATION"]
+matmul_kernel = PrebuiltKernel(
+    "matmul_kernel", ["a_ptr", "b_ptr", "c_ptr", "M", "N", "K", "stride_am", "stride_ak", "stride_bk", "stride_bn",
+                      "stride_cm", "stride_cn"] + _MMP_CONSTEXPRS, _MMP_CONSTEXPRS,
+    configs=[Config(dict(MATMUL_POINTER_CONFIG), num_stages=1, num_warps=1)], defaults={"ACTIVATION": ""})
+
+
+def tilize(x: torch.Tensor, TR: int, TC: int) -> torch.Tensor:
+    """Row-major [R,C] -> the flat tile-major buffer ``matmul_kernel`` addresses
+    (03-matrix-multiplication.py:326-337): TR x TC tiles, row-major inside a tile,
+    tiles in row-major order, ragged edges zero-filled."""
+    R, C_ = x.shape
+    tr, tc = cdiv(R, TR), cdiv(C_, TC)
+    if (tr * TR, tc * TC) != (R, C_):
+        x = torch.nn.functional.pad(x, (0, tc * TC - C_, 0, tr * TR - R))
+    return x.reshape(tr, TR, tc, TC).permute(0, 2, 1, 3).contiguous().reshape(-1)
+
+
+def untilize(flat: torch.Tensor, R: int, C_: int, TR: int, TC: int) -> torch.Tensor:
+    """Inverse of :func:`tilize`, dropping the padding."""
+    tr, tc = cdiv(R, TR), cdiv(C_, TC)
+    return flat.reshape(tr, tc, TR, TC).permute(0, 2, 1, 3).reshape(tr * TR, tc * TC)[:R, :C_].contiguous()
+
+
+def matmul_tiled(a_buf: torch.Tensor, b_buf: torch.Tensor, M: int, N: int, K: int, activation: str = "",
+                 **meta) -> torch.Tensor:
+    """Launch ``matmul_kernel`` on tile-major buffers (as :func:`tilize` makes them) and
+    return the flat tile-major fp16 result; any M, N, K."""
+    cfg = {**MATMUL_POINTER_CONFIG, **meta}
+    BM, BN = cfg["BLOCK_SIZE_M"], cfg["BLOCK_SIZE_N"]
+    c = torch.empty(cdiv(M, BM) * cdiv(N, BN) * BM * BN, device=a_buf.device, dtype=torch.float16)
+    grid = lambda META: (cdiv(M, META["BLOCK_SIZE_M"]) * cdiv(N, META["BLOCK_SIZE_N"]), )
+    # strides as the reference's wrapper passes them: those of row-major [M,K], [K,N], [M,N] views
+    matmul_kernel[grid](a_buf, b_buf, c, M, N, K, K, 1, N, 1, N, 1, ACTIVATION=activation, **meta)
+    return c
+
+
+def matmul(a: torch.Tensor, b: torch.Tensor, activation: str = "", **meta) -> torch.Tensor:
+    """The reference's wrapper (03-matrix-multiplication.py:403-421): ``a`` [M,K] and ``b``
+    [K,N] are handed to the kernel as they lie in memory, and the kernel reads that memory
+    tile-major; so is the [M,N] fp16 result laid out.  Without padding that needs whole tiles."""
+    assert a.shape[1] == b.shape[0], "Incompatible dimensions"
+    assert a.is_contiguous(), "Matrix A must be contiguous"
+    M, K = a.shape
+    K, N = b.shape
+    cfg = {**MATMUL_POINTER_CONFIG, **meta}
+    assert M % cfg["BLOCK_SIZE_M"] == 0 and N % cfg["BLOCK_SIZE_N"] == 0 and K % cfg["BLOCK_SIZE_K"] == 0, \
+        "tile-major operands without padding need whole tiles; use matmul_tiled on padded buffers"
+    c = torch.empty((M, N), device=a.device, dtype=torch.float16)
+    grid = lambda META: (cdiv(M, META["BLOCK_SIZE_M"]) * cdiv(N, META["BLOCK_SIZE_N"]), )
+    matmul_kernel[grid](a, b, c, M, N, K, a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                        ACTIVATION=activation, **meta)
+    return c
+
+
 _attn_fwd = PrebuiltKernel("_attn_fwd", ["sm_scale", "M", "Z", "H", "desc_q", "desc_k", "desc_v", "desc_o", "N_CTX"] +
                            _ATTN_CONSTEXPRS, _ATTN_CONSTEXPRS,
                            configs=[Config({"BLOCK_M": 128, "BLOCK_N": 64}, num_warps=4, pre_hook=_host_descriptor_pre_hook)])

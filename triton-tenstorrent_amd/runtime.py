@@ -82,6 +82,7 @@ SYMBOLS = {
     "tt_matmul_kernel_tma": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_fused": (C.c_int, [_DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma_fp8_scaled": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _f32, _f32, _i32, _i32, _i32, _i32, _G, _vp]),
+    "tt_matmul_kernel": (C.c_int, [_vp, _vp, _vp, _i32, _i32, _i32] + [C.c_int64] * 6 + [_i32] * 6 + [_G, _vp]),
     "tt_attn_fwd": (C.c_int, [_f32, _vp, _i32, _i32, _DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_last_kernel_name": (C.c_char_p, []),
 }
