@@ -74,7 +74,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,fused,fp8,tiled,attn,add0")
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,ops,fused,fp8,tiled,attn,add0")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -165,6 +165,23 @@ def main() -> int:
                                  "max_abs_err_vs_f64": float((outs[:1 << 20].double() - torch.sin(xs[:1 << 20].double())).abs().max())}
         rooflines["sin_f32_2p28"] = _roof("hbm", gbs, PEAK_HBM_GBS, "GB/s", "ew_sin_f32")
         del xs, outs
+    if want("ops"):
+        # the other operations of the elementwise family at the streaming size: they have to stay under the HBM shadow
+        xs = torch.rand(n_el, device="cuda") + 0.5
+        ys = torch.rand(n_el, device="cuda") + 0.5
+        outs = torch.empty_like(xs)
+        egrid = (K.cdiv(n_el, 1024), )
+        ops = {}
+        for op in ("exp", "log", "cos", "rsqrt", "sqrt"):
+            avg_ms, per, _ = _events_time(lambda: K.unary_kernel[egrid](xs, outs, n_el, BLOCK_SIZE=1024, OP=op),
+                                          max(3, steps // 4), 2, stream)
+            ops[op] = round(2 * 4 * n_el / (avg_ms * 1e-3) / 1e9, 1)
+        for op in ("div", "maximum"):
+            avg_ms, per, _ = _events_time(lambda: K.binary_kernel[egrid](xs, ys, outs, n_el, BLOCK_SIZE=1024, OP=op),
+                                          max(3, steps // 4), 2, stream)
+            ops[op] = round(3 * 4 * n_el / (avg_ms * 1e-3) / 1e9, 1)
+        extra["elementwise_ops_2p28_GBs"] = ops
+        del xs, ys, outs
     if want("add0"):
         n0 = 98432
         x0, y0 = torch.rand(n0, device="cuda"), torch.rand(n0, device="cuda")

@@ -53,7 +53,9 @@ typedef enum tt_dtype {
   TT_I32 = 1,     /* *i32     */
   TT_BF16 = 2,    /* *bf16    */
   TT_F16 = 3,     /* *fp16    */
-  TT_FP8E4M3 = 4  /* *fp8e4nv (OCP e4m3fn) */
+  TT_FP8E4M3 = 4, /* *fp8e4nv (OCP e4m3fn) */
+  TT_I16 = 5,     /* *i16 (result of a narrowing cast only) */
+  TT_I8 = 6       /* *i8  (result of a narrowing cast only) */
 } tt_dtype;
 
 /* ----------------------------------------------------------------------- */
@@ -179,6 +181,31 @@ TTAMD_API int tt_muladd_kernel(const void *x, const void *y, const void *z, void
  * examples/01-sin-kernel.py:17-29; fp32. */
 TTAMD_API int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
                   const uint32_t grid[3], void *stream);
+
+/* The elementwise operations the reference's compute lowering accepts
+ * (npu/lib/Dialect/TritonTenstorrent/Transforms/ConvertComputeOps.cpp:162-182), each as
+ * a kernel of the same masked-block form as sin_kernel / add_kernel: program pid owns
+ * BLOCK_SIZE consecutive fp32 elements, lanes at or past n_elements are masked.
+ *   unary (math.absf ceil cos exp exp2 floor log log2 rsqrt sin sqrt):  out[i] = op(x[i])
+ *   binary (arith.addf subf mulf divf maximumf minimumf):              out[i] = x[i] op y[i]
+ *   narrowing (arith.truncf fp32 -> bf16 / fp16, round to nearest even;
+ *              arith.trunci int32 -> int16 / int8, low bits kept)
+ * abs, ceil, floor, sqrt, the four arithmetic operations and the casts are exact
+ * (correctly rounded); maximum / minimum return NaN if either operand is NaN and
+ * order -0 below +0; the transcendental ones are within 2 ulp of the exact result. */
+typedef enum tt_unary_op {
+  TT_OP_ABS = 0, TT_OP_CEIL = 1, TT_OP_COS = 2, TT_OP_EXP = 3, TT_OP_EXP2 = 4, TT_OP_FLOOR = 5,
+  TT_OP_LOG = 6, TT_OP_LOG2 = 7, TT_OP_RSQRT = 8, TT_OP_SIN = 9, TT_OP_SQRT = 10
+} tt_unary_op;
+typedef enum tt_binary_op {
+  TT_OP_ADD = 0, TT_OP_SUB = 1, TT_OP_MUL = 2, TT_OP_DIV = 3, TT_OP_MAXIMUM = 4, TT_OP_MINIMUM = 5
+} tt_binary_op;
+TTAMD_API int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_elements,
+                    int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
+TTAMD_API int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_t n_elements,
+                     int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
+TTAMD_API int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
+                   int32_t in_dtype, int32_t out_dtype, const uint32_t grid[3], void *stream);
 
 /* matmul_kernel_tma(a_desc, b_desc, c_desc, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
  *                   BLOCK_SIZE_K, GROUP_SIZE_M, FP8_OUTPUT, WARP_SPECIALIZE)

@@ -20,6 +20,9 @@
  *       bijection properties
  *   orc_add_*      : closed form (numpy), bit-exact
  *   orc_sin_f32    : float64 libm sin rounded once to fp32
+ *   orc_unary/binary_f32: numpy's float32 operations bit for bit where the operation is
+ *       exact, numpy float64 rounded once elsewhere; hand-written tables for NaN and
+ *       signed zero in maximum/minimum
  *   orc_matmul_*   : textbook sum_k a*b vs numpy float64 on exactly
  *       representable inputs, B = I, tile-order independence
  *   orc_matmul_tiled: its tile-major index maps against a brute-force python
@@ -312,6 +315,91 @@ ORC_API void orc_sinf_f32(const float *x, float *out, int32_t n, int32_t block,
       int64_t lo = pid * (int64_t)block, hi = lo + block;
       if (hi > n) hi = n;
       for (int64_t i = lo; i < hi; ++i) out[i] = sinf(x[i]);
+    }
+  }
+}
+
+/*
+ * The unary and binary operations the reference's compute lowering accepts
+ * (npu/lib/Dialect/TritonTenstorrent/Transforms/ConvertComputeOps.cpp:162-182), in the
+ * masked-block form of sin_kernel / add_kernel.  Exact operations are done in fp32
+ * (IEEE: correctly rounded); transcendental ones in float64 libm, rounded once to fp32.
+ * arith.maximumf / minimumf: NaN if either operand is NaN, -0 ordered below +0.
+ * Operation codes are tt_unary_op / tt_binary_op of the C ABI header.
+ */
+static inline float orc_unary_apply(int op, float x) {
+  switch (op) {
+  case 0: return fabsf(x);
+  case 1: return ceilf(x);
+  case 2: return (float)cos((double)x);
+  case 3: return (float)exp((double)x);
+  case 4: return (float)exp2((double)x);
+  case 5: return floorf(x);
+  case 6: return (float)log((double)x);
+  case 7: return (float)log2((double)x);
+  case 8: return (float)(1.0 / sqrt((double)x));
+  case 9: return (float)sin((double)x);
+  default: return sqrtf(x);
+  }
+}
+static inline float orc_binary_apply(int op, float a, float b) {
+  switch (op) {
+  case 0: return a + b;
+  case 1: return a - b;
+  case 2: return a * b;
+  case 3: return a / b;
+  case 4:
+    if (a != a) return a;
+    if (b != b) return b;
+    if (a == b) return signbit(a) ? b : a;
+    return a > b ? a : b;
+  default:
+    if (a != a) return a;
+    if (b != b) return b;
+    if (a == b) return signbit(a) ? a : b;
+    return a < b ? a : b;
+  }
+}
+ORC_API int orc_unary_f32(int op, const float *x, float *out, int32_t n, int32_t block, int32_t grid,
+                          int nthreads) {
+  if (op < 0 || op > 10) return -1;
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      for (int64_t i = lo; i < hi; ++i) out[i] = orc_unary_apply(op, x[i]);
+    }
+  }
+  return 0;
+}
+ORC_API int orc_binary_f32(int op, const float *x, const float *y, float *out, int32_t n, int32_t block,
+                           int32_t grid, int nthreads) {
+  if (op < 0 || op > 5) return -1;
+  nthreads = pick_threads(nthreads);
+#pragma omp parallel for num_threads(nthreads) schedule(static, 1)
+  for (int w = 0; w < nthreads; ++w) {
+    int64_t bs, be;
+    orc_block_range(grid, nthreads, w, &bs, &be);
+    for (int64_t pid = bs; pid < be; ++pid) {
+      int64_t lo = pid * (int64_t)block, hi = lo + block;
+      if (hi > n) hi = n;
+      for (int64_t i = lo; i < hi; ++i) out[i] = orc_binary_apply(op, x[i], y[i]);
+    }
+  }
+  return 0;
+}
+/* arith.trunci: the low bits are kept */
+ORC_API void orc_trunci(const int32_t *x, void *out, int bits, int32_t n, int32_t block, int32_t grid) {
+  for (int64_t pid = 0; pid < grid; ++pid) {
+    int64_t lo = pid * (int64_t)block, hi = lo + block;
+    if (hi > n) hi = n;
+    for (int64_t i = lo; i < hi; ++i) {
+      if (bits == 16) ((int16_t *)out)[i] = (int16_t)(uint16_t)((uint32_t)x[i] & 0xffffu);
+      else ((int8_t *)out)[i] = (int8_t)(uint8_t)((uint32_t)x[i] & 0xffu);
     }
   }
 }

@@ -67,6 +67,11 @@ def lib() -> C.CDLL:
         L.orc_matmul.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, i32, i32, i32, i32,
                                  i32, i32, C.c_int, C.c_int, C.c_int, f32, C.c_int, C.c_int]
         L.orc_matmul.restype = C.c_int
+        L.orc_unary_f32.argtypes = [C.c_int, vp, vp, i32, i32, i32, C.c_int]
+        L.orc_unary_f32.restype = C.c_int
+        L.orc_binary_f32.argtypes = [C.c_int, vp, vp, vp, i32, i32, i32, C.c_int]
+        L.orc_binary_f32.restype = C.c_int
+        L.orc_trunci.argtypes = [vp, vp, C.c_int, i32, i32, i32]
         L.orc_matmul_tiled.argtypes = [vp, vp, vp] + [i32] * 8 + [C.c_int] * 4
         L.orc_matmul_tiled.restype = C.c_int
         L.orc_attn_fwd.argtypes = [f32, vp, i32, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
@@ -207,6 +212,41 @@ def matmul(a: np.ndarray, b: np.ndarray, *, in_dt: int = BF16, out_dt: int = BF1
                           BK, group_m, grid, in_dt, out_dt, epi, scale, int(acc64), nthreads)
     if rc != 0:
         raise ValueError(f"orc_matmul rejected the launch (code {rc})")
+    return out
+
+
+UNARY_OPS = {"abs": 0, "ceil": 1, "cos": 2, "exp": 3, "exp2": 4, "floor": 5, "log": 6, "log2": 7, "rsqrt": 8, "sin": 9,
+             "sqrt": 10}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
+
+
+def unary(op: str, x: np.ndarray, *, block: int = 1024, grid: int | None = None, out: np.ndarray | None = None,
+          nthreads: int = 0) -> np.ndarray:
+    """out[i] = op(x[i]) in the masked-block form (ConvertComputeOps.cpp:170-180)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros_like(x) if out is None else out
+    grid = cdiv(x.size, block) if grid is None else grid
+    if lib().orc_unary_f32(UNARY_OPS[op], _p(x), _p(out), x.size, block, grid, nthreads):
+        raise ValueError("orc_unary_f32 rejected the launch")
+    return out
+
+
+def binary(op: str, x: np.ndarray, y: np.ndarray, *, block: int = 1024, grid: int | None = None,
+           out: np.ndarray | None = None, nthreads: int = 0) -> np.ndarray:
+    """out[i] = x[i] op y[i] (ConvertComputeOps.cpp:162-167)."""
+    x, y = np.ascontiguousarray(x, dtype=np.float32), np.ascontiguousarray(y, dtype=np.float32)
+    out = np.zeros_like(x) if out is None else out
+    grid = cdiv(x.size, block) if grid is None else grid
+    if lib().orc_binary_f32(BINARY_OPS[op], _p(x), _p(y), _p(out), x.size, block, grid, nthreads):
+        raise ValueError("orc_binary_f32 rejected the launch")
+    return out
+
+
+def trunci(x: np.ndarray, bits: int, *, block: int = 1024, grid: int | None = None) -> np.ndarray:
+    """arith.trunci int32 -> int16 / int8 (ConvertComputeOps.cpp:182)."""
+    x = np.ascontiguousarray(x, dtype=np.int32)
+    out = np.zeros(x.shape, dtype=np.int16 if bits == 16 else np.int8)
+    lib().orc_trunci(_p(x), _p(out), bits, x.size, block, cdiv(x.size, block) if grid is None else grid)
     return out
 
 

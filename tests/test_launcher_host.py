@@ -63,7 +63,8 @@ def fake(monkeypatch):
     monkeypatch.setattr(drv.TTDriver, "get_current_device", lambda self: 0)
     monkeypatch.setattr(drv.TTDriver, "get_current_stream", lambda self, d=None: 0x1234)
     for k in (K.add_kernel, K.add_kernel_loop, K.sin_kernel, K.matmul_kernel_tma, K.matmul_kernel_fused, K._attn_fwd,
-              K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel):
+              K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel, K.unary_kernel, K.binary_kernel,
+              K.cast_kernel):
         k._cache.clear()
     return lib
 
@@ -250,3 +251,30 @@ def test_packaging_declares_the_triton_backends_entry_point():
     assert hasattr(comp, "TTBackend") and hasattr(drv_mod, "TTDriver")
     assert meta["tool"]["setuptools"]["package-dir"]["triton_tenstorrent_amd"] == "triton-tenstorrent_amd"
     assert (ROOT / "triton-tenstorrent_amd" / "backend" / "name.conf").exists()
+
+
+def test_generic_elementwise_ops_bind_by_mnemonic(fake):
+    x, o = FakeTensor((5000, ), torch.float32), FakeTensor((5000, ), torch.float32)
+    K.unary_kernel[(5, )](x, o, 5000, BLOCK_SIZE=1024, OP="exp2")
+    name, a = fake.calls[-1]
+    assert name == "tt_unary_kernel" and a[0] == rt.UNARY_OPS["exp2"] and a[3:5] == (5000, 1024) and list(a[5]) == [5, 1, 1]
+    K.binary_kernel[(5, )](x, x, o, 5000, BLOCK_SIZE=1024, OP="minimum")
+    name, a = fake.calls[-1]
+    assert name == "tt_binary_kernel" and a[0] == rt.BINARY_OPS["minimum"] and a[4:6] == (5000, 1024)
+    K.cast_kernel[(5, )](x, FakeTensor((5000, ), torch.bfloat16), 5000, BLOCK_SIZE=1024)
+    name, a = fake.calls[-1]
+    assert name == "tt_cast_kernel" and a[4:6] == (rt.TT_F32, rt.TT_BF16)
+    K.cast_kernel[(5, )](FakeTensor((5000, ), torch.int32), FakeTensor((5000, ), torch.int8), 5000, BLOCK_SIZE=1024)
+    assert fake.calls[-1][1][4:6] == (rt.TT_I32, rt.TT_I8)
+    with pytest.raises(rt.Unsupported):
+        K.unary_kernel[(5, )](x, o, 5000, BLOCK_SIZE=1024, OP="tanh")
+    with pytest.raises(rt.Unsupported):
+        K.binary_kernel[(5, )](x, FakeTensor((5000, ), torch.float16), o, 5000, BLOCK_SIZE=1024, OP="add")
+    # the op tables here, in the oracle and in the header agree
+    from oracle import oracle as orc
+    assert orc.UNARY_OPS == rt.UNARY_OPS and orc.BINARY_OPS == rt.BINARY_OPS
+    header = (ROOT / "include" / "ttamd_rt.h").read_text()
+    for name, code in rt.UNARY_OPS.items():
+        assert re.search(rf"TT_OP_{name.upper()} = {code}\b", header), name
+    for name, code in rt.BINARY_OPS.items():
+        assert re.search(rf"TT_OP_{name.upper()} = {code}\b", header), name

@@ -55,7 +55,7 @@ def _typestr_dtype(ty: str) -> int:
 def _torch_dtype_code(t) -> int:
     import torch
     table = {torch.float32: rt.TT_F32, torch.int32: rt.TT_I32, torch.bfloat16: rt.TT_BF16,
-             torch.float16: rt.TT_F16, torch.float8_e4m3fn: rt.TT_FP8E4M3}
+             torch.float16: rt.TT_F16, torch.float8_e4m3fn: rt.TT_FP8E4M3, torch.int16: rt.TT_I16, torch.int8: rt.TT_I8}
     if t.dtype not in table:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"tensor dtype {t.dtype} has no kernel")
     return table[t.dtype]
@@ -186,6 +186,45 @@ def _bind_sin(lib, cur, consts, grid, stream):
     return lib.tt_sin_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
 
 
+def _op_code(table: dict, consts: dict, who: str) -> int:
+    op = consts.get("OP")
+    if op not in table:
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"{who}: OP {op!r}; one of {sorted(table)}")
+    return table[op]
+
+
+def _bind_unary(lib, cur, consts, grid, stream):
+    """out[i] = OP(x[i]) for the unary operations of ConvertComputeOps.cpp:170-180."""
+    x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
+    n = int(cur.scalar("n_elements"))
+    cur.done()
+    if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "unary_kernel computes in fp32")
+    return lib.tt_unary_kernel(_op_code(rt.UNARY_OPS, consts, "unary_kernel"), x.data_ptr(), out.data_ptr(), n,
+                               int(consts["BLOCK_SIZE"]), grid, stream)
+
+
+def _bind_binary(lib, cur, consts, grid, stream):
+    """out[i] = x[i] OP y[i] for the binary operations of ConvertComputeOps.cpp:162-167."""
+    x, y, out = (_contiguous_1d(cur.tensor()) for _ in range(3))
+    n = int(cur.scalar("n_elements"))
+    cur.done()
+    for t in (x, y, out):
+        if _torch_dtype_code(t) != rt.TT_F32:
+            raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "binary_kernel computes in fp32")
+    return lib.tt_binary_kernel(_op_code(rt.BINARY_OPS, consts, "binary_kernel"), x.data_ptr(), y.data_ptr(),
+                                out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
+
+
+def _bind_cast(lib, cur, consts, grid, stream):
+    """out[i] = x[i].to(out dtype): arith.truncf / arith.trunci (ConvertComputeOps.cpp:181-182)."""
+    x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
+    n = int(cur.scalar("n_elements"))
+    cur.done()
+    return lib.tt_cast_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), _torch_dtype_code(x),
+                              _torch_dtype_code(out), grid, stream)
+
+
 def _mnk(cur: _Cursor, a: rt.tt_desc2d, b: rt.tt_desc2d):
     """M, N, K follow the descriptors when the signature carries them; the
     minimal variant reads them from ``desc.shape`` (kernel_matmul_tma.py:71-75).
@@ -283,6 +322,9 @@ KERNEL_TABLE: dict[str, Callable] = {
     "add_kernel": _bind_add,
     "muladd_kernel": _bind_muladd,
     "sin_kernel": _bind_sin,
+    "unary_kernel": _bind_unary,
+    "binary_kernel": _bind_binary,
+    "cast_kernel": _bind_cast,
     "matmul_kernel_tma": _bind_matmul_tma,
     "matmul_kernel_tma_fp8_scaled": _bind_matmul_tma,
     "matmul_kernel_fused": _bind_matmul_fused,

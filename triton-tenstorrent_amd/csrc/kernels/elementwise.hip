@@ -1,5 +1,7 @@
 // Elementwise streaming kernels for gfx950: add_kernel (fp32 / int32),
-// muladd_kernel, sin_kernel.
+// muladd_kernel, sin_kernel, and one kernel per unary / binary / narrowing
+// operation that the reference's compute lowering accepts
+// (npu/lib/Dialect/TritonTenstorrent/Transforms/ConvertComputeOps.cpp:162-182).
 //
 // Each follows the masked-block semantics of the example kernel sources
 // (python/tutorials/01-vector-add.py:29-54, 01-vector-mul-add.py:30-57,
@@ -118,9 +120,63 @@ __device__ __forceinline__ float sin_any(float x) {
   return ax < 2.44140625e-4f ? x : v;
 }
 
-template <int UNROLL>
-__device__ __forceinline__ void sin_body(const float *__restrict__ x, float *__restrict__ out,
-                                         uint32_t n) {
+// ---- cos: the same reduction as sin_fast, one quadrant on ----------------------
+__device__ __forceinline__ float cos_fast(float x) {
+  const float two_over_pi = 0.636619772367581343f;
+  const float p1 = 1.5707963705062866f, p2 = -4.371138828673793e-08f, p3 = -1.7151245100058819e-15f;
+  float kf = __builtin_rintf(x * two_over_pi);
+  float r = __builtin_fmaf(-kf, p1, x);
+  r = __builtin_fmaf(-kf, p2, r);
+  r = __builtin_fmaf(-kf, p3, r);
+  int q = (int)kf + 1; // cos(x) = sin(x + pi/2)
+  float r2 = r * r;
+  float s = __builtin_fmaf(r2, 2.7183114939898219064e-06f, -1.98393348360966317347e-04f);
+  s = __builtin_fmaf(s, r2, 8.3333293858894631756e-03f);
+  s = __builtin_fmaf(s, r2, -1.66666666416265235595e-01f);
+  s = __builtin_fmaf(s * r2, r, r);
+  float c = __builtin_fmaf(r2, 2.43904487962774090654e-05f, -1.38867637746099294692e-03f);
+  c = __builtin_fmaf(c, r2, 4.16666233237390631894e-02f);
+  c = __builtin_fmaf(c, r2, -4.99999997251031003120e-01f);
+  c = __builtin_fmaf(c, r2, 1.0f);
+  float v = (q & 1) ? c : s;
+  return (q & 2) ? -v : v;
+}
+
+// IEEE-754-2019 maximum / minimum (arith.maximumf / minimumf): NaN if either is NaN, -0 < +0
+__device__ __forceinline__ float ieee_maximum(float a, float b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == b) return __builtin_signbit(a) ? b : a;
+  return a > b ? a : b;
+}
+__device__ __forceinline__ float ieee_minimum(float a, float b) {
+  if (a != a) return a;
+  if (b != b) return b;
+  if (a == b) return __builtin_signbit(a) ? a : b;
+  return a < b ? a : b;
+}
+
+struct SinOp { __device__ static float apply(float x) { return sin_any(x); } };
+struct CosOp {
+  __device__ static float apply(float x) { return __builtin_fabsf(x) < 131072.0f ? cos_fast(x) : cosf(x); }
+};
+struct AbsOp { __device__ static float apply(float x) { return __builtin_fabsf(x); } };
+struct CeilOp { __device__ static float apply(float x) { return __builtin_ceilf(x); } };
+struct FloorOp { __device__ static float apply(float x) { return __builtin_floorf(x); } };
+struct ExpOp { __device__ static float apply(float x) { return expf(x); } };
+struct Exp2Op { __device__ static float apply(float x) { return exp2f(x); } };
+struct LogOp { __device__ static float apply(float x) { return logf(x); } };
+struct Log2Op { __device__ static float apply(float x) { return log2f(x); } };
+struct RsqrtOp { __device__ static float apply(float x) { return rsqrtf(x); } };
+struct SqrtOp { __device__ static float apply(float x) { return sqrtf(x); } };   // correctly rounded
+struct SubOp { __device__ static float apply(float a, float b) { return a - b; } };
+struct MulOp { __device__ static float apply(float a, float b) { return a * b; } };
+struct DivOp { __device__ static float apply(float a, float b) { return a / b; } }; // correctly rounded
+struct MaxOp { __device__ static float apply(float a, float b) { return ieee_maximum(a, b); } };
+struct MinOp { __device__ static float apply(float a, float b) { return ieee_minimum(a, b); } };
+
+template <typename Op, int UNROLL>
+__device__ __forceinline__ void unary_body(const float *__restrict__ x, float *__restrict__ out, uint32_t n) {
   using V = Vec4<float>::type;
   const uint32_t nvec = n >> 2;
   const V *xv = reinterpret_cast<const V *>(x);
@@ -134,10 +190,10 @@ __device__ __forceinline__ void sin_body(const float *__restrict__ x, float *__r
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       V r;
-      r.x = sin_any(a[u].x);
-      r.y = sin_any(a[u].y);
-      r.z = sin_any(a[u].z);
-      r.w = sin_any(a[u].w);
+      r.x = Op::apply(a[u].x);
+      r.y = Op::apply(a[u].y);
+      r.z = Op::apply(a[u].z);
+      r.w = Op::apply(a[u].w);
       __builtin_nontemporal_store(r, ov + i + u * kThreads);
     }
   } else {
@@ -146,16 +202,44 @@ __device__ __forceinline__ void sin_body(const float *__restrict__ x, float *__r
       const uint32_t j = i + u * kThreads;
       if (j < nvec) {
         V a = xv[j], r;
-        r.x = sin_any(a.x);
-        r.y = sin_any(a.y);
-        r.z = sin_any(a.z);
-        r.w = sin_any(a.w);
+        r.x = Op::apply(a.x);
+        r.y = Op::apply(a.y);
+        r.z = Op::apply(a.z);
+        r.w = Op::apply(a.w);
         ov[j] = r;
       }
     }
     const uint32_t t = (nvec << 2) + threadIdx.x;
-    if (t < n) out[t] = sin_any(x[t]);
+    if (t < n) out[t] = Op::apply(x[t]);
   }
+}
+template <typename Op> __device__ __forceinline__ void unary_scalar_body(const float *x, float *out, uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = Op::apply(x[i]);
+}
+
+// ---- narrowing conversions (arith.truncf, arith.trunci) ---------------------------
+// One element per lane and pass, grid-stride: 4-byte loads and 1- or 2-byte stores coalesce per
+// wavefront; these are conversions at the edge of a pipeline, not streaming hot spots.
+struct ToBf16 {
+  typedef float in_t; typedef uint16_t out_t;
+  __device__ static uint16_t apply(float f) { // round to nearest even, NaN kept quiet
+    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+  }
+};
+struct ToF16 {
+  typedef float in_t; typedef uint16_t out_t;
+  __device__ static uint16_t apply(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+};
+struct ToI16 { typedef int in_t; typedef int16_t out_t; __device__ static int16_t apply(int v) { return (int16_t)v; } };
+struct ToI8 { typedef int in_t; typedef int8_t out_t; __device__ static int8_t apply(int v) { return (int8_t)v; } };
+template <typename Op>
+__device__ __forceinline__ void cast_body(const typename Op::in_t *x, typename Op::out_t *out, uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = Op::apply(x[i]);
 }
 
 struct MulAdd {
@@ -185,13 +269,52 @@ __global__ __launch_bounds__(kThreads) void ew_add_i32_unaligned(const int *x, c
   binary_scalar_body<int, AddWrapOp>(x, y, out, n);
 }
 
-__global__ __launch_bounds__(kThreads) void ew_sin_f32(const float *x, float *out, uint32_t n) {
-  sin_body<4>(x, out, n);
+#define EW_UNARY(name, Op)                                                                              \
+  __global__ __launch_bounds__(kThreads) void ew_##name##_f32(const float *x, float *out, uint32_t n) { \
+    unary_body<Op, 4>(x, out, n);                                                                        \
+  }                                                                                                      \
+  __global__ __launch_bounds__(kThreads) void ew_##name##_f32_unaligned(const float *x, float *out,     \
+                                                                        uint32_t n) {                    \
+    unary_scalar_body<Op>(x, out, n);                                                                    \
+  }
+EW_UNARY(sin, SinOp)
+EW_UNARY(cos, CosOp)
+EW_UNARY(abs, AbsOp)
+EW_UNARY(ceil, CeilOp)
+EW_UNARY(floor, FloorOp)
+EW_UNARY(exp, ExpOp)
+EW_UNARY(exp2, Exp2Op)
+EW_UNARY(log, LogOp)
+EW_UNARY(log2, Log2Op)
+EW_UNARY(rsqrt, RsqrtOp)
+EW_UNARY(sqrt, SqrtOp)
+
+#define EW_BINARY(name, Op)                                                                               \
+  __global__ __launch_bounds__(kThreads) void ew_##name##_f32(const float *x, const float *y, float *out, \
+                                                              uint32_t n) {                                \
+    binary_body<float, Op, 4>(x, y, out, n);                                                               \
+  }                                                                                                        \
+  __global__ __launch_bounds__(kThreads) void ew_##name##_f32_unaligned(const float *x, const float *y,   \
+                                                                        float *out, uint32_t n) {          \
+    binary_scalar_body<float, Op>(x, y, out, n);                                                           \
+  }
+EW_BINARY(sub, SubOp)
+EW_BINARY(mul, MulOp)
+EW_BINARY(div, DivOp)
+EW_BINARY(max, MaxOp)
+EW_BINARY(min, MinOp)
+
+__global__ __launch_bounds__(kThreads) void ew_cast_f32_bf16(const float *x, uint16_t *out, uint32_t n) {
+  cast_body<ToBf16>(x, out, n);
 }
-__global__ __launch_bounds__(kThreads) void ew_sin_f32_unaligned(const float *x, float *out,
-                                                                 uint32_t n) {
-  const uint32_t stride = gridDim.x * kThreads;
-  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = sin_any(x[i]);
+__global__ __launch_bounds__(kThreads) void ew_cast_f32_f16(const float *x, uint16_t *out, uint32_t n) {
+  cast_body<ToF16>(x, out, n);
+}
+__global__ __launch_bounds__(kThreads) void ew_cast_i32_i16(const int *x, int16_t *out, uint32_t n) {
+  cast_body<ToI16>(x, out, n);
+}
+__global__ __launch_bounds__(kThreads) void ew_cast_i32_i8(const int *x, int8_t *out, uint32_t n) {
+  cast_body<ToI8>(x, out, n);
 }
 
 __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restrict__ x,

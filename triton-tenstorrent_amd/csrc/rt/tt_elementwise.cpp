@@ -1,6 +1,7 @@
 // tt_add_kernel / tt_add_kernel_loop / tt_muladd_kernel / tt_sin_kernel:
 // launch validation and binding to the streaming kernels of elementwise.hip.
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <map>
 #include <mutex>
@@ -121,6 +122,63 @@ int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SI
   void *args[] = {&x, &out, &n_eff};
   return launch("elementwise", al ? "ew_sin_f32" : "ew_sin_f32_unaligned",
                 dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 3);
+}
+
+int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
+                    const uint32_t grid[3], void *stream) {
+  static const char *const names[] = {"abs", "ceil", "cos", "exp", "exp2", "floor", "log", "log2", "rsqrt", "sin", "sqrt"};
+  if (!props()) return fail(RT_ERR_NOT_INIT, "unary_kernel: call rt_init first");
+  if (op < 0 || op >= (int)(sizeof(names) / sizeof(names[0])))
+    return fail(RT_ERR_UNSUPPORTED, "unary_kernel: op %d (tt_unary_op has 0..10)", op);
+  uint32_t n_eff = 0;
+  int rc = check_1d("unary_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !out) return fail(RT_ERR_INVALID, "unary_kernel: null tensor pointer");
+  bool al = aligned16(x) && aligned16(out);
+  char name[48];
+  snprintf(name, sizeof(name), "ew_%s_f32%s", names[op], al ? "" : "_unaligned");
+  void *args[] = {&x, &out, &n_eff};
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 3);
+}
+
+int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_t n_elements,
+                     int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream) {
+  static const char *const names[] = {"add", "sub", "mul", "div", "max", "min"};
+  if (!props()) return fail(RT_ERR_NOT_INIT, "binary_kernel: call rt_init first");
+  if (op < 0 || op >= (int)(sizeof(names) / sizeof(names[0])))
+    return fail(RT_ERR_UNSUPPORTED, "binary_kernel: op %d (tt_binary_op has 0..5)", op);
+  uint32_t n_eff = 0;
+  int rc = check_1d("binary_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !y || !out) return fail(RT_ERR_INVALID, "binary_kernel: null tensor pointer");
+  bool al = aligned16(x) && aligned16(y) && aligned16(out);
+  char name[48];
+  snprintf(name, sizeof(name), "ew_%s_f32%s", names[op], al ? "" : "_unaligned");
+  void *args[] = {&x, &y, &out, &n_eff};
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 4);
+}
+
+int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE, int32_t in_dtype,
+                   int32_t out_dtype, const uint32_t grid[3], void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "cast_kernel: call rt_init first");
+  const char *name = nullptr;
+  if (in_dtype == TT_F32 && out_dtype == TT_BF16) name = "ew_cast_f32_bf16";
+  else if (in_dtype == TT_F32 && out_dtype == TT_F16) name = "ew_cast_f32_f16";
+  else if (in_dtype == TT_I32 && out_dtype == TT_I16) name = "ew_cast_i32_i16";
+  else if (in_dtype == TT_I32 && out_dtype == TT_I8) name = "ew_cast_i32_i8";
+  else
+    return fail(RT_ERR_UNSUPPORTED, "cast_kernel: dtype %d -> %d (fp32 -> bf16/fp16 and int32 -> int16/int8 exist)",
+                in_dtype, out_dtype);
+  uint32_t n_eff = 0;
+  int rc = check_1d("cast_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !out) return fail(RT_ERR_INVALID, "cast_kernel: null tensor pointer");
+  if (reinterpret_cast<uintptr_t>(x) & 3) return fail(RT_ERR_INVALID, "cast_kernel: x must be 4-byte aligned");
+  void *args[] = {&x, &out, &n_eff};
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, false)), dim3(kThreads), 0, stream, args, 3);
 }
 
 } // extern "C"

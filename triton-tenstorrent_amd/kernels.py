@@ -29,6 +29,37 @@ muladd_kernel = PrebuiltKernel("muladd_kernel", ["x_ptr", "y_ptr", "z_ptr", "out
                                ["BLOCK_SIZE"])
 sin_kernel = PrebuiltKernel("sin_kernel", ["x_ptr", "output_ptr", "n_elements", "BLOCK_SIZE"], ["BLOCK_SIZE"])
 
+# the rest of the operation set the reference's compute lowering accepts (ConvertComputeOps.cpp:162-182),
+# in the same masked-block form; OP is the operation's mnemonic ("exp", "maximum", ...)
+unary_kernel = PrebuiltKernel("unary_kernel", ["x_ptr", "output_ptr", "n_elements", "BLOCK_SIZE", "OP"], ["BLOCK_SIZE", "OP"])
+binary_kernel = PrebuiltKernel("binary_kernel", ["x_ptr", "y_ptr", "output_ptr", "n_elements", "BLOCK_SIZE", "OP"],
+                               ["BLOCK_SIZE", "OP"])
+cast_kernel = PrebuiltKernel("cast_kernel", ["x_ptr", "output_ptr", "n_elements", "BLOCK_SIZE"], ["BLOCK_SIZE"])
+
+
+def unary(op: str, x: torch.Tensor) -> torch.Tensor:
+    """``op`` in abs, ceil, cos, exp, exp2, floor, log, log2, rsqrt, sin, sqrt; fp32."""
+    out = torch.empty_like(x)
+    n = out.numel()
+    unary_kernel[lambda meta: (cdiv(n, meta["BLOCK_SIZE"]), )](x, out, n, BLOCK_SIZE=1024, OP=op)
+    return out
+
+
+def binary(op: str, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """``op`` in add, sub, mul, div, maximum, minimum; fp32."""
+    out = torch.empty_like(x)
+    n = out.numel()
+    binary_kernel[lambda meta: (cdiv(n, meta["BLOCK_SIZE"]), )](x, y, out, n, BLOCK_SIZE=1024, OP=op)
+    return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """fp32 -> bf16 / fp16 (round to nearest even) or int32 -> int16 / int8 (low bits kept)."""
+    out = torch.empty(x.shape, device=x.device, dtype=dtype)
+    n = out.numel()
+    cast_kernel[lambda meta: (cdiv(n, meta["BLOCK_SIZE"]), )](x, out, n, BLOCK_SIZE=1024)
+    return out
+
 
 def add(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
     output = torch.empty_like(x)

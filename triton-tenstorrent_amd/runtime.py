@@ -13,7 +13,11 @@ PKG = Path(__file__).resolve().parent
 LIB_PATH = PKG / "lib" / "libttamd_rt.so"
 
 RT_OK, RT_ERR_INVALID, RT_ERR_HIP, RT_ERR_NOT_FOUND, RT_ERR_UNSUPPORTED, RT_ERR_NOT_INIT = 0, -1, -2, -3, -4, -5
-TT_F32, TT_I32, TT_BF16, TT_F16, TT_FP8E4M3 = 0, 1, 2, 3, 4
+TT_F32, TT_I32, TT_BF16, TT_F16, TT_FP8E4M3, TT_I16, TT_I8 = 0, 1, 2, 3, 4, 5, 6
+# tt_unary_op / tt_binary_op of the header, by the name of the MLIR operation's mnemonic
+UNARY_OPS = {"abs": 0, "ceil": 1, "cos": 2, "exp": 3, "exp2": 4, "floor": 5, "log": 6, "log2": 7, "rsqrt": 8, "sin": 9,
+             "sqrt": 10}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
 TT_EPI_NONE, TT_EPI_BIAS_FULL, TT_EPI_BIAS_ROW_GELU, TT_EPI_LEAKY_RELU, TT_EPI_BIAS_ROW = 0, 1, 2, 3, 4
 
 # Triton pointer type strings -> tt_dtype
@@ -79,6 +83,9 @@ SYMBOLS = {
     "tt_add_kernel_loop": (C.c_int, [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_muladd_kernel": (C.c_int, [_vp, _vp, _vp, _vp, _i32, _i32, _G, _vp]),
     "tt_sin_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _G, _vp]),
+    "tt_unary_kernel": (C.c_int, [_i32, _vp, _vp, _i32, _i32, _G, _vp]),
+    "tt_binary_kernel": (C.c_int, [_i32, _vp, _vp, _vp, _i32, _i32, _G, _vp]),
+    "tt_cast_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_fused": (C.c_int, [_DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma_fp8_scaled": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _f32, _f32, _i32, _i32, _i32, _i32, _G, _vp]),
