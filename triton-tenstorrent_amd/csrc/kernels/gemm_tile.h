@@ -155,9 +155,6 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // The 12 LDS reads of one sub-step, in the order the MFMAs will want them:
   // b0.lo b0.hi a0 b1.lo b1.hi b2.lo b2.hi b3.lo b3.hi a1 a2 a3
   auto rd = [&](Frags &f, const uint8_t *stage, int s, int r) {
-#ifdef EXP_NO_LDSREAD
-    if (g.K > 0) return;
-#endif
     switch (r) {
     case 2: f.a[0] = *(const vec *)(stage + a_pos[s]); break;
     case 9: f.a[1] = *(const vec *)(stage + a_pos[s] + 2048); break;
@@ -183,9 +180,6 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // hand instead: copies retire in issue order, and each step's barrier waits with
   // s_waitcnt vmcnt(n) for exactly the copies that the following reads depend on.
   auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
-#ifdef EXP_NO_DMA
-    if (g.K > 0) return;
-#endif
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
@@ -200,12 +194,6 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp) {
     int tm, tn;
     tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
-#ifdef EXP_SAME_TILE
-    tm = tn = 0;
-#endif
-#ifdef EXP_XCD_TILE
-    tm = blockIdx.x % 8; tn = 0;
-#endif
     ap = A + (TILED ? (int64_t)tm * (BM / 32) * ntk * 2048 : (int64_t)tm * BM * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
   };
@@ -214,12 +202,6 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   auto dma_single = [&](int kk, uint8_t *stage, int i) {
     const bool over = kk >= nk;
     const int k = over ? kk - nk : kk;
-#ifdef EXP_ONLY_A
-    if (i >= 4 && g.K > 0) return;
-#endif
-#ifdef EXP_ONLY_B
-    if (i < 4 && g.K > 0) return;
-#endif
     if (i < 4) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
