@@ -52,13 +52,20 @@ def _typestr_dtype(ty: str) -> int:
     return rt.DTYPE_OF_TYPESTR[t]
 
 
+_DTYPE_CODES: dict | None = None
+
+
 def _torch_dtype_code(t) -> int:
-    import torch
-    table = {torch.float32: rt.TT_F32, torch.int32: rt.TT_I32, torch.bfloat16: rt.TT_BF16,
-             torch.float16: rt.TT_F16, torch.float8_e4m3fn: rt.TT_FP8E4M3, torch.int16: rt.TT_I16, torch.int8: rt.TT_I8}
-    if t.dtype not in table:
+    global _DTYPE_CODES
+    if _DTYPE_CODES is None:
+        import torch
+        _DTYPE_CODES = {torch.float32: rt.TT_F32, torch.int32: rt.TT_I32, torch.bfloat16: rt.TT_BF16,
+                        torch.float16: rt.TT_F16, torch.float8_e4m3fn: rt.TT_FP8E4M3, torch.int16: rt.TT_I16,
+                        torch.int8: rt.TT_I8}
+    code = _DTYPE_CODES.get(t.dtype)
+    if code is None:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"tensor dtype {t.dtype} has no kernel")
-    return table[t.dtype]
+    return code
 
 
 def flatten_launch_args(sig_types: list[str], args: tuple, ranks_out: list | None = None) -> list:
@@ -385,25 +392,26 @@ class TTLauncher:
         self.signature = {idx: value for idx, value in src.signature.items()}
         self.arg_names = arg_names
         self.keepalive: list = []
+        # fixed per (kernel, specialisation): computed once, used on every launch
+        self._sig_types = list(self.signature.values())
+        self._constexpr_pos = [(i, n) for i, (n, ty) in enumerate(zip(arg_names, self._sig_types)) if ty == "constexpr"]
+        self._folded = [(arg_names[idx[0]], val) for idx, val in self.constants.items()
+                        if len(idx) == 1 and idx[0] < len(arg_names)]
 
     def __call__(self, gridX, gridY, gridZ, stream, function, *args):
         kernel_metadata, launch_metadata, launch_enter_hook, launch_exit_hook = args[0], args[1], args[2], args[3]
         del kernel_metadata  # num_warps / shared describe Triton codegen; the prebuilt kernels fix their own
         user_args = args[4:]
-        sig_types = list(self.signature.values())
+        sig_types = self._sig_types
         if len(user_args) != len(sig_types):
             raise rt.InvalidLaunch(rt.RT_ERR_INVALID,
                                    f"{function.name}: {len(user_args)} arguments for a {len(sig_types)}-entry signature")
         ranks: list = []
         flat = flatten_launch_args(sig_types, user_args, ranks)
         # constexprs by name: explicit constexpr parameters plus ints Triton specialised away (value 1)
-        consts = {}
-        for name, ty, val in zip(self.arg_names, sig_types, user_args):
-            if ty == "constexpr":
-                consts[name] = val
-        for idx, val in self.constants.items():
-            if len(idx) == 1 and idx[0] < len(self.arg_names):
-                consts.setdefault(self.arg_names[idx[0]], val)
+        consts = {name: user_args[i] for i, name in self._constexpr_pos}
+        for name, val in self._folded:
+            consts.setdefault(name, val)
         keep: list = []
         cur = _Cursor(flat, keep, ranks, consts, self.arg_names)
         lib = rt.init(0)

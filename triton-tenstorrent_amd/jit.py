@@ -37,6 +37,10 @@ def specialize(arg: Any, is_constexpr: bool) -> str:
     """Type string of one bound argument, as Triton's specializer writes it."""
     if is_constexpr or arg is None:
         return "constexpr"
+    if type(arg) is int:  # the common scalar, ahead of the duck-typed checks
+        if arg == 1:
+            return "constexpr"  # Triton folds the value 1 into the specialisation
+        return "i32" if -2**31 <= arg < 2**31 else "i64"
     if is_tensor_descriptor(arg):
         block = ",".join(str(int(b)) for b in arg.block_shape)
         return f"tensordesc<{_typestr_of_torch(arg.base.dtype)}[{block}]>"

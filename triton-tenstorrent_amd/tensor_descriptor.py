@@ -47,4 +47,8 @@ class TensorDescriptor:
 
 def is_tensor_descriptor(obj: Any) -> bool:
     """Duck-typed check accepting this class and Triton's."""
-    return all(hasattr(obj, a) for a in ("base", "shape", "strides", "block_shape", "padding"))
+    if type(obj) is TensorDescriptor:
+        return True
+    # block_shape first: tensors and scalars do not have it, so the common case is one lookup
+    return (hasattr(obj, "block_shape") and hasattr(obj, "base") and hasattr(obj, "shape") and hasattr(obj, "strides")
+            and hasattr(obj, "padding"))
