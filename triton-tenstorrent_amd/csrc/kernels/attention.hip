@@ -300,6 +300,11 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
 #pragma unroll
     for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+    // Make the loads land here.  Otherwise the compiler defers its s_waitcnt vmcnt(n) for them into
+    // the key loop, where n is wrong by the copies issued from assembly, which it cannot count: the
+    // wait then sits behind every block's freshly issued copies and serialises their whole latency.
+#pragma unroll
+    for (int s = 0; s < DK; ++s) asm volatile("" : "+v"(qf[s].v));
   }
   f32x16 acc[DT];
 #pragma unroll
