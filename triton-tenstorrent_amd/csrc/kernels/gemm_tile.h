@@ -293,6 +293,17 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
     //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
     const int64_t m = m0 + wm * 128 + l32;
+    // A row bias depends on n only: its 64 values for this lane are fetched once, all loads in flight
+    // together, instead of one dependent load per use in the loop below.
+    constexpr bool ROW_BIAS = EPI == EPI_BIAS_ROW || EPI == EPI_BIAS_ROW_GELU;
+    f32x4 brow[ROW_BIAS ? 4 : 1][ROW_BIAS ? 4 : 1];
+    if constexpr (ROW_BIAS) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+          brow[j][r4] = *(const f32x4 *)((const float *)g.bias + n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4);
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int64_t mi = m + i * 32;
@@ -303,7 +314,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
           float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = apply_epilogue_ct<OUT_DT, EPI>(g, acc[i][j][r4 * 4 + e] * g.scale, mi, n + e);
+          for (int e = 0; e < 4; ++e) {
+            const float x = acc[i][j][r4 * 4 + e] * g.scale;
+            if constexpr (EPI == EPI_BIAS_ROW_GELU)
+              v[e] = gelu_erf(x + brow[j][r4][e]);
+            else if constexpr (EPI == EPI_BIAS_ROW)
+              v[e] = x + brow[j][r4][e];
+            else
+              v[e] = apply_epilogue_ct<OUT_DT, EPI>(g, x, mi, n + e);
+          }
           u32x2 pk;
           if constexpr (OUT_DT == DT_BF16) {
             pk = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
