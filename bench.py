@@ -190,6 +190,21 @@ def main() -> int:
         avg_ms, per, wall = _events_time(lambda: K.add_kernel[(97, )](x0, y0, o0, n0, BLOCK_SIZE=1024), 200, 20, stream)
         extra["add_f32_98432"] = {"us_avg": round(avg_ms * 1e3, 2), "us_min": round(min(per) * 1e3, 2),
                                   "host_us_per_launch": round(wall * 1e3, 2), "GBs": round(3 * 4 * n0 / (avg_ms * 1e-3) / 1e9, 1)}
+        # the same launch recorded 100 times into a HIP graph: what is left when the host is out of the loop
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for _ in range(100):
+                K.add_kernel[(97, )](x0, y0, o0, n0, BLOCK_SIZE=1024)
+        gr.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            gr.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        extra["add_f32_98432"]["us_per_launch_in_hip_graph"] = round(e0.elapsed_time(e1) * 1e3 / 1000, 2)
+        del gr
 
     # ---------------- fused epilogue: GELU(A.B + bias) ----------------------
     if want("fused"):

@@ -1,0 +1,70 @@
+"""Launches are plain hipModuleLaunchKernel calls on the caller's stream with no allocation, memset or
+synchronisation inside, so a caller can record them into a HIP graph.  Each graph is replayed several times
+with eager work and synchronisations in between, and every replay is checked against the eager result."""
+import numpy as np
+import pytest
+import torch
+
+from triton_tenstorrent_amd import kernels as K
+from triton_tenstorrent_amd import runtime as rt
+
+pytestmark = pytest.mark.gpu
+
+
+def _capture(fn):
+    fn()                                    # warm-up outside the graph: library and code objects are loaded here
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return g
+
+
+def test_elementwise_chain_in_a_graph():
+    n = 98432
+    x, y = torch.rand(n, device="cuda"), torch.rand(n, device="cuda")
+    t, out = torch.empty_like(x), torch.empty_like(x)
+    grid = (K.cdiv(n, 1024), )
+
+    def chain():
+        K.add_kernel[grid](x, y, t, n, BLOCK_SIZE=1024)
+        K.sin_kernel[grid](t, out, n, BLOCK_SIZE=1024)
+        K.binary_kernel[grid](out, x, t, n, BLOCK_SIZE=1024, OP="mul")
+
+    g = _capture(chain)
+    for rep in range(4):
+        x.copy_(torch.rand(n, device="cuda"))          # eager work between replays, new inputs each time
+        torch.cuda.synchronize()
+        t.fill_(-1.0)
+        out.fill_(-1.0)
+        g.replay()
+        torch.cuda.synchronize()
+        want_out = K.sin(x + y)
+        assert torch.equal(out, want_out) and torch.equal(t, want_out * x), rep
+
+
+def test_matmul_and_attention_in_a_graph():
+    M = N = Kd = 512
+    a = (torch.randn(M, Kd, device="cuda") / 16).to(torch.bfloat16)
+    b = torch.randn(Kd, N, device="cuda").to(torch.bfloat16)
+    bias = torch.randn(N, device="cuda") * 0.02
+    q, k, v = (torch.randn(1, 2, 512, 128, device="cuda").to(torch.bfloat16) for _ in range(3))
+    res = {}
+
+    def work():
+        res["c"] = K.matmul_fused(a, b, bias, epilogue="gelu")
+        res["o"] = K.attention(q, k, v, True, 128 ** -0.5)
+
+    eager = {}
+    work()
+    torch.cuda.synchronize()
+    eager["c"], eager["o"] = res["c"].clone(), res["o"].clone()
+    g = _capture(work)                      # outputs are allocated by torch inside the capture: graph-private memory
+    for rep in range(3):
+        res["c"].zero_()
+        res["o"].zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert rt.last_kernel_name() is not None
+        assert torch.equal(res["c"], eager["c"]) and torch.equal(res["o"], eager["o"]), rep
