@@ -334,6 +334,16 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
         st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[s].v, st[kt], 0, 0, 0);
       }
     }
+    // Order for the scheduler: fragment reads run four MFMAs ahead of their use (left to itself it puts a
+    // read right in front of the MFMA that needs it, and half of the MFMAs then wait out the LDS latency).
+    constexpr int AHEAD = 4;
+    __builtin_amdgcn_sched_group_barrier(0x100, AHEAD, 0);
+#pragma unroll
+    for (int i = 0; i < 2 * DK - AHEAD; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
     // ---- online softmax (per lane = per query; keys run over registers and the hi half) ----
     const bool on_band = a.causal && (n0 + BN - 1 > qw);
     float rmax = -__builtin_inff();
@@ -409,6 +419,14 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
         acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[k4].v, acc[t], 0, 0, 0);
       }
     }
+    // the same for P.V: two transposing reads per fragment
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 1);
+#pragma unroll
+    for (int i = 0; i < 4 * DT - AHEAD; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 1);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // ---- epilogue ----
