@@ -149,7 +149,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   int t = blockIdx.x;
   if (t >= total) return;
   tile_bases(t, a_cur, b_cur);
-  tile_bases(t + gridDim.x < total ? t + gridDim.x : t, a_nxt, b_nxt);
+  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt);
   // fill the ring with steps 0..R-1
 #pragma unroll
   for (int s = 0; s < R; ++s)
