@@ -9,6 +9,7 @@ import torch
 
 triton = pytest.importorskip("triton")
 
+import triton.language as tl  # noqa: E402
 from triton.backends.compiler import GPUTarget  # noqa: E402
 
 from triton_tenstorrent_amd.backend import compiler as ttc  # noqa: E402
@@ -133,3 +134,96 @@ def test_triton_jit_launches_prebuilt_kernels(tmp_path, monkeypatch):
         from triton.backends import backends
         backends.pop("tenstorrent", None)
         triton.runtime.driver._active = None  # back to the stock driver, lazily
+
+
+# ---- kernels bound by the shape of their IR ---------------------------------------------------------
+@triton.jit
+def user_exp2(src_ptr, dst_ptr, count, BLOCK_SIZE: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offsets = pid * BLOCK_SIZE + tl.arange(0, BLOCK_SIZE)
+    mask = offsets < count
+    tl.store(dst_ptr + offsets, tl.exp2(tl.load(src_ptr + offsets, mask=mask)), mask=mask)
+
+
+@triton.jit
+def user_sub_swapped(out_ptr, a_ptr, b_ptr, n, BLOCK: tl.constexpr):
+    # output first, and the second tensor is the minuend: operand order must come from the IR, not the signature
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(out_ptr + offs, tl.load(b_ptr + offs, mask=m) - tl.load(a_ptr + offs, mask=m), mask=m)
+
+
+@triton.jit
+def user_to_bf16(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(y_ptr + offs, tl.load(x_ptr + offs, mask=m).to(tl.bfloat16), mask=m)
+
+
+@triton.jit
+def user_two_ops(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(y_ptr + offs, tl.exp(tl.sqrt(tl.load(x_ptr + offs, mask=m))), mask=m)
+
+
+@triton.jit
+def user_strided(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(y_ptr + offs, tl.exp(tl.load(x_ptr + 2 * offs, mask=m)), mask=m)
+
+
+def test_elementwise_kernels_are_recognised_by_shape(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    f32 = "*fp32"
+    k = _compile(user_exp2, {"src_ptr": f32, "dst_ptr": f32, "count": "i32", "BLOCK_SIZE": "constexpr"}, {"BLOCK_SIZE": 512})
+    rec = json.loads(k.kernel)
+    assert k.name == "user_exp2" and rec["kernel"] == "unary_kernel"
+    assert rec["match"] == {"kernel": "unary_kernel", "op": "exp2", "inputs": ["src_ptr"], "output": "dst_ptr",
+                            "n": "count", "n_const": None, "block": 512}
+    k = _compile(user_sub_swapped, {"out_ptr": f32, "a_ptr": f32, "b_ptr": f32, "n": "i32", "BLOCK": "constexpr"},
+                 {"BLOCK": 1024})
+    m = json.loads(k.kernel)["match"]
+    assert (m["kernel"], m["op"], m["inputs"], m["output"]) == ("binary_kernel", "sub", ["b_ptr", "a_ptr"], "out_ptr")
+    k = _compile(user_to_bf16, {"x_ptr": f32, "y_ptr": "*bf16", "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 1024})
+    assert json.loads(k.kernel)["match"]["kernel"] == "cast_kernel"
+    # not of the form: two operations, or addressing other than base + offsets
+    for fn in (user_two_ops, user_strided):
+        with pytest.raises(Exception, match="no prebuilt gfx950 implementation"):
+            _compile(fn, {"x_ptr": f32, "y_ptr": f32, "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 1024})
+    # wrong element type for the operation set
+    with pytest.raises(Exception, match="no prebuilt gfx950 implementation"):
+        _compile(user_sub_swapped, {"out_ptr": "*fp16", "a_ptr": "*fp16", "b_ptr": "*fp16", "n": "i32",
+                                    "BLOCK": "constexpr"}, {"BLOCK": 1024})
+
+
+@pytest.mark.gpu
+def test_shape_matched_kernels_run(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from oracle import oracle as orc
+    from triton_tenstorrent_amd import runtime as rt
+    ttc.register()
+    try:
+        n = 70001
+        a = torch.randn(n, device="cuda") * 3
+        b = torch.randn(n, device="cuda")
+        out = torch.full((n + 5, ), -7.0, device="cuda")
+        user_exp2[(triton.cdiv(n, 512), )](a, out, n, BLOCK_SIZE=512)
+        assert rt.last_kernel_name() == "ew_exp2_f32"
+        want = orc.unary("exp2", a.cpu().numpy())
+        got = out[:n].cpu().numpy()
+        assert np.all(np.abs(got.astype(np.float64) - want) <= 2 * np.spacing(np.abs(want))) and torch.all(out[n:] == -7.0)
+        user_sub_swapped[(triton.cdiv(n, 1024), )](out, a, b, n, BLOCK=1024)
+        assert torch.equal(out[:n], b - a)
+        h = torch.empty(n, device="cuda", dtype=torch.bfloat16)
+        user_to_bf16[(triton.cdiv(n, 1024), )](a, h, n, BLOCK=1024)
+        assert rt.last_kernel_name() == "ew_cast_f32_bf16" and torch.equal(h, a.to(torch.bfloat16))
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None

@@ -20,6 +20,7 @@ from types import ModuleType
 from typing import Dict, Tuple
 
 from .driver import BINARY_EXT, KERNEL_TABLE, GPUTarget, TTDriver
+from .patterns import match_streaming
 
 try:
     from triton.backends.compiler import BaseBackend, Language
@@ -154,14 +155,22 @@ class TTBackend(BaseBackend):
     def make_binary(src, metadata, options):
         """Final stage: bind the kernel by NAME to the prebuilt table and return the
         record the launcher loads.  No device code is generated."""
-        name = TTBackend.kernel_name_of(str(src))
+        text = str(src)
+        name = TTBackend.kernel_name_of(text)
+        record = {"kernel": name, "ext": BINARY_EXT, "arch": options.arch}
         if name not in KERNEL_TABLE:
-            raise RuntimeError(f"kernel '{name}' has no prebuilt gfx950 implementation; this backend runs "
-                               f"{sorted(KERNEL_TABLE)} and does no code generation")
+            # not one of the example kernels by name: a kernel of the masked-block elementwise form is
+            # bound by what its IR says it does (one operation of the reference's opcode set)
+            match = match_streaming(text)
+            if match is None:
+                raise RuntimeError(f"kernel '{name}' has no prebuilt gfx950 implementation; this backend runs "
+                                   f"{sorted(KERNEL_TABLE)}, and elementwise kernels of the masked-block form with "
+                                   f"one supported operation; it does no code generation")
+            record.update(kernel=match["kernel"], match=match)
         metadata["name"] = name
         metadata["shared"] = 0
         metadata["warp_size"] = 64
-        return json.dumps({"kernel": name, "ext": BINARY_EXT, "arch": options.arch}).encode()
+        return json.dumps(record).encode()
 
     def add_stages(self, stages, options, language=None):
         if language is not None and language == getattr(Language, "GLUON", object()):

@@ -9,6 +9,7 @@ kernel NAME to the matching ``tt_*`` entry point of the C ABI.
 from __future__ import annotations
 
 import ctypes as C
+import functools
 import json
 import time
 from typing import Any, Callable
@@ -126,6 +127,14 @@ class _Cursor:
 
     def has(self, name: str) -> bool:
         return name in self.arg_names
+
+    def named(self) -> dict:
+        """Every parameter by name: constexprs from the constants, the rest from the launch list in order
+        (no descriptors: used for the pointer-and-scalar kernels matched by shape)."""
+        out = {}
+        for name in self.arg_names:
+            out[name] = self.consts[name] if name in self.consts else self._next()
+        return out
 
     def desc(self) -> rt.tt_desc2d:
         rank = self.ranks.pop(0) if self.ranks else 2
@@ -325,6 +334,28 @@ def _bind_attn_fwd(lib, cur, consts, grid, stream):
                            int(consts["STAGE"]), grid, stream)
 
 
+def _bind_matched(match: dict, lib, cur, consts, grid, stream):
+    """A kernel recognised by ``patterns.match_streaming``: operands by the names the IR gave, operation
+    and BLOCK from the IR."""
+    vals = cur.named()
+    cur.done()
+    tensors = [vals[n] for n in match["inputs"]] + [vals[match["output"]]]
+    for t in tensors:
+        if not hasattr(t, "data_ptr") or not t.is_cuda:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "tensor arguments must live on the GPU")
+        _contiguous_1d(t)
+    cur.keep.extend(tensors)
+    n = int(match["n_const"] if match.get("n") is None else vals[match["n"]])
+    block = int(match["block"])
+    ptrs = [t.data_ptr() for t in tensors]
+    if match["kernel"] == "unary_kernel":
+        return lib.tt_unary_kernel(rt.UNARY_OPS[match["op"]], ptrs[0], ptrs[1], n, block, grid, stream)
+    if match["kernel"] == "binary_kernel":
+        return lib.tt_binary_kernel(rt.BINARY_OPS[match["op"]], ptrs[0], ptrs[1], ptrs[2], n, block, grid, stream)
+    return lib.tt_cast_kernel(ptrs[0], ptrs[1], n, block, _torch_dtype_code(tensors[0]), _torch_dtype_code(tensors[1]),
+                              grid, stream)
+
+
 KERNEL_TABLE: dict[str, Callable] = {
     "add_kernel": _bind_add,
     "muladd_kernel": _bind_muladd,
@@ -348,7 +379,8 @@ class BoundKernel:
             raise rt.RuntimeError_(rt.RT_ERR_NOT_FOUND, f"no prebuilt kernel named {name!r}; have {sorted(KERNEL_TABLE)}")
         self.name = name
         self.record = record
-        self.bind = KERNEL_TABLE[name]
+        match = record.get("match")
+        self.bind = functools.partial(_bind_matched, match) if match else KERNEL_TABLE[name]
 
     def __repr__(self):
         return f"<BoundKernel {self.name}>"

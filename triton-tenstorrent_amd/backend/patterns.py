@@ -1,0 +1,175 @@
+"""Recognise the masked-block elementwise form in TTIR.
+
+The operations the reference's compute lowering accepts
+(npu/lib/Dialect/TritonTenstorrent/Transforms/ConvertComputeOps.cpp:162-182) reach it inside kernels of one
+shape, the one of ``sin_kernel`` and ``add_kernel`` (examples/01-sin-kernel.py:17-29,
+python/tutorials/01-vector-add.py:29-54):
+
+    pid = program_id(0); offsets = pid * BLOCK + arange(0, BLOCK); mask = offsets < n
+    store(out + offsets, OP(load(x + offsets, mask) [, load(y + offsets, mask)]), mask)
+
+A kernel of that shape, whatever it is called, is bound to the prebuilt ``unary_kernel`` / ``binary_kernel`` /
+``cast_kernel`` with the operation read off the IR.  Nothing is generated: anything that is not exactly this
+shape over fp32 (or the two narrowing casts) is not matched and stays a compile error.
+"""
+from __future__ import annotations
+
+import re
+
+UNARY = {"math.absf": "abs", "math.ceil": "ceil", "math.cos": "cos", "math.exp": "exp", "math.exp2": "exp2",
+         "math.floor": "floor", "math.log": "log", "math.log2": "log2", "math.rsqrt": "rsqrt", "math.sin": "sin",
+         "math.sqrt": "sqrt"}
+BINARY = {"arith.addf": "add", "arith.subf": "sub", "arith.mulf": "mul", "arith.divf": "div",
+          "arith.maximumf": "maximum", "arith.minimumf": "minimum"}
+CASTS = {"arith.truncf", "arith.trunci"}
+_PLUMBING = {"tt.get_program_id", "arith.constant", "arith.muli", "tt.make_range", "tt.splat", "arith.addi",
+             "arith.cmpi", "tt.addptr", "tt.load", "tt.store", "tt.return"}
+
+_LOC = re.compile(r"\s*loc\(.*\)\s*$")
+_OP = re.compile(r"^\s*(?:(%[\w.#]+)\s*=\s*)?([a-z_]+\.[a-z_0-9.]+)\s*(.*)$")
+_SSA = re.compile(r"%[\w.#]+")
+
+
+def _strip_locs(text: str) -> str:
+    """Drop every ``loc(...)`` annotation (they nest: ``loc("x"(#loc))``)."""
+    out, i, n = [], 0, len(text)
+    while i < n:
+        j = text.find("loc(", i)
+        if j < 0 or (j > 0 and (text[j - 1].isalnum() or text[j - 1] in "_#")):
+            if j < 0:
+                out.append(text[i:])
+                break
+            out.append(text[i:j + 4])
+            i = j + 4
+            continue
+        out.append(text[i:j])
+        depth, k = 1, j + 4
+        while k < n and depth:
+            depth += text[k] == "("
+            depth -= text[k] == ")"
+            k += 1
+        i = k
+    return "".join(out)
+
+
+def _body(ttir: str):
+    ttir = _strip_locs(ttir)
+    m = re.search(r"tt\.func\s+public\s+@(\w+)\((.*?)\)\s*(?:attributes\s*\{.*?\}\s*)?\{\s*\n(.*?)\n\s*\}", ttir, re.S)
+    if not m:
+        return None
+    args = re.findall(r"(%[\w.]+)\s*:\s*([^,{]+?)\s*(?:\{[^}]*\})?\s*(?:,|$)", m.group(2))
+    return m.group(1), [(a, t.strip()) for a, t in args], m.group(3).splitlines()
+
+
+def match_streaming(ttir: str) -> dict | None:
+    """``{"kernel", "op", "inputs": [arg names], "output": name, "n": name, "block": int}`` or None."""
+    parsed = _body(ttir)
+    if parsed is None:
+        return None
+    _, args, lines = parsed
+    arg_types = dict(args)
+    defs: dict[str, tuple[str, list[str], str]] = {}
+    compute, store = [], []
+    for raw in lines:
+        line = _LOC.sub("", raw).strip()
+        if not line:
+            continue
+        m = _OP.match(line)
+        if not m:
+            return None
+        res, op, rest = m.groups()
+        operands = _SSA.findall(rest.split(" : ")[0])
+        if op in UNARY or op in BINARY or op in CASTS:
+            compute.append((res, op, operands, rest))
+        elif op == "tt.store":
+            store.append((operands, rest))
+        elif op not in _PLUMBING:
+            return None
+        if res:
+            defs[res] = (op, operands, rest)
+    if len(compute) != 1 or len(store) != 1:
+        return None
+    res, op, operands, rest = compute[0]
+
+    def pointer_arg(ptr_ssa):
+        # %p = tt.addptr %splat, %offsets ; %splat = tt.splat %arg
+        d = defs.get(ptr_ssa)
+        if not d or d[0] != "tt.addptr" or len(d[1]) != 2:
+            return None, None
+        s = defs.get(d[1][0])
+        if not s or s[0] != "tt.splat" or s[1][0] not in arg_types:
+            return None, None
+        return s[1][0], d[1][1]
+
+    (st_ops, _), = store
+    if len(st_ops) != 3 or st_ops[1] != res:
+        return None
+    out_arg, offsets = pointer_arg(st_ops[0])
+    mask = st_ops[2]
+    if out_arg is None:
+        return None
+    inputs = []
+    for o in operands:
+        d = defs.get(o)
+        if not d or d[0] != "tt.load" or len(d[1]) < 2 or d[1][1] != mask:
+            return None
+        a, offs = pointer_arg(d[1][0])
+        if a is None or offs != offsets:
+            return None
+        inputs.append(a)
+    # mask = offsets < splat(n)
+    md = defs.get(mask)
+    if not md or md[0] != "arith.cmpi" or not md[2].lstrip().startswith("slt") or md[1][0] != offsets:
+        return None
+    ns = defs.get(md[1][1])
+    if not ns or ns[0] != "tt.splat":
+        return None
+    n_src = ns[1][0] if ns[1] else None
+    n_const = None
+    if n_src not in arg_types:                 # n_elements folded to a constant (the value 1)
+        c = defs.get(n_src)
+        if not c or c[0] != "arith.constant":
+            return None
+        n_const = int(re.match(r"\s*(-?\d+)", c[2]).group(1))
+    # offsets = splat(pid * BLOCK) + make_range(0, BLOCK), either order
+    od = defs.get(offsets)
+    if not od or od[0] != "arith.addi" or len(od[1]) != 2:
+        return None
+    kinds = {defs[x][0]: x for x in od[1] if x in defs}
+    if set(kinds) != {"tt.splat", "tt.make_range"}:
+        return None
+    rng = re.search(r"end\s*=\s*(\d+)\s*:\s*i32,\s*start\s*=\s*(\d+)", defs[kinds["tt.make_range"]][2])
+    if not rng or int(rng.group(2)) != 0:
+        return None
+    block = int(rng.group(1))
+    mul = defs.get(defs[kinds["tt.splat"]][1][0])
+    if not mul or mul[0] != "arith.muli" or len(mul[1]) != 2:
+        return None
+    mk = {defs[x][0]: x for x in mul[1] if x in defs}
+    if set(mk) != {"tt.get_program_id", "arith.constant"} or not defs[mk["tt.get_program_id"]][2].lstrip().startswith("x"):
+        return None
+    if int(re.match(r"\s*(-?\d+)", defs[mk["arith.constant"]][2]).group(1)) != block:
+        return None
+    # element types
+    in_types = {arg_types[a] for a in inputs}
+    out_type = arg_types[out_arg]
+    if op in CASTS:
+        ok = (in_types, out_type) in (({"!tt.ptr<f32>"}, "!tt.ptr<bf16>"), ({"!tt.ptr<f32>"}, "!tt.ptr<f16>"),
+                                      ({"!tt.ptr<i32>"}, "!tt.ptr<i16>"), ({"!tt.ptr<i32>"}, "!tt.ptr<i8>"))
+        if not ok or len(inputs) != 1:
+            return None
+        kernel, opname = "cast_kernel", None
+    else:
+        if in_types != {"!tt.ptr<f32>"} or out_type != "!tt.ptr<f32>":
+            return None
+        if op in UNARY:
+            if len(inputs) != 1:
+                return None
+            kernel, opname = "unary_kernel", UNARY[op]
+        else:
+            if len(inputs) != 2:
+                return None
+            kernel, opname = "binary_kernel", BINARY[op]
+    strip = lambda a: a.lstrip("%")
+    return {"kernel": kernel, "op": opname, "inputs": [strip(a) for a in inputs], "output": strip(out_arg),
+            "n": strip(n_src) if n_const is None else None, "n_const": n_const, "block": block}
