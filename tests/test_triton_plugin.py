@@ -163,6 +163,22 @@ def user_to_bf16(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
 
 
 @triton.jit
+def user_fma(o_ptr, p_ptr, q_ptr, r_ptr, n, BLOCK: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(o_ptr + offs, tl.load(r_ptr + offs, mask=m) + tl.load(p_ptr + offs, mask=m) * tl.load(q_ptr + offs, mask=m), mask=m)
+
+
+@triton.jit
+def user_iadd(a_ptr, b_ptr, c_ptr, n, BLOCK: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(c_ptr + offs, tl.load(a_ptr + offs, mask=m) + tl.load(b_ptr + offs, mask=m), mask=m)
+
+
+@triton.jit
 def user_two_ops(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
     pid = tl.program_id(axis=0)
     offs = pid * BLOCK + tl.arange(0, BLOCK)
@@ -192,6 +208,14 @@ def test_elementwise_kernels_are_recognised_by_shape(tmp_path, monkeypatch):
     assert (m["kernel"], m["op"], m["inputs"], m["output"]) == ("binary_kernel", "sub", ["b_ptr", "a_ptr"], "out_ptr")
     k = _compile(user_to_bf16, {"x_ptr": f32, "y_ptr": "*bf16", "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 1024})
     assert json.loads(k.kernel)["match"]["kernel"] == "cast_kernel"
+    k = _compile(user_fma, {"o_ptr": f32, "p_ptr": f32, "q_ptr": f32, "r_ptr": f32, "n": "i32", "BLOCK": "constexpr"},
+                 {"BLOCK": 1024})
+    m = json.loads(k.kernel)["match"]
+    assert m["kernel"] == "muladd_kernel" and sorted(m["inputs"][:2]) == ["p_ptr", "q_ptr"] and m["inputs"][2] == "r_ptr"
+    k = _compile(user_iadd, {"a_ptr": "*i32", "b_ptr": "*i32", "c_ptr": "*i32", "n": "i32", "BLOCK": "constexpr"},
+                 {"BLOCK": 1024})
+    m = json.loads(k.kernel)["match"]
+    assert (m["kernel"], m["op"], m["inputs"], m["output"]) == ("add_kernel", "i32", ["a_ptr", "b_ptr"], "c_ptr")
     # not of the form: two operations, or addressing other than base + offsets
     for fn in (user_two_ops, user_strided):
         with pytest.raises(Exception, match="no prebuilt gfx950 implementation"):
@@ -220,6 +244,15 @@ def test_shape_matched_kernels_run(tmp_path, monkeypatch):
         assert np.all(np.abs(got.astype(np.float64) - want) <= 2 * np.spacing(np.abs(want))) and torch.all(out[n:] == -7.0)
         user_sub_swapped[(triton.cdiv(n, 1024), )](out, a, b, n, BLOCK=1024)
         assert torch.equal(out[:n], b - a)
+        c = torch.randn(n, device="cuda")
+        user_fma[(triton.cdiv(n, 1024), )](out, a, b, c, n, BLOCK=1024)
+        assert rt.last_kernel_name() == "ew_muladd_f32"
+        assert torch.equal(out[:n].cpu(), torch.from_numpy(np.float32(np.float64(a.cpu().numpy()) * np.float64(b.cpu().numpy())
+                                                                       + np.float64(c.cpu().numpy()))))
+        ia = torch.randint(-2**31, 2**31 - 1, (n, ), device="cuda", dtype=torch.int64).to(torch.int32)
+        ic = torch.empty_like(ia)
+        user_iadd[(triton.cdiv(n, 1024), )](ia, ia, ic, n, BLOCK=1024)
+        assert rt.last_kernel_name() == "ew_add_i32" and torch.equal(ic, ia + ia)
         h = torch.empty(n, device="cuda", dtype=torch.bfloat16)
         user_to_bf16[(triton.cdiv(n, 1024), )](a, h, n, BLOCK=1024)
         assert rt.last_kernel_name() == "ew_cast_f32_bf16" and torch.equal(h, a.to(torch.bfloat16))

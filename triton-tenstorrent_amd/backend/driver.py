@@ -348,6 +348,10 @@ def _bind_matched(match: dict, lib, cur, consts, grid, stream):
     n = int(match["n_const"] if match.get("n") is None else vals[match["n"]])
     block = int(match["block"])
     ptrs = [t.data_ptr() for t in tensors]
+    if match["kernel"] == "muladd_kernel":
+        return lib.tt_muladd_kernel(ptrs[0], ptrs[1], ptrs[2], ptrs[3], n, block, grid, stream)
+    if match["kernel"] == "add_kernel":
+        return lib.tt_add_kernel(ptrs[0], ptrs[1], ptrs[2], n, block, rt.TT_I32, grid, stream)
     if match["kernel"] == "unary_kernel":
         return lib.tt_unary_kernel(rt.UNARY_OPS[match["op"]], ptrs[0], ptrs[1], n, block, grid, stream)
     if match["kernel"] == "binary_kernel":

@@ -79,7 +79,8 @@ def match_streaming(ttir: str) -> dict | None:
             return None
         res, op, rest = m.groups()
         operands = _SSA.findall(rest.split(" : ")[0])
-        if op in UNARY or op in BINARY or op in CASTS:
+        is_int_add = op == "arith.addi" and operands and all(defs.get(o, ("",))[0] == "tt.load" for o in operands)
+        if op in UNARY or op in BINARY or op in CASTS or is_int_add:
             compute.append((res, op, operands, rest))
         elif op == "tt.store":
             store.append((operands, rest))
@@ -87,9 +88,19 @@ def match_streaming(ttir: str) -> dict | None:
             return None
         if res:
             defs[res] = (op, operands, rest)
-    if len(compute) != 1 or len(store) != 1:
+    if len(store) != 1 or len(compute) not in (1, 2):
         return None
-    res, op, operands, rest = compute[0]
+    fused = None
+    if len(compute) == 2:
+        # x * y + z, contracted to one fused multiply-add (01-vector-mul-add.py:30-57; enable_fp_fusion)
+        (mres, mop, mops, _), (ares, aop, aops, _) = compute
+        if mop != "arith.mulf" or aop != "arith.addf" or mres not in aops or len(aops) != 2:
+            return None
+        z = aops[0] if aops[1] == mres else aops[1]
+        fused = (mops, z)
+        res, op, operands = ares, "muladd", list(mops) + [z]
+    else:
+        res, op, operands, rest = compute[0]
 
     def pointer_arg(ptr_ssa):
         # %p = tt.addptr %splat, %offsets ; %splat = tt.splat %arg
@@ -153,7 +164,15 @@ def match_streaming(ttir: str) -> dict | None:
     # element types
     in_types = {arg_types[a] for a in inputs}
     out_type = arg_types[out_arg]
-    if op in CASTS:
+    if op == "muladd":
+        if in_types != {"!tt.ptr<f32>"} or out_type != "!tt.ptr<f32>" or len(inputs) != 3:
+            return None
+        kernel, opname = "muladd_kernel", None
+    elif op == "arith.addi":
+        if in_types != {"!tt.ptr<i32>"} or out_type != "!tt.ptr<i32>" or len(inputs) != 2:
+            return None
+        kernel, opname = "add_kernel", "i32"
+    elif op in CASTS:
         ok = (in_types, out_type) in (({"!tt.ptr<f32>"}, "!tt.ptr<bf16>"), ({"!tt.ptr<f32>"}, "!tt.ptr<f16>"),
                                       ({"!tt.ptr<i32>"}, "!tt.ptr<i16>"), ({"!tt.ptr<i32>"}, "!tt.ptr<i8>"))
         if not ok or len(inputs) != 1:
