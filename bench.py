@@ -204,6 +204,16 @@ def main() -> int:
         e1.record()
         torch.cuda.synchronize()
         extra["add_f32_98432"]["us_per_launch_in_hip_graph"] = round(e0.elapsed_time(e1) * 1e3 / 1000, 2)
+        # the single-block reductions: one program by construction, so a latency figure, not a roofline one
+        red = {}
+        for nr in (512, 1 << 20):
+            xr = torch.randn(nr, device="cuda")
+            zr = torch.empty(1, device="cuda")
+            for op in ("sum", "argmax"):
+                zi = zr if op == "sum" else torch.empty(1, device="cuda", dtype=torch.int32)
+                avg_ms, per, _ = _events_time(lambda: K.reduce1d_kernel[(1, )](xr, zi, BLOCK=nr, OP=op), 50, 5, stream)
+                red[f"{op}_f32_{nr}"] = {"us_avg": round(avg_ms * 1e3, 2), "us_min": round(min(per) * 1e3, 2)}
+        extra["reduce1d"] = red
         del gr
 
     # ---------------- fused epilogue: GELU(A.B + bias) ----------------------
@@ -304,6 +314,33 @@ def main() -> int:
         orc.sin(xf, of, libm_f32=True)
         dt = time.perf_counter() - t0
         extra["cpu_sin_f32"] = {"GBs": round(2 * 4 * xf.size / dt / 1e9, 3), "cores": cores, "sample": "N=2^24, libm sinf, one run"}
+        # Library-grade CPU line: the same operations through torch's CPU kernels, as the reference's examples
+        # compare against torch (01-vector-add.py:129-138).  Bounded samples, host tensors only.
+        tx, ty = torch.from_numpy(xh), torch.from_numpy(yh)
+        to = torch.empty_like(tx)
+        torch.add(tx, ty, out=to)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            torch.add(tx, ty, out=to)
+        dt_add = (time.perf_counter() - t0) / 3
+        tf32 = torch.from_numpy(xf)
+        tof = torch.empty_like(tf32)
+        torch.sin(tf32, out=tof)
+        t0 = time.perf_counter()
+        torch.sin(tf32, out=tof)
+        dt_sin = time.perf_counter() - t0
+        mt = 4096
+        ta = torch.randn(mt, mt) / math.sqrt(mt)
+        tb = torch.randn(mt, mt) / math.sqrt(mt)
+        torch.matmul(ta, tb)
+        t0 = time.perf_counter()
+        torch.matmul(ta, tb)
+        dt_mm = time.perf_counter() - t0
+        extra["cpu_torch"] = {"threads": torch.get_num_threads(),
+                              "add_i32_GBs": round(3 * 4 * ne / dt_add / 1e9, 2),
+                              "sin_f32_GBs": round(2 * 4 * xf.size / dt_sin / 1e9, 3),
+                              "matmul_f32_4096_TFLOPs": round(2.0 * mt ** 3 / dt_mm / 1e12, 4),
+                              "sample": "torch CPU kernels: add N=2^26 (mean of 3), sin N=2^24, fp32 matmul 4096^3 (one run each)"}
 
     line = {
         "metric": "GEMM TFLOP/s @8192^3 bf16 + elementwise GB/s, % of MI355X roofline",

@@ -54,8 +54,14 @@ typedef enum tt_dtype {
   TT_BF16 = 2,    /* *bf16    */
   TT_F16 = 3,     /* *fp16    */
   TT_FP8E4M3 = 4, /* *fp8e4nv (OCP e4m3fn) */
-  TT_I16 = 5,     /* *i16 (result of a narrowing cast only) */
-  TT_I8 = 6       /* *i8  (result of a narrowing cast only) */
+  TT_I16 = 5,     /* *i16 (result of a narrowing cast; reductions) */
+  TT_I8 = 6,      /* *i8  (result of a narrowing cast; reductions) */
+  TT_I64 = 7,     /* the rest: reductions only */
+  TT_F64 = 8,
+  TT_U8 = 9,      /* unsigned: Triton's IR is signless, the sign is that of the extension / compare ops */
+  TT_U16 = 10,
+  TT_U32 = 11,
+  TT_U64 = 12
 } tt_dtype;
 
 /* ----------------------------------------------------------------------- */
@@ -206,6 +212,28 @@ TTAMD_API int tt_binary_kernel(int32_t op, const void *x, const void *y, void *o
                      int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
 TTAMD_API int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
                    int32_t in_dtype, int32_t out_dtype, const uint32_t grid[3], void *stream);
+
+/* kernel(X, Z, BLOCK): x = tl.load(X + tl.arange(0, BLOCK)); tl.store(Z, tl.<op>(x, axis=0))
+ * The single-block reductions the reference's CI runs on its cpu/ path
+ * (.github/workflows/integration-tests-cpu.yml:105, test_core.py::test_reduce1d; cross-lane lowering
+ * cpu/lib/TritonCPUToLLVM/TargetInfo.cpp:95-225): sum, min, max, argmin, argmax, xor_sum over BLOCK
+ * elements of in_dtype (any of tt_dtype but fp8), 1 <= BLOCK <= 1048576.
+ * acc_dtype is the element type the tt.reduce of the IR runs in (i8 sums in i32, bf16 max in fp32 ...):
+ * integer sum / xor_sum wrap at that width and min / max are exact; float sums are carried in fp32
+ * (fp64 for f64) in tree order, so they agree with any other order only to rounding.
+ * out_dtype is Z's element type: acc_dtype or narrower (truncation / one RNE rounding); i32 or i64
+ * for the index of argmin / argmax, which is the smallest index attaining the extremum
+ * (tie_break_left; without it any such index is a legal result).  Float min / max drop NaN operands
+ * (arith.minnumf / maxnumf) unless propagate_nan (arith.minimumf / maximumf); the index reductions
+ * on NaN input return an index that depends on the fold order, as the reference's do.
+ * Every program of the grid would store the same value; it is computed once. */
+typedef enum tt_reduce_op {
+  TT_REDUCE_SUM = 0, TT_REDUCE_MIN = 1, TT_REDUCE_MAX = 2, TT_REDUCE_ARGMIN = 3, TT_REDUCE_ARGMAX = 4,
+  TT_REDUCE_XOR_SUM = 5
+} tt_reduce_op;
+TTAMD_API int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
+                       int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
+                       const uint32_t grid[3], void *stream);
 
 /* matmul_kernel_tma(a_desc, b_desc, c_desc, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
  *                   BLOCK_SIZE_K, GROUP_SIZE_M, FP8_OUTPUT, WARP_SPECIALIZE)

@@ -405,6 +405,149 @@ ORC_API void orc_trunci(const int32_t *x, void *out, int bits, int32_t n, int32_
 }
 
 /* ------------------------------------------------------------------ */
+/* Single-block reductions                                             */
+/* ------------------------------------------------------------------ */
+/*
+ * kernel(X, Z, BLOCK): tl.store(Z, tl.<op>(tl.load(X + arange(BLOCK)), axis=0)) -- the form the
+ * reference's CI runs on its cpu/ path (.github/workflows/integration-tests-cpu.yml:105,
+ * test_core.py::test_reduce1d).  What is restated is the tt.reduce of the IR, folded from the left:
+ *   sum      arith.addi / arith.addf in the accumulate type (i8 / i16 sums run in i32; a bf16 or f16
+ *            sum rounds to that type after every addition, as arith.addf on that type does)
+ *   min/max  arith.minsi|minui|maxsi|maxui, arith.minnumf|maxnumf (NaN dropped) or, with
+ *            propagate_nan, arith.minimumf|maximumf
+ *   argmin / argmax and min/max with indices: the combine region of triton/language/standard.py
+ *            (_argmin_combine / _argmax_combine):  tie = v1 == v2 and i1 < i2 (tie_break_left only);
+ *            first = v1 < v2 (resp. >) or tie;  select(first, (v1,i1), (v2,i2))
+ *   xor_sum  arith.xori
+ * dtype codes: 0 f32, 1 i32, 2 bf16, 3 f16, 5 i16, 6 i8, 7 i64, 8 f64, 9 u8, 10 u16, 11 u32, 12 u64.
+ * Returns 0, or -1 for a combination the IR cannot hold.
+ */
+static int red_bytes(int dt) {
+  switch (dt) {
+  case 6: case 9: return 1;
+  case 2: case 3: case 5: case 10: return 2;
+  case 0: case 1: case 11: return 4;
+  case 7: case 8: case 12: return 8;
+  default: return 0;
+  }
+}
+static int red_is_float(int dt) { return dt == 0 || dt == 2 || dt == 3 || dt == 8; }
+static int red_is_unsigned(int dt) { return dt >= 9 && dt <= 12; }
+
+static double red_load_f(const void *x, int64_t i, int dt) {
+  switch (dt) {
+  case 0: return ((const float *)x)[i];
+  case 2: return bf16_to_f32(((const uint16_t *)x)[i]);
+  case 3: return f16_to_f32(((const uint16_t *)x)[i]);
+  default: return ((const double *)x)[i];
+  }
+}
+/* the integer element, sign- or zero-extended to 64 bits and held as the bit pattern */
+static uint64_t red_load_i(const void *x, int64_t i, int dt) {
+  switch (dt) {
+  case 6: return (uint64_t)(int64_t)((const int8_t *)x)[i];
+  case 5: return (uint64_t)(int64_t)((const int16_t *)x)[i];
+  case 1: return (uint64_t)(int64_t)((const int32_t *)x)[i];
+  case 7: return (uint64_t)((const int64_t *)x)[i];
+  case 9: return ((const uint8_t *)x)[i];
+  case 10: return ((const uint16_t *)x)[i];
+  case 11: return ((const uint32_t *)x)[i];
+  default: return ((const uint64_t *)x)[i];
+  }
+}
+/* wrap a 64-bit pattern to the accumulate width and extend it again with the input's sign rule */
+static uint64_t red_wrap(uint64_t v, int acc_bytes, int is_unsigned) {
+  if (acc_bytes == 8) return v;
+  const int sh = 64 - 8 * acc_bytes;
+  return is_unsigned ? (v << sh) >> sh : (uint64_t)(((int64_t)(v << sh)) >> sh);
+}
+static double red_round_f(double v, int dt) {
+  switch (dt) {
+  case 0: return (float)v;
+  case 2: return bf16_to_f32(f32_to_bf16((float)v));
+  case 3: return f16_to_f32(f32_to_f16((float)v));
+  default: return v;
+  }
+}
+static int red_less_i(uint64_t a, uint64_t b, int is_unsigned) {
+  return is_unsigned ? a < b : (int64_t)a < (int64_t)b;
+}
+
+ORC_API int orc_reduce1d(int op, const void *x, int32_t n, int in_dt, int acc_dt, int out_dt,
+                         int tie_break_left, int propagate_nan, void *z) {
+  const int ib = red_bytes(in_dt), ab = red_bytes(acc_dt), ob = red_bytes(out_dt);
+  if (op < 0 || op > 5 || n <= 0 || !ib || !ab || !ob) return -1;
+  const int isf = red_is_float(in_dt), uns = red_is_unsigned(in_dt);
+  if (isf != red_is_float(acc_dt) || ab < ib) return -1;
+  if (op == 5 && isf) return -1;
+  const int arg = op == 3 || op == 4;
+  if (arg ? (out_dt != 1 && out_dt != 7) : (red_is_float(out_dt) != isf || ob > ab)) return -1;
+  int64_t idx = 0;
+  if (isf) {
+    /* f32 arithmetic on f16 / bf16 / f32 operands held in a double is exact before the rounding
+     * step below, except that an f32 sum is rounded twice (double, then float): innocuous, a double
+     * sum of two floats is exact unless their exponents differ by more than 29. */
+    double acc = red_round_f(red_load_f(x, 0, in_dt), acc_dt);
+    for (int64_t i = 1; i < n; ++i) {
+      const double v = red_round_f(red_load_f(x, i, in_dt), acc_dt);
+      switch (op) {
+      case 0: acc = red_round_f(acc + v, acc_dt); break;
+      case 1:
+        if (propagate_nan) acc = (acc != acc || v != v) ? NAN : (v < acc ? v : acc);
+        else acc = fmin(acc, v);
+        break;
+      case 2:
+        if (propagate_nan) acc = (acc != acc || v != v) ? NAN : (v > acc ? v : acc);
+        else acc = fmax(acc, v);
+        break;
+      default: {
+        const int tie = tie_break_left && acc == v && idx < i;
+        const int first = (op == 3 ? acc < v : acc > v) || tie;
+        if (!first) { acc = v; idx = i; }
+      }
+      }
+    }
+    if (!arg) {
+      switch (out_dt) {
+      case 0: *(float *)z = (float)acc; break;
+      case 2: *(uint16_t *)z = f32_to_bf16((float)acc); break;
+      case 3: *(uint16_t *)z = f32_to_f16((float)acc); break;
+      default: *(double *)z = acc;
+      }
+    }
+  } else {
+    uint64_t acc = red_wrap(red_load_i(x, 0, in_dt), ab, uns);
+    for (int64_t i = 1; i < n; ++i) {
+      const uint64_t v = red_wrap(red_load_i(x, i, in_dt), ab, uns);
+      switch (op) {
+      case 0: acc = red_wrap(acc + v, ab, uns); break;
+      case 5: acc = red_wrap(acc ^ v, ab, uns); break;
+      case 1: if (red_less_i(v, acc, uns)) acc = v; break;
+      case 2: if (red_less_i(acc, v, uns)) acc = v; break;
+      default: {
+        const int tie = tie_break_left && acc == v && idx < i;
+        const int first = (op == 3 ? red_less_i(acc, v, uns) : red_less_i(v, acc, uns)) || tie;
+        if (!first) { acc = v; idx = i; }
+      }
+      }
+    }
+    if (!arg) {
+      switch (ob) {
+      case 1: *(uint8_t *)z = (uint8_t)acc; break;
+      case 2: *(uint16_t *)z = (uint16_t)acc; break;
+      case 4: *(uint32_t *)z = (uint32_t)acc; break;
+      default: *(uint64_t *)z = acc;
+      }
+    }
+  }
+  if (arg) {
+    if (out_dt == 7) *(int64_t *)z = idx;
+    else *(int32_t *)z = (int32_t)idx;
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------ */
 /* Tile matmul family                                                  */
 /* ------------------------------------------------------------------ */
 

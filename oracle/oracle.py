@@ -72,6 +72,8 @@ def lib() -> C.CDLL:
         L.orc_binary_f32.argtypes = [C.c_int, vp, vp, vp, i32, i32, i32, C.c_int]
         L.orc_binary_f32.restype = C.c_int
         L.orc_trunci.argtypes = [vp, vp, C.c_int, i32, i32, i32]
+        L.orc_reduce1d.restype = C.c_int
+        L.orc_reduce1d.argtypes = [C.c_int, vp, i32, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, vp]
         L.orc_matmul_tiled.argtypes = [vp, vp, vp] + [i32] * 8 + [C.c_int] * 4
         L.orc_matmul_tiled.restype = C.c_int
         L.orc_attn_fwd.argtypes = [f32, vp, i32, i32, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
@@ -248,6 +250,29 @@ def trunci(x: np.ndarray, bits: int, *, block: int = 1024, grid: int | None = No
     out = np.zeros(x.shape, dtype=np.int16 if bits == 16 else np.int8)
     lib().orc_trunci(_p(x), _p(out), bits, x.size, block, cdiv(x.size, block) if grid is None else grid)
     return out
+
+
+REDUCE_OPS = {"sum": 0, "min": 1, "max": 2, "argmin": 3, "argmax": 4, "xor_sum": 5}
+I16, I8, I64, F64, U8, U16, U32, U64 = 5, 6, 7, 8, 9, 10, 11, 12
+_RED_NP = {F32: np.float32, I32: np.int32, BF16: np.uint16, F16: np.uint16, I16: np.int16, I8: np.int8, I64: np.int64,
+           F64: np.float64, U8: np.uint8, U16: np.uint16, U32: np.uint32, U64: np.uint64}
+
+
+def reduce1d(x: np.ndarray, op: str, in_dt: int, *, acc_dt: int | None = None, out_dt: int | None = None,
+             tie_break_left: bool = True, propagate_nan: bool = False):
+    """tl.<op>(x, axis=0) of one BLOCK-sized tensor, folded from the left in the accumulate type of
+    the IR (test_core.py::test_reduce1d, run by .github/workflows/integration-tests-cpu.yml:105).
+    bf16 / f16 data travel as uint16 bit patterns.  Returns a numpy scalar of the output type."""
+    acc_dt = in_dt if acc_dt is None else acc_dt
+    if out_dt is None:
+        out_dt = I32 if op in ("argmin", "argmax") else acc_dt
+    x = np.ascontiguousarray(x, dtype=_RED_NP[in_dt])
+    z = np.zeros(1, dtype=_RED_NP[out_dt])
+    rc = lib().orc_reduce1d(REDUCE_OPS[op], _p(x), x.size, in_dt, acc_dt, out_dt, int(tie_break_left),
+                            int(propagate_nan), _p(z))
+    if rc:
+        raise ValueError(f"reduce1d: {op} of dtype {in_dt} accumulated in {acc_dt} stored as {out_dt} is not expressible")
+    return z[0]
 
 
 def tilize(x: np.ndarray, TR: int, TC: int) -> np.ndarray:

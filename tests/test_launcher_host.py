@@ -64,7 +64,7 @@ def fake(monkeypatch):
     monkeypatch.setattr(drv.TTDriver, "get_current_stream", lambda self, d=None: 0x1234)
     for k in (K.add_kernel, K.add_kernel_loop, K.sin_kernel, K.matmul_kernel_tma, K.matmul_kernel_fused, K._attn_fwd,
               K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel, K.unary_kernel, K.binary_kernel,
-              K.cast_kernel):
+              K.cast_kernel, K.reduce1d_kernel):
         k._cache.clear()
     return lib
 
@@ -278,3 +278,34 @@ def test_generic_elementwise_ops_bind_by_mnemonic(fake):
         assert re.search(rf"TT_OP_{name.upper()} = {code}\b", header), name
     for name, code in rt.BINARY_OPS.items():
         assert re.search(rf"TT_OP_{name.upper()} = {code}\b", header), name
+
+
+def test_reduce1d_binds_with_tritons_accumulate_types(fake):
+    z = FakeTensor((1, ), torch.int32)
+    K.reduce1d_kernel[(1, )](FakeTensor((512, ), torch.int8), z, BLOCK=512, OP="sum")
+    name, a = fake.calls[-1]
+    assert name == "tt_reduce1d_kernel" and a[0] == rt.REDUCE_OPS["sum"] and a[3] == 512
+    assert a[4:8] == (rt.TT_I8, rt.TT_I32, rt.TT_I32, 0) and list(a[8]) == [1, 1, 1]
+    K.reduce1d_kernel[(1, )](FakeTensor((512, ), torch.uint8), FakeTensor((1, ), torch.uint32), BLOCK=512, OP="sum")
+    assert fake.calls[-1][1][4:7] == (rt.TT_U8, rt.TT_U32, rt.TT_U32)
+    K.reduce1d_kernel[(1, )](FakeTensor((64, ), torch.bfloat16), FakeTensor((1, ), torch.float32), BLOCK=64, OP="max",
+                             PROPAGATE_NAN=True)
+    assert fake.calls[-1][1][4:8] == (rt.TT_BF16, rt.TT_F32, rt.TT_F32, 1)
+    K.reduce1d_kernel[(1, )](FakeTensor((64, ), torch.bfloat16), FakeTensor((1, ), torch.bfloat16), BLOCK=64, OP="sum")
+    assert fake.calls[-1][1][4:7] == (rt.TT_BF16, rt.TT_BF16, rt.TT_BF16)
+    K.reduce1d_kernel[(1, )](FakeTensor((64, ), torch.float16), z, BLOCK=64, OP="argmin")
+    assert fake.calls[-1][1][0] == rt.REDUCE_OPS["argmin"] and fake.calls[-1][1][4:7] == (rt.TT_F16, rt.TT_F16, rt.TT_I32)
+    with pytest.raises(rt.InvalidLaunch):
+        K.reduce1d_kernel[(1, )](FakeTensor((64, ), torch.float32), z, BLOCK=64, OP="prod")
+    with pytest.raises(rt.InvalidLaunch):
+        K.reduce1d_kernel[(1, )](FakeTensor((32, ), torch.float32), z, BLOCK=64, OP="sum")     # reads past X
+    from oracle import oracle as orc
+    assert orc.REDUCE_OPS == rt.REDUCE_OPS
+    header = (ROOT / "include" / "ttamd_rt.h").read_text()
+    for name, code in rt.REDUCE_OPS.items():
+        assert re.search(rf"TT_REDUCE_{name.upper()} = {code}\b", header), name
+    for name, code in rt.DTYPE_OF_NAME.items():
+        short = {"float32": "F32", "int32": "I32", "bfloat16": "BF16", "float16": "F16", "int16": "I16", "int8": "I8",
+                 "int64": "I64", "float64": "F64", "uint8": "U8", "uint16": "U16", "uint32": "U32", "uint64": "U64"}[name]
+        assert re.search(rf"TT_{short} = {code}\b", header), name
+        assert getattr(orc, short) == code

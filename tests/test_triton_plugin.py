@@ -260,3 +260,95 @@ def test_shape_matched_kernels_run(tmp_path, monkeypatch):
         from triton.backends import backends
         backends.pop("tenstorrent", None)
         triton.runtime.driver._active = None
+
+
+# --- the single-block reductions of test_core.py::test_reduce1d (the reference's CI: integration-tests-cpu.yml:105) ---
+def _reduce_kernel(expr: str):
+    """The test's kernel with its GENERATE_TEST_HERE line filled in, as the test does by patching the source."""
+    src = ("import triton\nimport triton.language as tl\n\n@triton.jit\ndef kernel(X, Z, BLOCK: tl.constexpr):\n"
+           "    x = tl.load(X + tl.arange(0, BLOCK))\n" f"    {expr}\n" "    tl.store(Z, z)\n")
+    import importlib.util, tempfile, hashlib, os
+    path = os.path.join(tempfile.gettempdir(), f"ttamd_reduce_{hashlib.sha1(expr.encode()).hexdigest()[:12]}.py")
+    with open(path, "w") as f:
+        f.write(src)
+    spec = importlib.util.spec_from_file_location(os.path.basename(path)[:-3], path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.kernel
+
+
+REDUCE_FORMS = {
+    "sum": "z = tl.sum(x, axis=0)",
+    "min": "z = tl.min(x, axis=0)",
+    "max": "z = tl.max(x, axis=0)",
+    "min-with-indices": "z, _ = tl.min(x, axis=0, return_indices=True)",
+    "max-with-indices": "z, _ = tl.max(x, axis=0, return_indices=True)",
+    "argmin-tie-break-left": "z = tl.argmin(x, axis=0, tie_break_left=True)",
+    "argmax-tie-break-left": "z = tl.argmax(x, axis=0, tie_break_left=True)",
+    "xor_sum": "z = tl.xor_sum(x, axis=0)",
+}
+
+
+def test_reductions_are_recognised_by_shape(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton_tenstorrent_amd import runtime as rt
+
+    def match(form, x, z, block=512):
+        k = _compile(_reduce_kernel(REDUCE_FORMS[form]), {"X": x, "Z": z, "BLOCK": "constexpr"}, {"BLOCK": block})
+        rec = json.loads(k.kernel)
+        assert k.name == "kernel" and rec["kernel"] == "reduce1d_kernel"
+        m = rec["match"]
+        assert (m["inputs"], m["output"], m["block"]) == (["X"], "Z", block)
+        return m["op"], m["in_dtype"], m["acc_dtype"], m["out_dtype"], m["tie_break_left"]
+
+    assert match("sum", "*fp32", "*fp32") == ("sum", rt.TT_F32, rt.TT_F32, rt.TT_F32, False)
+    assert match("sum", "*i8", "*i32", 32) == ("sum", rt.TT_I8, rt.TT_I32, rt.TT_I32, False)        # narrow sums run in i32
+    assert match("sum", "*u16", "*u32") == ("sum", rt.TT_U16, rt.TT_I32, rt.TT_U32, False)      # zero-extended
+    assert match("sum", "*bf16", "*bf16") == ("sum", rt.TT_BF16, rt.TT_BF16, rt.TT_BF16, False)
+    assert match("max", "*bf16", "*fp32") == ("max", rt.TT_BF16, rt.TT_F32, rt.TT_F32, False)       # promoted to fp32
+    assert match("max", "*u8", "*u8") == ("max", rt.TT_U8, rt.TT_I32, rt.TT_U8, False)          # extui, maxsi, trunci
+    assert match("min", "*u32", "*u32") == ("min", rt.TT_U32, rt.TT_U32, rt.TT_U32, False)      # minui
+    assert match("min", "*i64", "*i64") == ("min", rt.TT_I64, rt.TT_I64, rt.TT_I64, False)
+    assert match("max", "*fp64", "*fp64") == ("max", rt.TT_F64, rt.TT_F64, rt.TT_F64, False)
+    assert match("min-with-indices", "*fp32", "*fp32") == ("min", rt.TT_F32, rt.TT_F32, rt.TT_F32, True)
+    assert match("max-with-indices", "*i32", "*i32") == ("max", rt.TT_I32, rt.TT_I32, rt.TT_I32, True)
+    assert match("argmin-tie-break-left", "*fp32", "*i32") == ("argmin", rt.TT_F32, rt.TT_F32, rt.TT_I32, True)
+    assert match("argmax-tie-break-left", "*i16", "*i32", 128)[0:2] == ("argmax", rt.TT_I16)
+    assert match("xor_sum", "*i32", "*i32") == ("xor_sum", rt.TT_I32, rt.TT_I32, rt.TT_I32, False)
+    # a reduction outside the set stays a compile error
+    with pytest.raises(Exception, match="no prebuilt gfx950 implementation"):
+        _compile(_reduce_kernel("z = tl.sum(x * x, axis=0)"), {"X": "*fp32", "Z": "*fp32", "BLOCK": "constexpr"}, {"BLOCK": 64})
+
+
+@pytest.mark.gpu
+def test_reductions_run_through_triton(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from oracle import oracle as orc
+    from triton_tenstorrent_amd import runtime as rt
+    ttc.register()
+    try:
+        rng = np.random.default_rng(3)
+        for form, np_dt, dt, shape in (("sum", np.int8, orc.I8, 512), ("max", np.uint8, orc.U8, 64),
+                                       ("argmin-tie-break-left", np.int32, orc.I32, 128), ("xor_sum", np.int32, orc.I32, 32),
+                                       ("min-with-indices", np.int16, orc.I16, 512)):
+            info = np.iinfo(np_dt)
+            x = rng.integers(info.min, info.max, shape, dtype=np_dt, endpoint=True)
+            op = form.split("-")[0]
+            narrow_sum = op == "sum" and np.dtype(np_dt).itemsize < 4
+            z_dt = torch.int32 if (op.startswith("arg") or narrow_sum) else torch.from_numpy(x).dtype
+            z = torch.zeros(1, device="cuda", dtype=z_dt)
+            _reduce_kernel(REDUCE_FORMS[form])[(1, )](torch.from_numpy(x).cuda(), z, BLOCK=shape)
+            assert rt.last_kernel_name().startswith("reduce1d_")
+            want = {"sum": lambda: x.astype(np.int64).sum(), "max": x.max, "min": x.min, "argmin": lambda: np.argmin(x),
+                    "xor_sum": lambda: np.bitwise_xor.reduce(x)}[op]()
+            assert int(z.cpu()[0]) == int(want), (form, np_dt)
+        xf = (rng.standard_normal(512) * 10).astype(np.float32)
+        z = torch.zeros(1, device="cuda")
+        _reduce_kernel(REDUCE_FORMS["sum"])[(1, )](torch.from_numpy(xf).cuda(), z, BLOCK=512)
+        np.testing.assert_allclose(float(z.cpu()[0]), float(np.sum(xf.astype(np.float64))), rtol=1e-5, atol=1e-3)
+        _reduce_kernel(REDUCE_FORMS["max"])[(1, )](torch.from_numpy(xf).cuda().to(torch.bfloat16), z, BLOCK=512)
+        assert float(z.cpu()[0]) == float(torch.from_numpy(xf).to(torch.bfloat16).float().max())
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None

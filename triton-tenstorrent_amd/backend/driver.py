@@ -62,7 +62,8 @@ def _torch_dtype_code(t) -> int:
         import torch
         _DTYPE_CODES = {torch.float32: rt.TT_F32, torch.int32: rt.TT_I32, torch.bfloat16: rt.TT_BF16,
                         torch.float16: rt.TT_F16, torch.float8_e4m3fn: rt.TT_FP8E4M3, torch.int16: rt.TT_I16,
-                        torch.int8: rt.TT_I8}
+                        torch.int8: rt.TT_I8, torch.int64: rt.TT_I64, torch.float64: rt.TT_F64, torch.uint8: rt.TT_U8,
+                        torch.uint16: rt.TT_U16, torch.uint32: rt.TT_U32, torch.uint64: rt.TT_U64}
     code = _DTYPE_CODES.get(t.dtype)
     if code is None:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, f"tensor dtype {t.dtype} has no kernel")
@@ -241,6 +242,41 @@ def _bind_cast(lib, cur, consts, grid, stream):
                               _torch_dtype_code(out), grid, stream)
 
 
+_FLOATS = (rt.TT_F32, rt.TT_BF16, rt.TT_F16, rt.TT_F64)
+_UNSIGNED = (rt.TT_U8, rt.TT_U16, rt.TT_U32, rt.TT_U64)
+_NARROW = (rt.TT_I8, rt.TT_I16, rt.TT_U8, rt.TT_U16, rt.TT_BF16, rt.TT_F16)
+
+
+def reduce_acc_dtype(op: str, in_dtype: int) -> int:
+    """The element type Triton's front end runs ``tl.<op>`` in (triton/language/standard.py): sums of
+    integers narrower than 32 bits run in (u)int32, min / max promote every type narrower than 32 bits
+    to int32 or fp32, xor_sum and the index reductions keep the type."""
+    if in_dtype not in _NARROW:
+        return in_dtype
+    if op == "sum":
+        if in_dtype in _FLOATS:
+            return in_dtype
+        return rt.TT_U32 if in_dtype in _UNSIGNED else rt.TT_I32
+    if op in ("xor_sum", "argmin", "argmax"):
+        return in_dtype
+    return rt.TT_F32 if in_dtype in _FLOATS else rt.TT_I32
+
+
+def _bind_reduce1d(lib, cur, consts, grid, stream):
+    """Z[0] = tl.<OP>(X[0:BLOCK], axis=0): the single-block reductions of test_core.py::test_reduce1d."""
+    x, z = _contiguous_1d(cur.tensor()), cur.tensor()
+    cur.done()
+    op = consts.get("OP")
+    if op not in rt.REDUCE_OPS:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"reduce1d_kernel: OP {op!r}, have {sorted(rt.REDUCE_OPS)}")
+    block = int(consts["BLOCK"])
+    if x.numel() < block or z.numel() < 1:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"reduce1d_kernel: X holds {x.numel()} elements, BLOCK is {block}")
+    in_dt = _torch_dtype_code(x)
+    return lib.tt_reduce1d_kernel(rt.REDUCE_OPS[op], x.data_ptr(), z.data_ptr(), block, in_dt, reduce_acc_dtype(op, in_dt),
+                                  _torch_dtype_code(z), int(bool(consts.get("PROPAGATE_NAN", False))), grid, stream)
+
+
 def _mnk(cur: _Cursor, a: rt.tt_desc2d, b: rt.tt_desc2d):
     """M, N, K follow the descriptors when the signature carries them; the
     minimal variant reads them from ``desc.shape`` (kernel_matmul_tma.py:71-75).
@@ -348,6 +384,11 @@ def _bind_matched(match: dict, lib, cur, consts, grid, stream):
     n = int(match["n_const"] if match.get("n") is None else vals[match["n"]])
     block = int(match["block"])
     ptrs = [t.data_ptr() for t in tensors]
+    if match["kernel"] == "reduce1d_kernel":
+        if tensors[0].numel() < block:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"the kernel reads {block} elements, its input holds {tensors[0].numel()}")
+        return lib.tt_reduce1d_kernel(rt.REDUCE_OPS[match["op"]], ptrs[0], ptrs[1], block, match["in_dtype"],
+                                      match["acc_dtype"], match["out_dtype"], int(match["propagate_nan"]), grid, stream)
     if match["kernel"] == "muladd_kernel":
         return lib.tt_muladd_kernel(ptrs[0], ptrs[1], ptrs[2], ptrs[3], n, block, grid, stream)
     if match["kernel"] == "add_kernel":
@@ -367,6 +408,7 @@ KERNEL_TABLE: dict[str, Callable] = {
     "unary_kernel": _bind_unary,
     "binary_kernel": _bind_binary,
     "cast_kernel": _bind_cast,
+    "reduce1d_kernel": _bind_reduce1d,
     "matmul_kernel_tma": _bind_matmul_tma,
     "matmul_kernel_tma_fp8_scaled": _bind_matmul_tma,
     "matmul_kernel_fused": _bind_matmul_fused,

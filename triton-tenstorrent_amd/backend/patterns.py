@@ -11,6 +11,13 @@ python/tutorials/01-vector-add.py:29-54):
 A kernel of that shape, whatever it is called, is bound to the prebuilt ``unary_kernel`` / ``binary_kernel`` /
 ``cast_kernel`` with the operation read off the IR.  Nothing is generated: anything that is not exactly this
 shape over fp32 (or the two narrowing casts) is not matched and stays a compile error.
+
+The second form is the single-block reduction the reference's CI runs on its cpu/ path
+(.github/workflows/integration-tests-cpu.yml:105, test_core.py::test_reduce1d):
+
+    x = load(X + arange(0, BLOCK)); store(Z, reduce(x, axis=0))
+
+bound to ``reduce1d_kernel`` with the reduction, the element types and the NaN rule read off the ``tt.reduce``.
 """
 from __future__ import annotations
 
@@ -90,14 +97,12 @@ def match_streaming(ttir: str) -> dict | None:
             defs[res] = (op, operands, rest)
     if len(store) != 1 or len(compute) not in (1, 2):
         return None
-    fused = None
     if len(compute) == 2:
         # x * y + z, contracted to one fused multiply-add (01-vector-mul-add.py:30-57; enable_fp_fusion)
         (mres, mop, mops, _), (ares, aop, aops, _) = compute
         if mop != "arith.mulf" or aop != "arith.addf" or mres not in aops or len(aops) != 2:
             return None
         z = aops[0] if aops[1] == mres else aops[1]
-        fused = (mops, z)
         res, op, operands = ares, "muladd", list(mops) + [z]
     else:
         res, op, operands, rest = compute[0]
@@ -192,3 +197,140 @@ def match_streaming(ttir: str) -> dict | None:
     strip = lambda a: a.lstrip("%")
     return {"kernel": kernel, "op": opname, "inputs": [strip(a) for a in inputs], "output": strip(out_arg),
             "n": strip(n_src) if n_const is None else None, "n_const": n_const, "block": block}
+
+
+_ELEM = {"f32": 0, "i32": 1, "bf16": 2, "f16": 3, "i16": 5, "i8": 6, "i64": 7, "f64": 8}
+_UNSIGNED_OF = {6: 9, 5: 10, 1: 11, 7: 12}
+_REDUCE = re.compile(r'(%[\w.#]+)(?::(\d))?\s*=\s*"tt\.reduce"\(([^)]*)\)\s*<\{axis = 0 : i32\}>\s*\(\{\s*\n(.*?)\n\s*\}\)'
+                     r'\s*:\s*\(([^)]*)\)\s*->\s*([^\n]*)\n', re.S)
+_FOLDS = {"arith.addf": ("sum", None), "arith.addi": ("sum", None), "arith.xori": ("xor_sum", None),
+          "arith.maxnumf": ("max", None), "arith.minnumf": ("min", None),
+          "arith.maximumf": ("max", "nan"), "arith.minimumf": ("min", "nan"),
+          "arith.maxsi": ("max", "s"), "arith.minsi": ("min", "s"), "arith.maxui": ("max", "u"), "arith.minui": ("min", "u")}
+
+
+def _ops_of(lines):
+    out = []
+    for raw in lines:
+        line = raw.strip()
+        if not line or line.startswith("^bb") or line == "}":
+            continue
+        m = _OP.match(line)
+        if not m:
+            return None
+        res, op, rest = m.groups()
+        out.append((res, op, _SSA.findall(rest.split(" : ")[0]), rest))
+    return out
+
+
+def match_reduce1d(ttir: str) -> dict | None:
+    """``{"kernel": "reduce1d_kernel", "op", "inputs": [X], "output": Z, "block", "in_dtype", "acc_dtype",
+    "out_dtype", "propagate_nan", "tie_break_left"}`` (dtypes as tt_dtype codes) or None."""
+    text = _strip_locs(ttir)
+    f = re.search(r"tt\.func\s+public\s+@(\w+)\((.*?)\)\s*(?:attributes\s*\{.*?\}\s*)?\{\s*\n", text, re.S)
+    if not f:
+        return None
+    arg_types = {a: t.strip() for a, t in re.findall(r"(%[\w.]+)\s*:\s*([^,{]+?)\s*(?:\{[^}]*\})?\s*(?:,|$)", f.group(2))}
+    body = text[f.end():]
+    r = _REDUCE.search(body)
+    if not r or _REDUCE.search(body, r.end()):
+        return None
+    res, nres, red_operands, region, in_tensors, out_types = r.groups()
+    red_operands = _SSA.findall(red_operands)
+    tail = body[r.end():]
+    end = tail.find("tt.return")
+    if end < 0:
+        return None
+    pre, fold, post = (_ops_of(t.splitlines()) for t in (body[:r.start()], region, tail[:end + len("tt.return")]))
+    if pre is None or fold is None or post is None or len(red_operands) not in (1, 2):
+        return None
+    defs = {o[0]: o for o in pre if o[0]}
+    if any(o[1] not in ("tt.make_range", "tt.splat", "tt.addptr", "tt.load", "arith.extsi", "arith.extui", "arith.extf")
+           for o in pre):
+        return None
+    # value operand: [ext of] load(addptr(splat(X), make_range(0, BLOCK))), no mask
+    v = defs.get(red_operands[0])
+    ext = None
+    if v and v[1].startswith("arith.ext"):
+        ext, v = v[1], defs.get(v[2][0])
+    if not v or v[1] != "tt.load" or len(v[2]) != 1:
+        return None
+    ap = defs.get(v[2][0])
+    if not ap or ap[1] != "tt.addptr" or len(ap[2]) != 2:
+        return None
+    sp, rg = defs.get(ap[2][0]), defs.get(ap[2][1])
+    if not sp or sp[1] != "tt.splat" or sp[2][0] not in arg_types or not rg or rg[1] != "tt.make_range":
+        return None
+    x_arg = sp[2][0]
+    span = re.search(r"end\s*=\s*(\d+)\s*:\s*i32,\s*start\s*=\s*(\d+)", rg[3])
+    if not span or int(span.group(2)) != 0:
+        return None
+    block = int(span.group(1))
+    if len(red_operands) == 2 and red_operands[1] != rg[0]:      # the index operand is the same arange
+        return None
+    # element types: X's, the one the reduction runs in, Z's
+    pe = re.fullmatch(r"!tt\.ptr<(\w+)>", arg_types[x_arg])
+    te = re.match(r"tensor<%dx(\w+)>" % block, in_tensors.strip())
+    if not pe or not te or pe.group(1) not in _ELEM or te.group(1) not in _ELEM:
+        return None
+    in_dt, acc_dt = _ELEM[pe.group(1)], _ELEM[te.group(1)]
+    if (ext is None) != (in_dt == acc_dt):
+        return None
+    kinds = [o[1] for o in fold if o[1] != "tt.reduce.return"]
+    unsigned, nan, tie = ext == "arith.extui", False, False
+    if len(red_operands) == 1:
+        if len(kinds) != 1 or kinds[0] not in _FOLDS:
+            return None
+        op, rule = _FOLDS[kinds[0]]
+        unsigned |= rule == "u"
+        nan = rule == "nan"
+        want = None
+    else:
+        # the (value, index) combine of triton/language/standard.py: compares, and / or, two selects
+        if any(k not in ("arith.cmpf", "arith.cmpi", "arith.andi", "arith.ori", "arith.select") for k in kinds) \
+                or kinds.count("arith.select") != 2:
+            return None
+        preds = [o[3].split()[0].rstrip(",") for o in fold if o[1] in ("arith.cmpf", "arith.cmpi")]
+        order = [p for p in preds if p in ("olt", "ogt", "slt", "sgt", "ult", "ugt")]
+        # with tie_break_left the index compare adds one `slt`; the value compare is the last one written
+        tie = any(p in ("oeq", "eq") for p in preds)
+        if not order or len(order) != (2 if tie else 1) or (tie and order[0] != "slt"):
+            return None
+        unsigned |= order[-1] in ("ult", "ugt")
+        op = "min" if order[-1].endswith("lt") else "max"
+        want = {"0": "value", "1": "index"}
+    if unsigned:
+        if in_dt not in _UNSIGNED_OF:
+            return None
+        in_dt = _UNSIGNED_OF[in_dt]
+        acc_dt = _UNSIGNED_OF.get(acc_dt, acc_dt) if ext is None else acc_dt
+    # after the reduction: [trunc] then store(Z, result)
+    if not post or post[-1][1] != "tt.return" or len(post) not in (2, 3):
+        return None
+    st = post[-2]
+    if st[1] != "tt.store" or len(st[2]) != 2 or st[2][0] not in arg_types:
+        return None
+    stored = st[2][1]
+    if len(post) == 3:
+        if post[0][1] not in ("arith.trunci", "arith.truncf") or post[0][0] != stored or len(post[0][2]) != 1:
+            return None
+        stored = post[0][2][0]
+    if want is None:
+        if stored != res:
+            return None
+    else:
+        which = stored.split("#")
+        if len(which) != 2 or which[0] != res or which[1] not in want:
+            return None
+        if which[1] == "1":
+            op = "arg" + op
+    ze = re.fullmatch(r"!tt\.ptr<(\w+)>", arg_types[st[2][0]])
+    if not ze or ze.group(1) not in _ELEM:
+        return None
+    out_dt = _ELEM[ze.group(1)]
+    if unsigned and not op.startswith("arg"):
+        out_dt = _UNSIGNED_OF.get(out_dt, out_dt)
+    strip = lambda a: a.lstrip("%")
+    return {"kernel": "reduce1d_kernel", "op": op, "inputs": [strip(x_arg)], "output": strip(st[2][0]), "n": None,
+            "n_const": block, "block": block, "in_dtype": in_dt, "acc_dtype": acc_dt, "out_dtype": out_dt,
+            "propagate_nan": nan, "tie_break_left": tie}

@@ -21,8 +21,8 @@ BUILD = PKG / "build"
 LIB = PKG / "lib" / "libttamd_rt.so"
 ARCH = "gfx950"
 
-CODE_OBJECTS = ["elementwise", "gemm", "attention"]
-RT_SOURCES = ["ttamd_rt.cpp", "tt_elementwise.cpp", "tt_gemm.cpp", "tt_attention.cpp"]
+CODE_OBJECTS = ["elementwise", "gemm", "attention", "reduce"]
+RT_SOURCES = ["ttamd_rt.cpp", "tt_elementwise.cpp", "tt_gemm.cpp", "tt_attention.cpp", "tt_reduce.cpp"]
 
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 on this target
 DEVICE_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

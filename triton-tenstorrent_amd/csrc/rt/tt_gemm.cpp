@@ -14,7 +14,7 @@ namespace {
 int check_desc(const char *who, const char *what, const tt_desc2d *d, int64_t rows, int64_t cols) {
   if (!d) return fail(RT_ERR_INVALID, "%s: null %s descriptor", who, what);
   if (!d->base) return fail(RT_ERR_INVALID, "%s: %s descriptor has a null base", who, what);
-  if (dtype_size(d->dtype) == 0 || d->dtype == TT_I32)
+  if (d->dtype != TT_F32 && d->dtype != TT_BF16 && d->dtype != TT_F16 && d->dtype != TT_FP8E4M3)
     return fail(RT_ERR_UNSUPPORTED, "%s: %s dtype %d", who, what, d->dtype);
   if (d->padding_nan)
     return fail(RT_ERR_UNSUPPORTED, "%s: %s descriptor asks for NaN padding; only zero padding exists",

@@ -20,9 +20,10 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline size_t dtype_size(int dt) {
   switch (dt) {
-  case TT_F32: case TT_I32: return 4;
-  case TT_BF16: case TT_F16: return 2;
-  case TT_FP8E4M3: return 1;
+  case TT_F32: case TT_I32: case TT_U32: return 4;
+  case TT_BF16: case TT_F16: case TT_I16: case TT_U16: return 2;
+  case TT_FP8E4M3: case TT_I8: case TT_U8: return 1;
+  case TT_I64: case TT_U64: case TT_F64: return 8;
   default: return 0;
   }
 }

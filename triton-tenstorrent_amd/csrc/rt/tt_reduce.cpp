@@ -1,0 +1,66 @@
+// tt_reduce1d_kernel: launch validation and kernel selection for the single-block reductions.
+#include "tt_internal.h"
+
+using namespace ttamd;
+
+namespace {
+struct TypeInfo { const char *kernel; int bytes; bool is_float; };
+bool type_info(int dt, TypeInfo *t) {
+  switch (dt) {
+  case TT_I8: *t = {"reduce1d_i8", 1, false}; return true;
+  case TT_I16: *t = {"reduce1d_i16", 2, false}; return true;
+  case TT_I32: *t = {"reduce1d_i32", 4, false}; return true;
+  case TT_I64: *t = {"reduce1d_i64", 8, false}; return true;
+  case TT_U8: *t = {"reduce1d_u8", 1, false}; return true;
+  case TT_U16: *t = {"reduce1d_u16", 2, false}; return true;
+  case TT_U32: *t = {"reduce1d_u32", 4, false}; return true;
+  case TT_U64: *t = {"reduce1d_u64", 8, false}; return true;
+  case TT_F32: *t = {"reduce1d_f32", 4, true}; return true;
+  case TT_BF16: *t = {"reduce1d_bf16", 2, true}; return true;
+  case TT_F16: *t = {"reduce1d_f16", 2, true}; return true;
+  case TT_F64: *t = {"reduce1d_f64", 8, true}; return true;
+  default: return false;
+  }
+}
+} // namespace
+
+extern "C" int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
+                                  int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
+                                  const uint32_t grid[3], void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "reduce1d: call rt_init first");
+  if (!grid) return fail(RT_ERR_INVALID, "reduce1d: null grid");
+  if (!x || !z) return fail(RT_ERR_INVALID, "reduce1d: null pointer");
+  if (op < TT_REDUCE_SUM || op > TT_REDUCE_XOR_SUM) return fail(RT_ERR_INVALID, "reduce1d: op %d", op);
+  // TRITON_MAX_TENSOR_NUMEL
+  if (BLOCK <= 0 || BLOCK > 1048576) return fail(RT_ERR_INVALID, "reduce1d: BLOCK %d (1..1048576)", BLOCK);
+  if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return fail(RT_ERR_INVALID, "reduce1d: empty grid");
+  TypeInfo in, acc, out;
+  if (!type_info(in_dtype, &in) || !type_info(acc_dtype, &acc) || !type_info(out_dtype, &out))
+    return fail(RT_ERR_UNSUPPORTED, "reduce1d: dtypes in %d, accumulate %d, out %d", in_dtype, acc_dtype, out_dtype);
+  if (reinterpret_cast<uintptr_t>(x) % in.bytes || reinterpret_cast<uintptr_t>(z) % out.bytes)
+    return fail(RT_ERR_INVALID, "reduce1d: pointer not aligned to its element size");
+  const bool arg = op == TT_REDUCE_ARGMIN || op == TT_REDUCE_ARGMAX;
+  if (in.is_float != acc.is_float || acc.bytes < in.bytes)
+    return fail(RT_ERR_UNSUPPORTED, "reduce1d: accumulate dtype %d for input dtype %d", acc_dtype, in_dtype);
+  if (op == TT_REDUCE_XOR_SUM && in.is_float) return fail(RT_ERR_INVALID, "reduce1d: xor_sum of a float tensor");
+  if (propagate_nan && (!in.is_float || (op != TT_REDUCE_MIN && op != TT_REDUCE_MAX)))
+    return fail(RT_ERR_INVALID, "reduce1d: propagate_nan applies to float min / max only");
+  int out_kind = 0;
+  if (arg) {
+    if (out_dtype != TT_I32 && out_dtype != TT_I64)
+      return fail(RT_ERR_UNSUPPORTED, "reduce1d: the index result is i32 or i64, got dtype %d", out_dtype);
+  } else if (in.is_float) {
+    // the value leaves in the accumulator's type or narrower (arith.truncf), never widened
+    if (!out.is_float || out.bytes > acc.bytes || (in_dtype == TT_F64) != (acc_dtype == TT_F64))
+      return fail(RT_ERR_UNSUPPORTED, "reduce1d: float accumulate %d -> out %d", acc_dtype, out_dtype);
+    out_kind = out_dtype == TT_F64 ? 4 : out_dtype == TT_F32 ? 1 : out_dtype == TT_BF16 ? 2 : 3;
+  } else {
+    if (out.is_float || out.bytes > acc.bytes)
+      return fail(RT_ERR_UNSUPPORTED, "reduce1d: integer accumulate %d -> out %d (widening after the reduction "
+                  "is not offered)", acc_dtype, out_dtype);
+  }
+  int32_t n = BLOCK, op_ = op, nan_ = propagate_nan ? 1 : 0, ob = out.bytes;
+  void *args[] = {(void *)&x, (void *)&z, &n, &op_, &nan_, &ob, &out_kind};
+  // Every program of the logical grid computes and stores the same value; one workgroup does it once.
+  return launch("reduce", in.kernel, dim3(1), dim3(1024), 0, stream, args, 7);
+}

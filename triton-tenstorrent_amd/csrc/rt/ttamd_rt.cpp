@@ -37,6 +37,7 @@
 TTAMD_EMBED(ttamd_co_elementwise, "elementwise.hsaco")
 TTAMD_EMBED(ttamd_co_gemm, "gemm.hsaco")
 TTAMD_EMBED(ttamd_co_attention, "attention.hsaco")
+TTAMD_EMBED(ttamd_co_reduce, "reduce.hsaco")
 
 struct rt_module_s {
   hipModule_t mod = nullptr;
@@ -158,7 +159,8 @@ int rt_init(int device) {
   struct Img { const char *name; const char *b; const char *e; };
   const Img imgs[] = {{"elementwise", ttamd_co_elementwise_begin, ttamd_co_elementwise_end},
                       {"gemm", ttamd_co_gemm_begin, ttamd_co_gemm_end},
-                      {"attention", ttamd_co_attention_begin, ttamd_co_attention_end}};
+                      {"attention", ttamd_co_attention_begin, ttamd_co_attention_end},
+                      {"reduce", ttamd_co_reduce_begin, ttamd_co_reduce_end}};
   for (const Img &im : imgs) {
     auto *m = new rt_module_s();
     hipError_t e = hipModuleLoadData(&m->mod, im.b);

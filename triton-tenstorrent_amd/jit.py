@@ -29,7 +29,8 @@ def _typestr_of_torch(dtype) -> str:
         import torch
         _TORCH_TYPESTR = {torch.float32: "fp32", torch.int32: "i32", torch.bfloat16: "bf16", torch.float16: "fp16",
                           torch.float8_e4m3fn: "fp8e4nv", torch.float8_e5m2: "fp8e5", torch.int64: "i64",
-                          torch.float64: "fp64", torch.int8: "i8", torch.uint8: "u8", torch.int16: "i16"}
+                          torch.float64: "fp64", torch.int8: "i8", torch.uint8: "u8", torch.int16: "i16",
+                          torch.uint16: "u16", torch.uint32: "u32", torch.uint64: "u64"}
     return _TORCH_TYPESTR[dtype]
 
 

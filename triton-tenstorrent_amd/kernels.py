@@ -61,6 +61,28 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+reduce1d_kernel = PrebuiltKernel("reduce1d_kernel", ["X", "Z", "BLOCK", "OP", "PROPAGATE_NAN"], ["BLOCK", "OP", "PROPAGATE_NAN"],
+                                 defaults={"PROPAGATE_NAN": False})
+
+
+def reduce1d(op: str, x: torch.Tensor, out_dtype: torch.dtype | None = None, propagate_nan: bool = False) -> torch.Tensor:
+    """``tl.<op>(x, axis=0)`` of one block: ``op`` in sum, min, max, argmin, argmax, xor_sum
+    (test_core.py::test_reduce1d).  The result has the dtype the reduction runs in (int32 for the
+    index reductions and for sums of narrow integers, fp32 for min / max of bf16 and fp16) unless
+    ``out_dtype`` names a narrower one."""
+    from .backend.driver import reduce_acc_dtype, _torch_dtype_code
+    if out_dtype is None:
+        if op in ("argmin", "argmax"):
+            out_dtype = torch.int32
+        else:
+            code = reduce_acc_dtype(op, _torch_dtype_code(x))
+            from .backend import driver as _d
+            out_dtype = next(k for k, v in _d._DTYPE_CODES.items() if v == code)
+    z = torch.empty(1, device=x.device, dtype=out_dtype)
+    reduce1d_kernel[(1, )](x, z, BLOCK=x.numel(), OP=op, PROPAGATE_NAN=propagate_nan)
+    return z
+
+
 def add(x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
     output = torch.empty_like(x)
     n_elements = output.numel()

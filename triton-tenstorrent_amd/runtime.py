@@ -14,10 +14,17 @@ LIB_PATH = PKG / "lib" / "libttamd_rt.so"
 
 RT_OK, RT_ERR_INVALID, RT_ERR_HIP, RT_ERR_NOT_FOUND, RT_ERR_UNSUPPORTED, RT_ERR_NOT_INIT = 0, -1, -2, -3, -4, -5
 TT_F32, TT_I32, TT_BF16, TT_F16, TT_FP8E4M3, TT_I16, TT_I8 = 0, 1, 2, 3, 4, 5, 6
+TT_I64, TT_F64, TT_U8, TT_U16, TT_U32, TT_U64 = 7, 8, 9, 10, 11, 12
 # tt_unary_op / tt_binary_op of the header, by the name of the MLIR operation's mnemonic
 UNARY_OPS = {"abs": 0, "ceil": 1, "cos": 2, "exp": 3, "exp2": 4, "floor": 5, "log": 6, "log2": 7, "rsqrt": 8, "sin": 9,
              "sqrt": 10}
 BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
+# tt_reduce_op of the header, by the name of the tl.* reduction
+REDUCE_OPS = {"sum": 0, "min": 1, "max": 2, "argmin": 3, "argmax": 4, "xor_sum": 5}
+# element type names (numpy / torch spelling) -> tt_dtype, for the reductions
+DTYPE_OF_NAME = {"float32": TT_F32, "int32": TT_I32, "bfloat16": TT_BF16, "float16": TT_F16, "int16": TT_I16,
+                 "int8": TT_I8, "int64": TT_I64, "float64": TT_F64, "uint8": TT_U8, "uint16": TT_U16,
+                 "uint32": TT_U32, "uint64": TT_U64}
 TT_EPI_NONE, TT_EPI_BIAS_FULL, TT_EPI_BIAS_ROW_GELU, TT_EPI_LEAKY_RELU, TT_EPI_BIAS_ROW = 0, 1, 2, 3, 4
 
 # Triton pointer type strings -> tt_dtype
@@ -86,6 +93,7 @@ SYMBOLS = {
     "tt_unary_kernel": (C.c_int, [_i32, _vp, _vp, _i32, _i32, _G, _vp]),
     "tt_binary_kernel": (C.c_int, [_i32, _vp, _vp, _vp, _i32, _i32, _G, _vp]),
     "tt_cast_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _G, _vp]),
+    "tt_reduce1d_kernel": (C.c_int, [_i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_fused": (C.c_int, [_DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma_fp8_scaled": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _f32, _f32, _i32, _i32, _i32, _i32, _G, _vp]),
