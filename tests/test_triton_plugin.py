@@ -352,3 +352,25 @@ def test_reductions_run_through_triton(tmp_path, monkeypatch):
         from triton.backends import backends
         backends.pop("tenstorrent", None)
         triton.runtime.driver._active = None
+
+
+def test_offline_compile_tool_accepts_the_tenstorrent_target(tmp_path, monkeypatch):
+    """README.md:74-77 of the reference: `compile.py --target tenstorrent:0:1 --signature "*fp32,*fp32,*fp32,i32,1024"
+    --grid 1,1,1 -n add_kernel <source>` prints nothing and leaves its artefacts in the Triton cache."""
+    import sys
+    import triton.tools.compile as aot
+    from triton_tenstorrent_amd.examples import triton_kernels as tk
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path / "cache"))
+    monkeypatch.setattr(sys, "argv", ["compile.py", "--target", "tenstorrent:0:1", "--signature", "*fp32,*fp32,*fp32,i32,1024",
+                                      "--grid", "1,1,1", "-n", "add_kernel", "-o", str(tmp_path / "out"), tk.__file__])
+    ttc.register()
+    try:
+        aot.main()
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None
+    made = {p.name for p in (tmp_path / "cache").rglob("add_kernel.*")}
+    assert {"add_kernel.ttir", "add_kernel.ttamd", "add_kernel.json"} <= made
+    record = json.loads(next((tmp_path / "cache").rglob("add_kernel.ttamd")).read_text())
+    assert record["kernel"] == "add_kernel" and record["arch"] == "gfx950"

@@ -170,6 +170,11 @@ class TTBackend(BaseBackend):
         metadata["name"] = name
         metadata["shared"] = 0
         metadata["warp_size"] = 64
+        # read by triton/tools/compile.py after an ahead-of-time compile (backend/compiler.py:385-386)
+        metadata["global_scratch_size"] = 0
+        metadata["global_scratch_align"] = 1
+        metadata["profile_scratch_size"] = 0
+        metadata["profile_scratch_align"] = 1
         return json.dumps(record).encode()
 
     def add_stages(self, stages, options, language=None):
