@@ -181,6 +181,10 @@ def main() -> int:
             avg_ms, per, _ = _events_time(lambda: K.binary_kernel[egrid](xs, ys, outs, n_el, BLOCK_SIZE=1024, OP=op),
                                           max(3, steps // 4), 2, stream)
             ops[op] = round(3 * 4 * n_el / (avg_ms * 1e-3) / 1e9, 1)
+        ob = torch.empty(n_el, device="cuda", dtype=torch.bfloat16)
+        avg_ms, per, _ = _events_time(lambda: K.cast_kernel[egrid](xs, ob, n_el, BLOCK_SIZE=1024), max(3, steps // 4), 2, stream)
+        ops["truncf_bf16"] = round((4 + 2) * n_el / (avg_ms * 1e-3) / 1e9, 1)
+        del ob
         extra["elementwise_ops_2p28_GBs"] = ops
         del xs, ys, outs
     if want("add0"):

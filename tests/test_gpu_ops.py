@@ -94,6 +94,29 @@ def test_narrowing_casts_exact():
         K.cast(xf.cuda(), torch.int8)
 
 
+@pytest.mark.parametrize("n", [1, 7, 16, 8191, 8192, 16384, 32768 + 5, 131072 + 17, 1 << 22])
+@pytest.mark.parametrize("offset", [0, 1, 4])
+def test_narrowing_casts_sizes_alignments_and_sentinel(n, offset):
+    # whole runs of the 16-byte path, ragged ends, operands off the 16-byte grid (element offsets 1) and on it (4);
+    # nothing is written past n
+    g = torch.Generator().manual_seed(n + offset)
+    xf = (torch.randn(n + offset, generator=g) * 100)[offset:]
+    xi = torch.randint(-2**31, 2**31 - 1, (n + offset, ), dtype=torch.int64, generator=g).to(torch.int32)[offset:]
+    for src, dt, want in ((xf, torch.bfloat16, xf.to(torch.bfloat16)), (xf, torch.float16, xf.to(torch.float16)),
+                          (xi, torch.int16, torch.from_numpy(orc.trunci(xi.numpy(), 16))),
+                          (xi, torch.int8, torch.from_numpy(orc.trunci(xi.numpy(), 8)))):
+        sent = 77 if dt in (torch.int16, torch.int8) else 7.5
+        buf = torch.full((n + offset + 40, ), sent, dtype=dt, device="cuda")
+        out = buf[offset:offset + n]
+        xs = src.cuda()
+        xs = torch.cat([torch.zeros(offset, dtype=xs.dtype, device="cuda"), xs])[offset:]      # same misalignment on the input
+        K.cast_kernel[lambda meta: (K.cdiv(n, meta["BLOCK_SIZE"]), )](xs, out, n, BLOCK_SIZE=1024)
+        aligned = xs.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0
+        assert rt.last_kernel_name().endswith("_unaligned") != aligned
+        assert torch.equal(out.cpu(), want), (dt, n, offset)
+        assert torch.all(buf[:offset] == sent) and torch.all(buf[offset + n:] == sent)
+
+
 def test_full_size_streaming_properties():
     # 2^28 elements: exp(log(x)) ~ x, sqrt(x)^2 ~ x, x/x == 1, max(x,y)+min(x,y) == x+y bit for bit
     n = 1 << 28

@@ -242,6 +242,43 @@ __device__ __forceinline__ void cast_body(const typename Op::in_t *x, typename O
   for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = Op::apply(x[i]);
 }
 
+// 16-byte aligned operands: a lane turns 16 / sizeof(out) inputs (2 or 4 loads of 16 bytes) into one 16-byte
+// store; a workgroup owns one contiguous run of kThreads * UNROLL such items, the last one also the ragged end.
+template <typename Op, int UNROLL>
+__device__ __forceinline__ void cast_vec_body(const typename Op::in_t *__restrict__ x, typename Op::out_t *__restrict__ out,
+                                              uint32_t n) {
+  using In = typename Op::in_t;
+  using Out = typename Op::out_t;
+  constexpr int E = 16 / (int)sizeof(Out);   // elements per item: 8 or 16
+  constexpr int LOADS = E / 4;
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  union InV { u32x4_t q; In e[4]; };
+  union OutV { u32x4_t q; Out e[E]; };
+  const uint32_t nitem = n / E;
+  const u32x4_t *xv = reinterpret_cast<const u32x4_t *>(x);
+  u32x4_t *ov = reinterpret_cast<u32x4_t *>(out);
+  const uint32_t base = blockIdx.x * (kThreads * UNROLL);
+  const uint32_t i = base + threadIdx.x;
+  if (base + kThreads * UNROLL <= nitem) {
+    InV a[UNROLL][LOADS];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+      for (int l = 0; l < LOADS; ++l) a[u][l].q = __builtin_nontemporal_load(xv + (size_t)(i + u * kThreads) * LOADS + l);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      OutV r;
+#pragma unroll
+      for (int l = 0; l < LOADS; ++l)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r.e[l * 4 + e] = Op::apply(a[u][l].e[e]);
+      __builtin_nontemporal_store(r.q, ov + i + u * kThreads);
+    }
+  } else {
+    for (uint32_t j = (size_t)base * E + threadIdx.x; j < n; j += kThreads) out[j] = Op::apply(x[j]);
+  }
+}
+
 struct MulAdd {
   __device__ static float apply(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 };
@@ -304,18 +341,17 @@ EW_BINARY(div, DivOp)
 EW_BINARY(max, MaxOp)
 EW_BINARY(min, MinOp)
 
-__global__ __launch_bounds__(kThreads) void ew_cast_f32_bf16(const float *x, uint16_t *out, uint32_t n) {
-  cast_body<ToBf16>(x, out, n);
-}
-__global__ __launch_bounds__(kThreads) void ew_cast_f32_f16(const float *x, uint16_t *out, uint32_t n) {
-  cast_body<ToF16>(x, out, n);
-}
-__global__ __launch_bounds__(kThreads) void ew_cast_i32_i16(const int *x, int16_t *out, uint32_t n) {
-  cast_body<ToI16>(x, out, n);
-}
-__global__ __launch_bounds__(kThreads) void ew_cast_i32_i8(const int *x, int8_t *out, uint32_t n) {
-  cast_body<ToI8>(x, out, n);
-}
+#define EW_CAST(name, Op, IN, OUT)                                                                          \
+  __global__ __launch_bounds__(kThreads) void name(const IN *x, OUT *out, uint32_t n) {                     \
+    cast_vec_body<Op, 4>(x, out, n);                                                                        \
+  }                                                                                                         \
+  __global__ __launch_bounds__(kThreads) void name##_unaligned(const IN *x, OUT *out, uint32_t n) {         \
+    cast_body<Op>(x, out, n);                                                                               \
+  }
+EW_CAST(ew_cast_f32_bf16, ToBf16, float, uint16_t)
+EW_CAST(ew_cast_f32_f16, ToF16, float, uint16_t)
+EW_CAST(ew_cast_i32_i16, ToI16, int, int16_t)
+EW_CAST(ew_cast_i32_i8, ToI8, int, int8_t)
 
 __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restrict__ x,
                                                           const float *__restrict__ y,

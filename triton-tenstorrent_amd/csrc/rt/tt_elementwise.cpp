@@ -163,11 +163,11 @@ int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_
 int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE, int32_t in_dtype,
                    int32_t out_dtype, const uint32_t grid[3], void *stream) {
   if (!props()) return fail(RT_ERR_NOT_INIT, "cast_kernel: call rt_init first");
-  const char *name = nullptr;
-  if (in_dtype == TT_F32 && out_dtype == TT_BF16) name = "ew_cast_f32_bf16";
-  else if (in_dtype == TT_F32 && out_dtype == TT_F16) name = "ew_cast_f32_f16";
-  else if (in_dtype == TT_I32 && out_dtype == TT_I16) name = "ew_cast_i32_i16";
-  else if (in_dtype == TT_I32 && out_dtype == TT_I8) name = "ew_cast_i32_i8";
+  const char *stem = nullptr;
+  if (in_dtype == TT_F32 && out_dtype == TT_BF16) stem = "ew_cast_f32_bf16";
+  else if (in_dtype == TT_F32 && out_dtype == TT_F16) stem = "ew_cast_f32_f16";
+  else if (in_dtype == TT_I32 && out_dtype == TT_I16) stem = "ew_cast_i32_i16";
+  else if (in_dtype == TT_I32 && out_dtype == TT_I8) stem = "ew_cast_i32_i8";
   else
     return fail(RT_ERR_UNSUPPORTED, "cast_kernel: dtype %d -> %d (fp32 -> bf16/fp16 and int32 -> int16/int8 exist)",
                 in_dtype, out_dtype);
@@ -178,6 +178,13 @@ int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_S
   if (!x || !out) return fail(RT_ERR_INVALID, "cast_kernel: null tensor pointer");
   if (reinterpret_cast<uintptr_t>(x) & 3) return fail(RT_ERR_INVALID, "cast_kernel: x must be 4-byte aligned");
   void *args[] = {&x, &out, &n_eff};
+  if (aligned16(x) && aligned16(out)) {
+    // one workgroup per run of kThreads * kUnroll 16-byte stores, plus the ragged end
+    const uint32_t per_item = out_dtype == TT_I8 ? 16 : 8, per_wg = kThreads * kUnroll * per_item;
+    return launch("elementwise", stem, dim3((uint32_t)cdiv64(n_eff, per_wg)), dim3(kThreads), 0, stream, args, 3);
+  }
+  char name[48];
+  snprintf(name, sizeof(name), "%s_unaligned", stem);
   return launch("elementwise", name, dim3(streaming_grid(n_eff, false)), dim3(kThreads), 0, stream, args, 3);
 }
 
