@@ -78,6 +78,66 @@ def test_matmul_ragged_shapes_strided_views_and_sentinel():
     assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
 
 
+# Shapes that are whole 32-deep K steps and 8-column chunks but not whole 256x256x128 macro tiles take the fast
+# kernel's clamping variant: rows / chunks past the edge are fetched from inside the matrix, K is padded with
+# steps of zeros, stores are clipped.
+RAGGED_SHAPES = [(33, 8, 32), (256, 256, 32), (260, 264, 160), (511, 520, 96), (1000, 1000, 992), (257, 1032, 4128),
+                 (4000, 4096, 1024)]
+
+
+@pytest.mark.parametrize("M,N,K_", RAGGED_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matmul_ragged_fast_path(M, N, K_, dtype):
+    a, b = _ab(M, N, K_, dtype, seed=M + N)
+    # C sits inside a larger buffer: the sentinel shows that nothing outside C[:M,:N] is written
+    cbuf = torch.full((M + 3, N + 16), 7.5, dtype=dtype, device="cuda")
+    c = cbuf[:M, :N]
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a.cuda(), b.cuda(), c))
+    K.matmul_kernel_tma[(K.cdiv(M, 64) * K.cdiv(N, 64), )](ad, bd, cd, M, N, K_, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64,
+                                                          BLOCK_SIZE_K=32, GROUP_SIZE_M=1, FP8_OUTPUT=False,
+                                                          WARP_SPECIALIZE=False)
+    assert rt.last_kernel_name() == f"gemm_ragged_{'bf16' if dtype == torch.bfloat16 else 'f16'}_epi0"
+    _check(c, a, b, BM=64, BN=64, BK=32)
+    assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
+
+
+def test_matmul_ragged_fast_path_exact_and_with_wild_values_next_door():
+    # small integers: bit for bit against the oracle.  The operands are views into larger buffers whose
+    # neighbouring rows and columns hold inf and NaN: whatever the clamped fetches and the padding steps
+    # read, none of it may reach C
+    g = torch.Generator().manual_seed(12)
+    M, N, K_ = 300, 328, 224
+    abuf = torch.full((M + 5, K_ + 8), float("nan"), dtype=torch.bfloat16)
+    bbuf = torch.full((K_ + 7, N + 8), float("inf"), dtype=torch.bfloat16)
+    abuf[:M, :K_] = torch.randint(-4, 5, (M, K_), generator=g).to(torch.bfloat16)
+    bbuf[:K_, :N] = torch.randint(-4, 5, (K_, N), generator=g).to(torch.bfloat16)
+    a, b = abuf.cuda()[:M, :K_], bbuf.cuda()[:K_, :N]
+    c = K.matmul_tma(a, b)
+    assert rt.last_kernel_name() == "gemm_ragged_bf16_epi0"
+    want = orc.matmul(bits(abuf[:M, :K_]), bits(bbuf[:K_, :N]), BM=64, BN=64, BK=64)
+    assert np.array_equal(bits(c), want)
+
+
+@pytest.mark.parametrize("epilogue", [None, "gelu", "bias_row", "leaky_relu"])
+def test_matmul_ragged_fast_path_epilogues(epilogue):
+    M, N, K_ = 390, 520, 160
+    a, b = _ab(M, N, K_, seed=21)
+    gen = torch.Generator().manual_seed(22)
+    if epilogue is None:
+        bias = torch.randn(M, N, generator=gen).to(torch.bfloat16)
+        okw = dict(bias=bits(bias), epi=orc.EPI_BIAS_FULL)
+    else:
+        bias = torch.randn(N, generator=gen) * 0.02
+        okw = dict(bias=bias.numpy(), epi={"gelu": orc.EPI_BIAS_ROW_GELU, "bias_row": orc.EPI_BIAS_ROW,
+                                          "leaky_relu": orc.EPI_LEAKY_RELU}[epilogue])
+        if epilogue == "leaky_relu":
+            okw.pop("bias")
+    c = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda(), epilogue=epilogue)
+    assert rt.last_kernel_name().startswith("gemm_ragged_bf16_epi")
+    ref = orc.from_bf16(orc.matmul(bits(a), bits(b), acc64=True, **okw))
+    assert close_bf16(decode(c), ref, RTOL, 1e-2 if epilogue is None else ATOL)
+
+
 def test_matmul_partial_grid_runs_only_its_programs():
     a, b = _ab(256, 256, 128)
     c = torch.full((256, 256), 7.5, dtype=torch.bfloat16, device="cuda")

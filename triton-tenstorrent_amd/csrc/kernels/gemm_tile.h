@@ -33,12 +33,21 @@
 // wide.  B fragments need k along the lane's registers while memory has n
 // contiguous: ds_read_b64_tr_b16 transposes a 4x16 block of 16-bit values
 // across each group of 16 lanes on the way out of LDS.
+//
+// RAGGED variant (M any, N a multiple of 8, K a multiple of 32): same kernel, three differences.  Rows of A
+// beyond M and 16-byte column chunks of B beyond N are fetched from the last valid row / chunk instead (their
+// products land in parts of the macro tile that are never stored); K is padded to whole turns of the ring
+// with steps whose A and B slabs are copied from a page of zeros (exact: 0 * 0 accumulates nothing, whatever
+// the real operands hold); and the stores are clipped at M and N.  The MFMA stream has no branch in it.
 #pragma once
 #include <type_traits>
 
 #include "gemm_common.h"
 
 namespace fast {
+
+// source of the zero steps of the RAGGED variant: 256 lanes x 16 bytes
+__device__ __attribute__((aligned(4096))) const uint8_t zero_page[4096] = {0};
 
 constexpr int BM = 256, BN = 256, BK = 32;
 constexpr int R = 4;                        // ring depth
@@ -93,16 +102,18 @@ struct Ring {
 // contiguous, i.e. exactly 32 of this kernel's 64-byte LDS rows, so only the global addresses
 // of the copies and of the result change: a thread's offset inside a slab, the distance
 // between slabs and between K steps.  LDS layout, fragments and MFMA schedule are the same.
-template <int IN_DT, int OUT_DT, int EPI, bool TILED = false>
+template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
+  static_assert(!(TILED && RAGGED), "tile-major operands come padded to whole tiles");
   using X = MFMA<IN_DT>;
   using vec = typename X::vec;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
   const int total = tiles_m * tiles_n;
-  const int nk = g.K / BK; // steps per tile, a multiple of R
+  const int nk_real = g.K / BK;                                   // steps that carry data
+  const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
   // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
   // A slab i (64 rows): row = i*64 + (t>>2), chunk position t&3 holds logical chunk (t&3)^((row>>2)&3)
@@ -191,18 +202,42 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // a_cur/b_cur point at the current tile's A rows / B columns, a_nxt/b_nxt at the next
   // tile's (or the current one again when there is none: a harmless refetch).
   const uint8_t *a_cur, *b_cur, *a_nxt, *b_nxt;
-  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp) {
+  // RAGGED: per-thread byte offsets of a tile's copies, rows and column chunks clamped into the matrix.
+  // The A offsets then carry the whole row offset from the tile's first row (a clamp can point backwards
+  // from a slab's own first row, and the instruction's register offset is unsigned).
+  struct Voffs { uint32_t a[4]; uint32_t b; };
+  Voffs vo_cur, vo_nxt;
+  const uint32_t z_voff = (uint32_t)tid * 16;
+  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
     int tm, tn;
     tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
     ap = A + (TILED ? (int64_t)tm * (BM / 32) * ntk * 2048 : (int64_t)tm * BM * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
+    if constexpr (RAGGED) {
+      const int last_row = g.M - 1 - tm * BM;                 // >= 0
+      const int last_chunk = (g.N - tn * BN) / 8 - 1;         // >= 0: N is a multiple of 8
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        vo.a[i] = (uint32_t)(((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 8) * 2);
+      vo.b = (uint32_t)(((int64_t)b_k * g.ldb + min(b_chunk, last_chunk) * 8) * 2);
+    }
   };
   // copy number i (0..3: A slabs, 4..7: B slabs) of step kk into `stage`; kk may run past
   // nk into the next tile
   auto dma_single = [&](int kk, uint8_t *stage, int i) {
     const bool over = kk >= nk;
     const int k = over ? kk - nk : kk;
-    if (i < 4) {
+    if constexpr (RAGGED) {
+      const bool zero = k >= nk_real;                         // a padding step: both operands are zeros
+      const Voffs &vo = over ? vo_nxt : vo_cur;
+      if (i < 4) {
+        const uint8_t *ap = zero ? zero_page : (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
+        dma_one(ap, zero ? z_voff : vo.a[i], stage + i * 4096);
+      } else {
+        const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - 4) * b_slab;
+        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - 4) * 4096);
+      }
+    } else if (i < 4) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
@@ -255,8 +290,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // ---- fill the ring: steps 0..R-1 of the first tile ----
   int t = blockIdx.x;
   if (t >= total) return;
-  tile_bases(t, a_cur, b_cur);
-  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt);
+  tile_bases(t, a_cur, b_cur, vo_cur);
+  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
   // steps 0..R-2 whole, and the first half of step R-1 (step 0's first sub-step issues the rest)
 #pragma unroll
   for (int s = 0; s < R; ++s)
@@ -285,9 +320,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // the ring already holds the next tile's first steps; move the tile window on
     a_cur = a_nxt;
     b_cur = b_nxt;
+    vo_cur = vo_nxt;
     {
       const int t2 = t + 2 * (int)gridDim.x;
-      tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt);
+      tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt, vo_nxt);
     }
 
     // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
@@ -302,7 +338,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4)
-          brow[j][r4] = *(const f32x4 *)((const float *)g.bias + n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4);
+          brow[j][r4] = *(const f32x4 *)((const float *)g.bias +
+                                         (RAGGED ? min(n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4, (int64_t)g.N - 4)
+                                                 : n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4));
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -312,6 +350,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
+          if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // N is a multiple of 8: the four columns stand or fall together
           float v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -365,6 +404,25 @@ extern "C" {
 
 GEMM_TILE_ALL_EPI(gemm_tile_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
+
+// the same kernels for M any, N % 8 == 0, K % 32 == 0
+#define GEMM_TILE_RAGGED(name, IN, OUT, EPI)                                                       \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
+    fast::body<IN, OUT, EPI, false, true>(g, ring);                                                 \
+  }
+#define GEMM_TILE_RAGGED_ALL_EPI(prefix, IN, OUT)             \
+  GEMM_TILE_RAGGED(prefix##_epi0, IN, OUT, EPI_NONE)           \
+  GEMM_TILE_RAGGED(prefix##_epi1, IN, OUT, EPI_BIAS_FULL)      \
+  GEMM_TILE_RAGGED(prefix##_epi2, IN, OUT, EPI_BIAS_ROW_GELU)  \
+  GEMM_TILE_RAGGED(prefix##_epi3, IN, OUT, EPI_LEAKY_RELU)     \
+  GEMM_TILE_RAGGED(prefix##_epi4, IN, OUT, EPI_BIAS_ROW)
+GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_bf16, DT_BF16, DT_BF16)
+GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
 
 // matmul_kernel on tile-major fp16 buffers, plain and with leaky_relu
 #define GEMM_TILED(name, EPI)                                                                      \

@@ -103,10 +103,14 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   const bool fast_shape = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
   const bool fast_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 8 == 0 &&
                           g.ldb % 8 == 0 && g.ldc % 8 == 0;
-  if (full_grid && half_io && fast_shape && fast_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+  // The same kernel with clamped fetches, zero-padded K steps and clipped stores takes every other shape
+  // whose rows can be fetched in 16-byte pieces and whose K is a whole number of 32-deep steps.
+  const bool ragged_shape = !fast_shape && N % 8 == 0 && K % 32 == 0 && g.lda < (1 << 23) && g.ldb < (1 << 23);
+  if (full_grid && half_io && (fast_shape || ragged_shape) && fast_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     char fast_name[64];
-    snprintf(fast_name, sizeof(fast_name), "gemm_tile_%s_epi%d", in == TT_BF16 ? "bf16" : "f16", epi);
-    const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+    snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
+             epi);
+    const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
     // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
