@@ -138,6 +138,24 @@ def test_matmul_ragged_fast_path_epilogues(epilogue):
     assert close_bf16(decode(c), ref, RTOL, 1e-2 if epilogue is None else ATOL)
 
 
+@pytest.mark.parametrize("M,N,K_", [(40, 16, 64), (300, 336, 192), (1000, 1008, 960), (4000, 4096, 1088)])
+def test_fp8_scaled_ragged_fast_path(M, N, K_):
+    g = torch.Generator().manual_seed(M)
+    x, w = torch.randn(M, K_, generator=g), torch.randn(K_, N, generator=g)
+    qa, sa = K.quantize_fp8(x)
+    qb, sb = K.quantize_fp8(w)
+    # operands are views into buffers whose surroundings are NaN codes (0x7f): none of it may reach C
+    abuf = torch.full((M + 2, K_ + 16), 0x7f, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    bbuf = torch.full((K_ + 2, N + 16), 0x7f, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    abuf[:M, :K_] = qa
+    bbuf[:K_, :N] = qb
+    c = K.matmul_fp8_scaled(abuf.cuda()[:M, :K_], bbuf.cuda()[:K_, :N], sa, sb)
+    assert rt.last_kernel_name() == "gemm_ragged_fp8_bf16"
+    ref = orc.from_bf16(orc.matmul(bits(qa), bits(qb), in_dt=orc.FP8E4M3, out_dt=orc.BF16,
+                                   scale=float(np.float32(sa) * np.float32(sb)), acc64=True))
+    assert close_bf16(decode(c), ref, RTOL, fp8_atol(ref))
+
+
 def test_matmul_partial_grid_runs_only_its_programs():
     a, b = _ab(256, 256, 128)
     c = torch.full((256, 256), 7.5, dtype=torch.bfloat16, device="cuda")

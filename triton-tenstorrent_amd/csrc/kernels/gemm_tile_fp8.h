@@ -34,14 +34,18 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
 typedef __attribute__((address_space(3))) void lds_void;
 
-template <int OUT_DT>
+// RAGGED (M any, N a multiple of 16, K a multiple of 64): as in the 16-bit kernel, fetches past the edges are
+// clamped into the matrix, K is padded to whole turns of the ring with steps copied from a page of zeros, and
+// the stores are clipped.
+template <int OUT_DT, bool RAGGED = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
   const int total = tiles_m * tiles_n;
-  const int nk = g.K / BK; // steps per tile, a multiple of R
+  const int nk_real = g.K / BK;                                   // steps that carry data
+  const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
   // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
   // A slab i (64 rows of 64 B): row = i*64 + (t>>2), position t&3 holds chunk (t&3)^((row>>2)&3)
@@ -104,16 +108,36 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
                  : "memory", "m0");
   };
   const uint8_t *a_cur, *b_cur, *a_nxt, *b_nxt;
-  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp) {
+  struct Voffs { uint32_t a[4]; uint32_t b; };   // RAGGED: a tile's per-thread offsets, clamped into the matrix
+  Voffs vo_cur, vo_nxt;
+  const uint32_t z_voff = (uint32_t)tid * 16;
+  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
     int tm, tn;
     fast::tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
     ap = A + (int64_t)tm * BM * g.lda;
     bp = B + (int64_t)tn * BN;
+    if constexpr (RAGGED) {
+      const int last_row = g.M - 1 - tm * BM;
+      const int last_chunk = (g.N - tn * BN) / 16 - 1;        // N is a multiple of 16
+#pragma unroll
+      for (int i = 0; i < 4; ++i) vo.a[i] = (uint32_t)((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 16);
+      vo.b = (uint32_t)((int64_t)b_k * g.ldb + min(b_chunk, last_chunk) * 16);
+    }
   };
   auto dma_single = [&](int kk, uint8_t *stage, int i) {
     const bool over = kk >= nk;
     const int k = over ? kk - nk : kk;
-    if (i < 4) {
+    if constexpr (RAGGED) {
+      const bool zero = k >= nk_real;
+      const Voffs &vo = over ? vo_nxt : vo_cur;
+      if (i < 4) {
+        const uint8_t *ap = zero ? fast::zero_page : (over ? a_nxt : a_cur) + (int64_t)k * BK;
+        dma_one(ap, zero ? z_voff : vo.a[i], stage + i * 4096);
+      } else {
+        const uint8_t *bp = zero ? fast::zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - 4) * b_slab;
+        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - 4) * 4096);
+      }
+    } else if (i < 4) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * BK;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
@@ -148,8 +172,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
   int t = blockIdx.x;
   if (t >= total) return;
-  tile_bases(t, a_cur, b_cur);
-  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt);
+  tile_bases(t, a_cur, b_cur, vo_cur);
+  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
   // fill the ring with steps 0..R-1
 #pragma unroll
   for (int s = 0; s < R; ++s)
@@ -175,9 +199,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     }
     a_cur = a_nxt;
     b_cur = b_nxt;
+    vo_cur = vo_nxt;
     {
       const int t2 = t + 2 * (int)gridDim.x;
-      tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt);
+      tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt, vo_nxt);
     }
     // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
     //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
@@ -190,6 +215,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
+          if (RAGGED && (mi >= g.M || n >= g.N)) continue;
           float v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[i][j][r4 * 4 + e] * g.scale;
@@ -224,5 +250,17 @@ extern "C" {
 
 GEMM_TILE_FP8(gemm_tile_fp8_bf16, DT_BF16)
 GEMM_TILE_FP8(gemm_tile_fp8_f16, DT_F16)
+
+#define GEMM_RAGGED_FP8(name, OUT)                                                                  \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast8::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast8::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                    \
+    fast8::body<OUT, true>(g, ring);                                                                 \
+  }
+GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16, DT_BF16)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_f16, DT_F16)
 
 } // extern "C"

@@ -135,12 +135,14 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   const bool fp8_shape = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
   const bool fp8_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 16 == 0 && g.ldb % 16 == 0 &&
                          g.ldc % 4 == 0;
-  if (full_grid && fp8_io && fp8_shape && fp8_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
-    const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+  const bool fp8_ragged = !fp8_shape && N % 16 == 0 && K % 64 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24);
+  if (full_grid && fp8_io && (fp8_shape || fp8_ragged) && fp8_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+    const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
     void *fargs[] = {&g};
-    return launch("gemm", out == TT_BF16 ? "gemm_tile_fp8_bf16" : "gemm_tile_fp8_f16", dim3(wgs), dim3(256), 0, stream,
-                  fargs, 1);
+    char fp8_name[48];
+    snprintf(fp8_name, sizeof(fp8_name), "gemm_%s_fp8_%s", fp8_shape ? "tile" : "ragged", out == TT_BF16 ? "bf16" : "f16");
+    return launch("gemm", fp8_name, dim3(wgs), dim3(256), 0, stream, fargs, 1);
   }
 
   const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
