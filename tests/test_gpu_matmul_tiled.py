@@ -34,6 +34,7 @@ def _close(got, ref):
     (70, 45, 50, {}),                                               # ragged in all three
     (128, 192, 96, {"BLOCK_SIZE_M": 64, "BLOCK_SIZE_N": 32, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 4}),
     (33, 31, 17, {"BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 64, "BLOCK_SIZE_K": 16}),
+    (257, 31, 33, {}), (300, 333, 200, {}), (1000, 1000, 1000, {}), (256, 256, 96, {}),   # the clamping fast kernel
 ])
 @pytest.mark.parametrize("act", ["", "leaky_relu"])
 def test_tiled_matmul_vs_oracle(M, N, K_, cfg, act):
@@ -43,7 +44,8 @@ def test_tiled_matmul_vs_oracle(M, N, K_, cfg, act):
     at, bt = K.tilize(a, BM, BK), K.tilize(b, BK, BN)
     assert np.array_equal(_bits(at), orc.tilize(_bits(a), BM, BK))          # same tiling as the oracle's
     ct = K.matmul_tiled(at.cuda(), bt.cuda(), M, N, K_, activation=act, **cfg)
-    assert rt.last_kernel_name() == "gemm_anytiled_f16_f16"
+    # the reference's 32x32x32 tiling takes the fast kernel's clamping instantiation, other tilings the any-shape one
+    assert rt.last_kernel_name() == (f"gemm_tiledragged_f16_epi{3 if act else 0}" if not cfg else "gemm_anytiled_f16_f16")
     ref = orc.matmul_tiled(_bits(at), _bits(bt), M, N, K_, in_dt=orc.F16, BM=BM, BN=BN, BK=BK,
                            group_m=c["GROUP_SIZE_M"], leaky_relu=bool(act), acc64=True)
     got = _bits(ct.cpu())

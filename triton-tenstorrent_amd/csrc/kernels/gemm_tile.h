@@ -104,7 +104,11 @@ struct Ring {
 // between slabs and between K steps.  LDS layout, fragments and MFMA schedule are the same.
 template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
-  static_assert(!(TILED && RAGGED), "tile-major operands come padded to whole tiles");
+  // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
+  // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
+  // real M and N (the padding of C is never written, as under the reference's store mask).
+  const int Mf = TILED ? (g.M + 31) / 32 * 32 : g.M, Nf = TILED ? (g.N + 31) / 32 * 32 : g.N;   // fetchable extent
+  const int Kf = TILED ? (g.K + 31) / 32 * 32 : g.K;
   using X = MFMA<IN_DT>;
   using vec = typename X::vec;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -112,7 +116,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
   const int total = tiles_m * tiles_n;
-  const int nk_real = g.K / BK;                                   // steps that carry data
+  const int nk_real = Kf / BK;                                    // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
   // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
@@ -125,7 +129,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // row-major:  A(m,k) at m*lda + k,  B(k,n) at k*ldb + n
   // tile-major: A(m,k) at ((m/32)*ntk + k/32)*1024 + (m%32)*32 + k%32,
   //             B(k,n) at ((k/32)*ntn + n/32)*1024 + (k%32)*32 + n%32          (elements)
-  const int64_t ntk = g.K / 32, ntn = g.N / 32;
+  const int64_t ntk = Kf / 32, ntn = Nf / 32;
   const uint32_t a_voff = TILED ? (uint32_t)((((int64_t)(a_row >> 5) * ntk << 10) + (a_row & 31) * 32 + a_chunk * 8) * 2)
                                 : (uint32_t)(((int64_t)a_row * g.lda + a_chunk * 8) * 2); // bytes, per thread
   const uint32_t b_voff = TILED ? (uint32_t)((((b_chunk >> 2) << 10) + b_k * 32 + (b_chunk & 3) * 8) * 2)
@@ -214,12 +218,17 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     ap = A + (TILED ? (int64_t)tm * (BM / 32) * ntk * 2048 : (int64_t)tm * BM * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
     if constexpr (RAGGED) {
-      const int last_row = g.M - 1 - tm * BM;                 // >= 0
-      const int last_chunk = (g.N - tn * BN) / 8 - 1;         // >= 0: N is a multiple of 8
+      const int last_row = Mf - 1 - tm * BM;                  // >= 0
+      const int last_chunk = (Nf - tn * BN) / 8 - 1;          // >= 0: the fetchable N is a multiple of 8
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        vo.a[i] = (uint32_t)(((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 8) * 2);
-      vo.b = (uint32_t)(((int64_t)b_k * g.ldb + min(b_chunk, last_chunk) * 8) * 2);
+      for (int i = 0; i < 4; ++i) {
+        const int r = min(i * 64 + a_row, last_row);
+        vo.a[i] = TILED ? (uint32_t)((((int64_t)(r >> 5) * ntk << 10) + (r & 31) * 32 + a_chunk * 8) * 2)
+                        : (uint32_t)(((int64_t)r * g.lda + a_chunk * 8) * 2);
+      }
+      const int cc = min(b_chunk, last_chunk);
+      vo.b = TILED ? (uint32_t)((((cc >> 2) << 10) + b_k * 32 + (cc & 3) * 8) * 2)
+                   : (uint32_t)(((int64_t)b_k * g.ldb + cc * 8) * 2);
     }
   };
   // copy number i (0..3: A slabs, 4..7: B slabs) of step kk into `stage`; kk may run past
@@ -350,7 +359,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
-          if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // N is a multiple of 8: the four columns stand or fall together
+          if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // row-major: N is a multiple of 8, the four columns stand or fall together
           float v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -370,6 +379,11 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                          (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
           }
           const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
+          if (TILED && RAGGED && n + 3 >= g.N) {               // N is anything here: the last group goes by element
+            for (int e = 0; e < 4 && n + e < g.N; ++e)
+              ((uint16_t *)g.c)[coff + e] = (uint16_t)(e & 1 ? pk[e >> 1] >> 16 : pk[e >> 1] & 0xffffu);
+            continue;
+          }
           *(u32x2 *)((uint16_t *)g.c + coff) = pk;
         }
       }
@@ -436,5 +450,18 @@ GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
   }
 GEMM_TILED(gemm_tiled_f16_epi0, EPI_NONE)
 GEMM_TILED(gemm_tiled_f16_epi3, EPI_LEAKY_RELU)
+
+// the same for any M, N, K (buffers padded to whole 32x32 tiles)
+#define GEMM_TILED_RAGGED(name, EPI)                                                               \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
+    fast::body<DT_F16, DT_F16, EPI, true, true>(g, ring);                                           \
+  }
+GEMM_TILED_RAGGED(gemm_tiledragged_f16_epi0, EPI_NONE)
+GEMM_TILED_RAGGED(gemm_tiledragged_f16_epi3, EPI_LEAKY_RELU)
 
 } // extern "C"

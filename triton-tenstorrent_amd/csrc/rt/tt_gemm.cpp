@@ -225,16 +225,18 @@ int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t 
   g.tiled = 1;
   void *args[] = {&g};
 
-  // Fast path: 32x32x32 tiles (the reference's configuration), whole 256x256x128 macro
-  // tiles, fp16, 16-byte aligned buffers, a grid that covers the problem.
+  // Fast path: 32x32x32 tiles (the reference's configuration), fp16, 16-byte aligned buffers, a grid that
+  // covers the problem.  Whole 256x256x128 macro tiles take the plain kernel, everything else its clamping
+  // instantiation (the buffers are padded to whole 32x32 tiles, which is all it needs).
   const bool full_grid = (int64_t)grid[0] == num_pid_m * num_pid_n;
-  if (full_grid && in_dtype == TT_F16 && BM == 32 && BN == 32 && BK == 32 && M % 256 == 0 && N % 256 == 0 &&
-      K % 128 == 0 && K >= 128 && aligned16(a_ptr) && aligned16(b_ptr) && aligned16(c_ptr) &&
-      !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
-    const int64_t tiles = (int64_t)(M / 256) * (N / 256);
+  if (full_grid && in_dtype == TT_F16 && BM == 32 && BN == 32 && BK == 32 && aligned16(a_ptr) && aligned16(b_ptr) &&
+      aligned16(c_ptr) && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+    const bool whole = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
+    const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
-    return launch("gemm", leaky_relu ? "gemm_tiled_f16_epi3" : "gemm_tiled_f16_epi0", dim3(wgs), dim3(256), 0, stream,
-                  args, 1);
+    char name[48];
+    snprintf(name, sizeof(name), "gemm_tiled%s_f16_epi%d", whole ? "" : "ragged", leaky_relu ? 3 : 0);
+    return launch("gemm", name, dim3(wgs), dim3(256), 0, stream, args, 1);
   }
   const int64_t items = (int64_t)grid[0] * (BM / 32) * (BN / 32);
   const int64_t cap = (int64_t)props()->multiprocessor_count * 8;
