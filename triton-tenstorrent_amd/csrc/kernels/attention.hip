@@ -220,7 +220,11 @@ typedef __attribute__((address_space(3))) void lds_void;
 
 constexpr int WAVES = 8, BM = WAVES * 32, BN = 64;
 
-template <int D>
+// RAGGED: N_CTX a multiple of 32 but not of 256.  A wavefront is then either wholly inside the sequence or
+// wholly outside it (it computes and stores nothing, but keeps up with the barriers and its share of the copies);
+// the last key block may hold 32 keys only: its copies fetch the rows past N_CTX from the last row instead, the
+// second 32-key tile is left out of both products and its scores count as -inf.
+template <int D, bool RAGGED = false>
 __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *lds1) {
   constexpr int DK = D / 16;            // k-steps of S^T
   constexpr int DT = D / 32;            // 32-row tiles of O^T
@@ -235,7 +239,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   const int c32 = lane & 31, hi = lane >> 5;
 
   // ---- which (head, query block) ----
-  const int qblocks = a.rows / BM;
+  const int qblocks = RAGGED ? (a.rows + BM - 1) / BM : a.rows / BM;
   const int total = qblocks * a.heads;
   int id = blockIdx.x;
   if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
@@ -246,8 +250,9 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   const int my_q = qw + c32;
   const int64_t base = (int64_t)head * a.n_ctx;
   const float qk_scale = a.sm_scale * 1.44269504f;
-  const int n_end = a.causal ? q0 + BM : a.n_ctx;
-  const int nblk = n_end / BN;
+  const int n_end = a.causal ? (RAGGED ? min(q0 + BM, a.n_ctx) : q0 + BM) : a.n_ctx;
+  const int nblk = RAGGED ? (n_end + BN - 1) / BN : n_end / BN;
+  const bool live = !RAGGED || qw < a.n_ctx;   // wave-uniform
 
   // ---- global -> LDS copy constants ----
   // Only wavefronts 4-7 copy, thread t - 256 owning byte 16*(t - 256) of each slab: a copy instruction
@@ -274,6 +279,21 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   auto dma_block = [&](int blk, uint8_t *stage) { // K tile then V tile of key block blk
     if (wave < 4) return;
     const int64_t row0 = (int64_t)blk * BN;
+    if (RAGGED && row0 + BN > a.n_ctx) {
+      // the half block at the end of the sequence: rows past it are fetched from its last row
+      const int last = a.n_ctx - 1 - (int)row0;
+#pragma unroll
+      for (int i = 0; i < NSLAB; ++i) {
+        const int r = min(i * (SLAB / ROW) + crow, last);
+        dma_one(kg + row0 * a.ldk * 2, (uint32_t)(((int64_t)r * a.ldk + k_chunk * 8) * 2), stage + i * SLAB);
+      }
+#pragma unroll
+      for (int i = 0; i < NSLAB; ++i) {
+        const int r = min(i * (SLAB / ROW) + crow, last);
+        dma_one(vg + row0 * a.ldv * 2, (uint32_t)(((int64_t)r * a.ldv + v_chunk * 8) * 2), stage + TILE + i * SLAB);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < NSLAB; ++i)
       dma_one(kg + (row0 + i * (SLAB / ROW)) * a.ldk * 2, k_voff, stage + i * SLAB);
@@ -296,7 +316,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   // ---- Q fragments (B operand of S^T), straight from global ----
   union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; uint32_t w[4]; };
   Frag qf[DK];
-  {
+  if (live) {
     const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
 #pragma unroll
     for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
@@ -319,13 +339,19 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     if (b + 1 < nblk) dma_block(b + 1, nxt);
     const int n0 = b * BN;
-    if (a.causal && n0 > qw + 31) continue; // wholly above this wavefront's diagonal (wave-uniform)
+    if (!live || (a.causal && n0 > qw + 31)) continue; // outside the sequence, or wholly above this wavefront's diagonal
+    const bool both = !RAGGED || n0 + 32 < n_end;      // the block's second 32-key tile exists (wave-uniform)
 
     // ---- S^T = K . Q^T : two 32-key tiles ----
     f32x16 st[2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       st[kt] = (f32x16){0};
+      if (RAGGED && kt == 1 && !both) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[1][r] = -__builtin_inff();
+        break;
+      }
       const uint8_t *kb = cur + kt * 32 * ROW + k_rowoff;
 #pragma unroll
       for (int s = 0; s < DK; ++s) {
@@ -406,6 +432,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     const uint8_t *vb = cur + TILE;
 #pragma unroll
     for (int k4 = 0; k4 < 4; ++k4) {
+      if (RAGGED && k4 == 2 && !both) break;           // P is zero there; leave the clamped V rows out altogether
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
         Frag vf;
@@ -429,6 +456,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 1);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (!live) return;
   // ---- epilogue ----
   if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
   uint16_t *orow = a.o + (base + my_q) * a.ldo;
@@ -456,5 +484,14 @@ extern "C" {
   }
 ATTN_TILE(64)
 ATTN_TILE(128)
+
+#define ATTN_RAGGED(D)                                                                     \
+  __global__ __launch_bounds__(512) void attn_ragged_d##D(AttnArgs a) {                    \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[2 * 64 * D * 2];                \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
+    fastattn::body<D, true>(a, lds0, lds1);                                                \
+  }
+ATTN_RAGGED(64)
+ATTN_RAGGED(128)
 
 } // extern "C"

@@ -1,5 +1,6 @@
 // tt_attn_fwd: launch validation and kernel selection for fused attention.
 #include <algorithm>
+#include <cstdio>
 #include <cstring>
 
 #include "tt_internal.h"
@@ -60,15 +61,17 @@ extern "C" int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const
   a.ldo = desc_o->strides[0];
   a.n_ctx = N_CTX; a.rows = (int32_t)(grid[0] * (int64_t)BLOCK_M); a.heads = (int32_t)grid[1];
   a.causal = STAGE == 3; a.sm_scale = sm_scale;
-  // Fast path: whole 256-row query blocks of every head, 16-byte aligned rows.
+  // Fast path: every query of every head, 16-byte aligned rows, N_CTX in whole wavefronts of 32 queries.
+  // Whole 256-query blocks take the plain kernel, other lengths its instantiation with a clipped tail.
   const bool full = (int64_t)grid[0] * BLOCK_M == N_CTX && (int64_t)grid[1] == (int64_t)Z * H;
   const bool al = aligned16(a.q) && aligned16(a.k) && aligned16(a.v) && aligned16(a.o) && a.ldq % 8 == 0 &&
                   a.ldk % 8 == 0 && a.ldv % 8 == 0 && a.ldo % 4 == 0;
-  if (full && al && N_CTX % 256 == 0 && (HEAD_DIM == 64 || HEAD_DIM == 128) && !env_int("TTAMD_ATTN_FORCE_ANY", 0)) {
+  if (full && al && N_CTX % 32 == 0 && (HEAD_DIM == 64 || HEAD_DIM == 128) && !env_int("TTAMD_ATTN_FORCE_ANY", 0)) {
     void *fargs[] = {&a};
-    const uint32_t wgs = (uint32_t)((N_CTX / 256) * (int64_t)Z * H);
-    return launch("attention", HEAD_DIM == 128 ? "attn_tile_d128" : "attn_tile_d64", dim3(wgs), dim3(512), 0, stream,
-                  fargs, 1);
+    const uint32_t wgs = (uint32_t)(cdiv64(N_CTX, 256) * (int64_t)Z * H);
+    char name[32];
+    snprintf(name, sizeof(name), "attn_%s_d%d", N_CTX % 256 == 0 ? "tile" : "ragged", HEAD_DIM);
+    return launch("attention", name, dim3(wgs), dim3(512), 0, stream, fargs, 1);
   }
   const char *name = nullptr;
   switch (HEAD_DIM) {

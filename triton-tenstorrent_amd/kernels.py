@@ -321,8 +321,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, causal: bool, s
     desc_v = TensorDescriptor(v, shape=[y_dim, HEAD_DIM_K], strides=[HEAD_DIM_K, 1], block_shape=dummy_block)
     desc_k = TensorDescriptor(k, shape=[y_dim, HEAD_DIM_K], strides=[HEAD_DIM_K, 1], block_shape=dummy_block)
     desc_o = TensorDescriptor(o, shape=[y_dim, HEAD_DIM_K], strides=[HEAD_DIM_K, 1], block_shape=dummy_block)
-    if "BLOCK_M" not in meta and q.shape[2] < 128:
-        meta["BLOCK_M"] = 32 if q.shape[2] % 64 else 64
+    if "BLOCK_M" not in meta and q.shape[2] % 128:
+        meta["BLOCK_M"] = 32 if q.shape[2] % 64 else 64      # the largest of the reference's block sizes that divides N_CTX
     if "BLOCK_N" not in meta:
         meta["BLOCK_N"] = min(meta.get("BLOCK_M", 128), 64, HEAD_DIM_K)
 
