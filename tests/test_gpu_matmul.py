@@ -234,6 +234,19 @@ def test_fp8_inputs_fp8_output_unscaled():
     assert np.max(np.abs(orc.from_fp8(got) - orc.from_fp8(want))) <= 0.125 * np.max(np.abs(orc.from_fp8(want)))
 
 
+@pytest.mark.parametrize("M,N,K_", [(256, 256, 256), (512, 768, 512), (300, 336, 192)])
+def test_fp8_output_fast_path_exact_on_small_integers(M, N, K_):
+    # FP8_OUTPUT (09-persistent-matmul.py:116,173) on the fast kernel: exact sums, one rounding to e4m3 (saturating)
+    g = torch.Generator().manual_seed(M + K_)
+    a = torch.randint(-2, 3, (M, K_), generator=g).float().to(torch.float8_e4m3fn)
+    b = torch.randint(-2, 3, (K_, N), generator=g).float().to(torch.float8_e4m3fn)
+    c = K.matmul_tma(a.cuda(), b.cuda())
+    assert c.dtype == torch.float8_e4m3fn
+    assert rt.last_kernel_name() == ("gemm_tile_fp8_fp8" if M % 256 == 0 and N % 256 == 0 and K_ % 256 == 0 else "gemm_ragged_fp8_fp8")
+    want = orc.matmul(bits(a), bits(b), in_dt=orc.FP8E4M3, out_dt=orc.FP8E4M3, acc64=True)
+    assert np.array_equal(bits(c), want)
+
+
 def test_matmul_errors():
     a, b = _ab(64, 64, 64)
     with pytest.raises(NotImplementedError):

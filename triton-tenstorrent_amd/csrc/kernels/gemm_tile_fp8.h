@@ -219,6 +219,13 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
           float v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[i][j][r4 * 4 + e] * g.scale;
+          if constexpr (OUT_DT == DT_FP8) {
+            // FP8_OUTPUT (09-persistent-matmul.py:116,173): four e4m3 codes, one 4-byte store
+            const uint32_t q = (uint32_t)f32_to_fp8(v[0]) | ((uint32_t)f32_to_fp8(v[1]) << 8) |
+                               ((uint32_t)f32_to_fp8(v[2]) << 16) | ((uint32_t)f32_to_fp8(v[3]) << 24);
+            *(uint32_t *)((uint8_t *)g.c + mi * g.ldc + n) = q;
+            continue;
+          }
           u32x2 pk;
           if constexpr (OUT_DT == DT_BF16) {
             pk = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
@@ -250,6 +257,7 @@ extern "C" {
 
 GEMM_TILE_FP8(gemm_tile_fp8_bf16, DT_BF16)
 GEMM_TILE_FP8(gemm_tile_fp8_f16, DT_F16)
+GEMM_TILE_FP8(gemm_tile_fp8_fp8, DT_FP8)
 
 #define GEMM_RAGGED_FP8(name, OUT)                                                                  \
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
@@ -262,5 +270,6 @@ GEMM_TILE_FP8(gemm_tile_fp8_f16, DT_F16)
   }
 GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16, DT_BF16)
 GEMM_RAGGED_FP8(gemm_ragged_fp8_f16, DT_F16)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_fp8, DT_FP8)
 
 } // extern "C"

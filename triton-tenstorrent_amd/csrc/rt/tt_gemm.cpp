@@ -131,7 +131,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   }
 
   // fp8 fast path: e4m3 in, bf16/fp16 out, scale in the epilogue, K in steps of 64 through a 4-stage ring
-  const bool fp8_io = in == TT_FP8E4M3 && (out == TT_BF16 || out == TT_F16) && epi == TT_EPI_NONE;
+  const bool fp8_io = in == TT_FP8E4M3 && (out == TT_BF16 || out == TT_F16 || out == TT_FP8E4M3) && epi == TT_EPI_NONE;
   const bool fp8_shape = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
   const bool fp8_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 16 == 0 && g.ldb % 16 == 0 &&
                          g.ldc % 4 == 0;
@@ -141,7 +141,8 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
     void *fargs[] = {&g};
     char fp8_name[48];
-    snprintf(fp8_name, sizeof(fp8_name), "gemm_%s_fp8_%s", fp8_shape ? "tile" : "ragged", out == TT_BF16 ? "bf16" : "f16");
+    snprintf(fp8_name, sizeof(fp8_name), "gemm_%s_fp8_%s", fp8_shape ? "tile" : "ragged",
+             out == TT_BF16 ? "bf16" : out == TT_F16 ? "f16" : "fp8");
     return launch("gemm", fp8_name, dim3(wgs), dim3(256), 0, stream, fargs, 1);
   }
 
