@@ -218,19 +218,23 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 typedef __attribute__((address_space(3))) void lds_void;
 
-constexpr int WAVES = 8, BM = WAVES * 32, BN = 64;
+constexpr int BN = 64;
 
 // RAGGED: N_CTX a multiple of 32 but not of 256.  A wavefront is then either wholly inside the sequence or
 // wholly outside it (it computes and stores nothing, but keeps up with the barriers and its share of the copies);
 // the last key block may hold 32 keys only: its copies fetch the rows past N_CTX from the last row instead, the
 // second 32-key tile is left out of both products and its scores count as -inf.
-template <int D, bool RAGGED = false>
+//
+// WAVES = 4 (head dim 256): 128 queries per workgroup, one wavefront per SIMD with the whole register file
+// (O^T alone is 128 registers and Q 64 at that head dim), and all four wavefronts share the copies.
+template <int D, bool RAGGED = false, int WAVES = 8>
 __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *lds1) {
+  constexpr int BM = WAVES * 32;
   constexpr int DK = D / 16;            // k-steps of S^T
   constexpr int DT = D / 32;            // 32-row tiles of O^T
   constexpr int ROW = D * 2;            // bytes per K/V row
   constexpr int CH = D / 8;             // 16-byte chunks per row
-  constexpr int RPB = 256 / ROW;        // rows per 256 bytes (1 for D=128, 2 for D=64)
+  constexpr int RPB = ROW >= 256 ? 1 : 256 / ROW;   // rows per 256 bytes (1 for D >= 128, 2 for D=64, 4 for D=32)
   constexpr int TILE = BN * ROW;        // bytes of one K (or V) tile
   constexpr int SLAB = 256 * 16;        // bytes one pass of the four copying wavefronts moves
   constexpr int NSLAB = TILE / SLAB;    // 4 for D=128, 2 for D=64
@@ -261,10 +265,19 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   // slab i covers rows i*(SLAB/ROW) ..; row = i*(SLAB/ROW) + t/CH, position t%CH
   const int ctid = tid & 255;
   const int crow = ctid / CH, cpos = ctid % CH;
-  const int k_chunk = cpos ^ ((crow / RPB) & (CH - 1));
-  const int v_swz = (D == 128) ? (crow & 3) : ((crow >> 1) & 1);
+  // the K swizzle follows the row's index in the tile; with 512-byte rows (D = 256) a slab holds 8 rows only, so
+  // the chunk a thread fetches differs between slabs: NV variants, slab i uses variant i % NV
+  constexpr int RPS = SLAB / ROW;                               // rows per slab
+  constexpr int NV = (CH * RPB > RPS) ? (CH * RPB) / RPS : 1;   // 4 for D=256, else 1
+  const int v_swz = (D >= 128) ? (crow & 3) : (D == 64) ? ((crow >> 1) & 1) : 0;   // D = 32: a row is the whole window
   const int v_chunk = cpos ^ (v_swz << 2);
-  const uint32_t k_voff = (uint32_t)(((int64_t)crow * a.ldk + k_chunk * 8) * 2);
+  int k_chunks[NV];
+  uint32_t k_voffs[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    k_chunks[j] = cpos ^ (((j * RPS + crow) / RPB) & (CH - 1));
+    k_voffs[j] = (uint32_t)(((int64_t)crow * a.ldk + k_chunks[j] * 8) * 2);
+  }
   const uint32_t v_voff = (uint32_t)(((int64_t)crow * a.ldv + v_chunk * 8) * 2);
   const int lds_wave = (wave & 3) * 1024;
   const uint8_t *kg = (const uint8_t *)(a.k + base * a.ldk);
@@ -277,7 +290,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
                  : "memory", "m0");
   };
   auto dma_block = [&](int blk, uint8_t *stage) { // K tile then V tile of key block blk
-    if (wave < 4) return;
+    if (WAVES == 8 && wave < 4) return;
     const int64_t row0 = (int64_t)blk * BN;
     if (RAGGED && row0 + BN > a.n_ctx) {
       // the half block at the end of the sequence: rows past it are fetched from its last row
@@ -285,7 +298,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
 #pragma unroll
       for (int i = 0; i < NSLAB; ++i) {
         const int r = min(i * (SLAB / ROW) + crow, last);
-        dma_one(kg + row0 * a.ldk * 2, (uint32_t)(((int64_t)r * a.ldk + k_chunk * 8) * 2), stage + i * SLAB);
+        dma_one(kg + row0 * a.ldk * 2, (uint32_t)(((int64_t)r * a.ldk + k_chunks[i % NV] * 8) * 2), stage + i * SLAB);
       }
 #pragma unroll
       for (int i = 0; i < NSLAB; ++i) {
@@ -296,7 +309,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     }
 #pragma unroll
     for (int i = 0; i < NSLAB; ++i)
-      dma_one(kg + (row0 + i * (SLAB / ROW)) * a.ldk * 2, k_voff, stage + i * SLAB);
+      dma_one(kg + (row0 + i * (SLAB / ROW)) * a.ldk * 2, k_voffs[i % NV], stage + i * SLAB);
 #pragma unroll
     for (int i = 0; i < NSLAB; ++i)
       dma_one(vg + (row0 + i * (SLAB / ROW)) * a.ldv * 2, v_voff, stage + TILE + i * SLAB);
@@ -439,7 +452,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
           const int key = k4 * 16 + h2 * 8 + v_key; // row in the tile
-          const int swz = (D == 128) ? (key & 3) : ((key >> 1) & 1);
+          const int swz = (D >= 128) ? (key & 3) : (D == 64) ? ((key >> 1) & 1) : 0;
           const int chunk = (t * 4 + v_cc) ^ (swz << 2);
           vf.h[h2] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(vb + key * ROW + (chunk << 4) + v_half));
         }
@@ -482,6 +495,7 @@ extern "C" {
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
     fastattn::body<D>(a, lds0, lds1);                                                      \
   }
+ATTN_TILE(32)
 ATTN_TILE(64)
 ATTN_TILE(128)
 
@@ -491,7 +505,18 @@ ATTN_TILE(128)
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
     fastattn::body<D, true>(a, lds0, lds1);                                                \
   }
+ATTN_RAGGED(32)
 ATTN_RAGGED(64)
 ATTN_RAGGED(128)
+
+// head dim 256: four wavefronts, 128 queries per workgroup
+#define ATTN_TILE4(name, D, RAGGED)                                                        \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(AttnArgs a) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[2 * 64 * D * 2];                \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
+    fastattn::body<D, RAGGED, 4>(a, lds0, lds1);                                           \
+  }
+ATTN_TILE4(attn_tile_d256, 256, false)
+ATTN_TILE4(attn_ragged_d256, 256, true)
 
 } // extern "C"

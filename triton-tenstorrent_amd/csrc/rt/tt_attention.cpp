@@ -66,12 +66,14 @@ extern "C" int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const
   const bool full = (int64_t)grid[0] * BLOCK_M == N_CTX && (int64_t)grid[1] == (int64_t)Z * H;
   const bool al = aligned16(a.q) && aligned16(a.k) && aligned16(a.v) && aligned16(a.o) && a.ldq % 8 == 0 &&
                   a.ldk % 8 == 0 && a.ldv % 8 == 0 && a.ldo % 4 == 0;
-  if (full && al && N_CTX % 32 == 0 && (HEAD_DIM == 64 || HEAD_DIM == 128) && !env_int("TTAMD_ATTN_FORCE_ANY", 0)) {
+  if (full && al && N_CTX % 32 == 0 && (HEAD_DIM == 32 || HEAD_DIM == 64 || HEAD_DIM == 128 || HEAD_DIM == 256) &&
+      !env_int("TTAMD_ATTN_FORCE_ANY", 0)) {
     void *fargs[] = {&a};
-    const uint32_t wgs = (uint32_t)(cdiv64(N_CTX, 256) * (int64_t)Z * H);
+    const int queries = HEAD_DIM == 256 ? 128 : 256;   // per workgroup: 4 or 8 wavefronts of 32
+    const uint32_t wgs = (uint32_t)(cdiv64(N_CTX, queries) * (int64_t)Z * H);
     char name[32];
-    snprintf(name, sizeof(name), "attn_%s_d%d", N_CTX % 256 == 0 ? "tile" : "ragged", HEAD_DIM);
-    return launch("attention", name, dim3(wgs), dim3(512), 0, stream, fargs, 1);
+    snprintf(name, sizeof(name), "attn_%s_d%d", N_CTX % queries == 0 ? "tile" : "ragged", HEAD_DIM);
+    return launch("attention", name, dim3(wgs), dim3(2 * queries), 0, stream, fargs, 1);
   }
   const char *name = nullptr;
   switch (HEAD_DIM) {
