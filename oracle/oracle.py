@@ -12,7 +12,6 @@ the oracle itself uses.
 from __future__ import annotations
 
 import ctypes as C
-import os
 import subprocess
 from pathlib import Path
 

@@ -12,7 +12,7 @@ import ctypes as C
 import functools
 import json
 import time
-from typing import Any, Callable
+from typing import Callable
 
 from .. import runtime as rt
 from ..tensor_descriptor import is_tensor_descriptor

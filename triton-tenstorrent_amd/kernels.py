@@ -9,7 +9,6 @@ in the same order; host wrappers mirror the reference's own
 """
 from __future__ import annotations
 
-import math
 
 import torch
 
