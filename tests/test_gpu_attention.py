@@ -122,6 +122,26 @@ def test_fast_attention_ragged_sequence_lengths(causal, Z, H, S, D):
     assert np.max(np.abs(M.cpu().numpy() - wM)) <= M_ATOL
 
 
+def test_fast_attention_random_lengths_and_head_dims():
+    # a seeded sweep: N_CTX any multiple of 32 up to 800, every head dim of the fast kernel, both mask modes
+    from triton_tenstorrent_amd import runtime as rt
+    rng = np.random.default_rng(31)
+    for case in range(16):
+        D = int(rng.choice([32, 64, 128, 256]))
+        S = 32 * int(rng.integers(1, 26))
+        Z, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+        causal = bool(case % 2)
+        q, k, v = _qkv(Z, H, S, D, seed=100 + case)
+        sm = D ** -0.5
+        o, M = K.attention(q.cuda(), k.cuda(), v.cuda(), causal, sm, return_lse=True)
+        per_wg = 128 if D == 256 else 256
+        assert rt.last_kernel_name() == f"attn_{'tile' if S % per_wg == 0 else 'ragged'}_d{D}", (S, D)
+        bm = 128 if S % 128 == 0 else (64 if S % 64 == 0 else 32)
+        wo, wM = orc.attn_fwd(bits(q), bits(k), bits(v), sm, causal=causal, BLOCK_M=bm, BLOCK_N=min(bm, 64, D))
+        assert np.max(np.abs(decode(o) - orc.from_bf16(wo))) <= O_ATOL, (Z, H, S, D, causal)
+        assert np.max(np.abs(M.cpu().numpy() - wM)) <= M_ATOL, (Z, H, S, D, causal)
+
+
 def test_fast_attention_closed_forms_and_any_path_agreement():
     import os
     from triton_tenstorrent_amd import runtime as rt

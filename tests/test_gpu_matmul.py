@@ -101,6 +101,33 @@ def test_matmul_ragged_fast_path(M, N, K_, dtype):
     assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
 
 
+def test_matmul_ragged_fast_path_random_shapes_exact():
+    # a seeded sweep over shapes (M anything, N in steps of 8, K in steps of 32), small integers: bit for bit, with
+    # a sentinel frame around C and NaN frames around A and B
+    rng = np.random.default_rng(2025)
+    for case in range(24):
+        M = int(rng.integers(1, 700))
+        N = 8 * int(rng.integers(1, 90))
+        K_ = 32 * int(rng.integers(1, 12))
+        dtype = torch.bfloat16 if case % 2 else torch.float16
+        g = torch.Generator().manual_seed(case)
+        abuf = torch.full((M + 2, K_ + 8), float("nan"), dtype=dtype)
+        bbuf = torch.full((K_ + 2, N + 8), float("nan"), dtype=dtype)
+        abuf[:M, :K_] = torch.randint(-3, 4, (M, K_), generator=g).to(dtype)
+        bbuf[:K_, :N] = torch.randint(-3, 4, (K_, N), generator=g).to(dtype)
+        cbuf = torch.full((M + 2, N + 8), 7.5, dtype=dtype, device="cuda")
+        c = cbuf[:M, :N]
+        ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (abuf.cuda()[:M, :K_], bbuf.cuda()[:K_, :N], c))
+        K.matmul_kernel_tma[(K.cdiv(M, 32) * K.cdiv(N, 32), )](ad, bd, cd, M, N, K_, BLOCK_SIZE_M=32, BLOCK_SIZE_N=32,
+                                                              BLOCK_SIZE_K=32, GROUP_SIZE_M=1, FP8_OUTPUT=False,
+                                                              WARP_SPECIALIZE=False)
+        whole = M % 256 == 0 and N % 256 == 0 and K_ % 128 == 0
+        assert rt.last_kernel_name().startswith("gemm_tile_" if whole else "gemm_ragged_"), (M, N, K_)
+        want = abuf[:M, :K_].float() @ bbuf[:K_, :N].float()            # exact in fp32, and in the half types up to 2^8
+        assert torch.equal(c.float().cpu(), want.to(dtype).float()), (M, N, K_)
+        assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5), (M, N, K_)
+
+
 def test_matmul_ragged_fast_path_exact_and_with_wild_values_next_door():
     # small integers: bit for bit against the oracle.  The operands are views into larger buffers whose
     # neighbouring rows and columns hold inf and NaN: whatever the clamped fetches and the padding steps

@@ -73,6 +73,30 @@ def test_tiled_matmul_small_integers_are_exact_and_padding_is_untouched():
     assert not torch.isnan(full[:M, :N]).any() and torch.isnan(full[M:, :]).all() and torch.isnan(full[:, N:]).all()
 
 
+def test_tiled_matmul_random_shapes_exact_and_padding_untouched():
+    # a seeded sweep over any M, N, K at the reference's 32x32x32 tiling: small integers, bit for bit; the padding of
+    # the C tiles keeps the NaN it was filled with
+    rng = np.random.default_rng(77)
+    for case in range(16):
+        M, N, K_ = (int(rng.integers(1, 600)) for _ in range(3))
+        g = torch.Generator().manual_seed(case)
+        a = torch.randint(-3, 4, (M, K_), generator=g).to(torch.float16)
+        b = torch.randint(-3, 4, (K_, N), generator=g).to(torch.float16)
+        tm, tn = K.cdiv(M, 32), K.cdiv(N, 32)
+        c = torch.full((tm * tn * 1024, ), float("nan"), dtype=torch.float16, device="cuda")
+        act = "leaky_relu" if case % 3 == 0 else ""
+        K.matmul_kernel[(tm * tn, )](K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), c, M, N, K_, K_, 1, N, 1, N, 1,
+                                     ACTIVATION=act)
+        whole = M % 256 == 0 and N % 256 == 0 and K_ % 128 == 0
+        assert rt.last_kernel_name().startswith("gemm_tiled_f16" if whole else "gemm_tiledragged_f16"), (M, N, K_)
+        full = c.cpu().reshape(tm, tn, 32, 32).permute(0, 2, 1, 3).reshape(tm * 32, tn * 32)
+        want = a.float() @ b.float()
+        if act:
+            want = torch.where(want >= 0, want, 0.01 * want)
+        assert torch.equal(full[:M, :N], want.to(torch.float16)), (M, N, K_)
+        assert torch.isnan(full[M:, :]).all() and torch.isnan(full[:, N:]).all(), (M, N, K_)
+
+
 def test_tiled_matmul_bf16_inputs_give_fp16():
     M, N, K_ = 64, 96, 128
     a, b = _rand((M, K_), 4, torch.bfloat16), _rand((K_, N), 5, torch.bfloat16)
