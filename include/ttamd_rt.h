@@ -210,6 +210,12 @@ TTAMD_API int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_el
                     int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
 TTAMD_API int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_t n_elements,
                      int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
+/* The same with one operand a compile-time constant of the kernel: out[i] = x[i] OP c, or c OP x[i] when flip
+ * is set.  x and out may be the same buffer.  With BLOCK_SIZE = 1 and n_elements = grid[0] this is the
+ * one-element-per-program form of test_core.py::test_load_store_same_ptr (x = load(p + pid); store(p + pid, x * 2)),
+ * which the reference's CI runs beside test_reduce1d (.github/workflows/integration-tests-cpu.yml:105). */
+TTAMD_API int tt_binary_const_kernel(int32_t op, const void *x, float c, int32_t flip, void *out, int32_t n_elements,
+                           int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
 TTAMD_API int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
                    int32_t in_dtype, int32_t out_dtype, const uint32_t grid[3], void *stream);
 

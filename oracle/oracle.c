@@ -392,6 +392,18 @@ ORC_API int orc_binary_f32(int op, const float *x, const float *y, float *out, i
   }
   return 0;
 }
+/* one operand a constant of the kernel: out[i] = x[i] OP c, or c OP x[i] when flip is set; x and out may be
+ * the same buffer (the one-element-per-program form of test_core.py::test_load_store_same_ptr has block = 1) */
+ORC_API int orc_binary_const_f32(int op, const float *x, float c, int flip, float *out, int32_t n, int32_t block,
+                                 int32_t grid) {
+  if (op < 0 || op > 5) return -1;
+  for (int64_t pid = 0; pid < grid; ++pid) {
+    int64_t lo = pid * (int64_t)block, hi = lo + block;
+    if (hi > n) hi = n;
+    for (int64_t i = lo; i < hi; ++i) out[i] = flip ? orc_binary_apply(op, c, x[i]) : orc_binary_apply(op, x[i], c);
+  }
+  return 0;
+}
 /* arith.trunci: the low bits are kept */
 ORC_API void orc_trunci(const int32_t *x, void *out, int bits, int32_t n, int32_t block, int32_t grid) {
   for (int64_t pid = 0; pid < grid; ++pid) {

@@ -70,6 +70,8 @@ def lib() -> C.CDLL:
         L.orc_unary_f32.restype = C.c_int
         L.orc_binary_f32.argtypes = [C.c_int, vp, vp, vp, i32, i32, i32, C.c_int]
         L.orc_binary_f32.restype = C.c_int
+        L.orc_binary_const_f32.argtypes = [C.c_int, vp, f32, C.c_int, vp, i32, i32, i32]
+        L.orc_binary_const_f32.restype = C.c_int
         L.orc_trunci.argtypes = [vp, vp, C.c_int, i32, i32, i32]
         L.orc_reduce1d.restype = C.c_int
         L.orc_reduce1d.argtypes = [C.c_int, vp, i32, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, vp]
@@ -240,6 +242,19 @@ def binary(op: str, x: np.ndarray, y: np.ndarray, *, block: int = 1024, grid: in
     grid = cdiv(x.size, block) if grid is None else grid
     if lib().orc_binary_f32(BINARY_OPS[op], _p(x), _p(y), _p(out), x.size, block, grid, nthreads):
         raise ValueError("orc_binary_f32 rejected the launch")
+    return out
+
+
+def binary_const(op: str, x: np.ndarray, c: float, *, flip: bool = False, block: int = 1024, grid: int | None = None,
+                 out: np.ndarray | None = None) -> np.ndarray:
+    """out[i] = x[i] OP c (c OP x[i] with ``flip``) in fp32; ``out`` may be ``x`` itself."""
+    x = np.ascontiguousarray(x, dtype=np.float32) if out is not x else x
+    if out is None:
+        out = np.zeros_like(x)
+    rc = lib().orc_binary_const_f32(BINARY_OPS[op], _p(x), float(np.float32(c)), int(flip), _p(out), x.size, block,
+                                    cdiv(x.size, block) if grid is None else grid)
+    if rc:
+        raise ValueError(f"unknown binary operation {op!r}")
     return out
 
 

@@ -77,6 +77,21 @@ def test_masked_tail_partial_grid_and_unaligned():
         K.unary("sqrt", x.cuda().half())
 
 
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "maximum", "minimum"])
+def test_constant_operand_forms_exact(op):
+    for c in (2.0, -0.75, 0.0, float("inf"), float("nan")):
+        for flip in (False, True):
+            got = K.binary_const(op, X.cuda(), c, flip=flip).cpu().numpy()
+            assert rt.last_kernel_name() == f"ew_{ {'maximum': 'max', 'minimum': 'min'}.get(op, op)}c_f32"
+            assert _bits_equal(got, orc.binary_const(op, X.numpy(), c, flip=flip)), (op, c, flip)
+    # in place, an odd length and an operand off the 16-byte grid
+    buf = torch.cat([torch.zeros(1), X]).cuda()
+    view = buf[1:]
+    K.binary_const(op, view, 1.5, out=view)
+    assert rt.last_kernel_name().endswith("_unaligned")
+    assert _bits_equal(view.cpu().numpy(), orc.binary_const(op, X.numpy(), 1.5)) and float(buf[0]) == 0.0
+
+
 def test_narrowing_casts_exact():
     xf = torch.cat([X, torch.tensor([65504.0, 65520.0, 65519.99, 1e-8, 3.3895e38], dtype=torch.float32)])
     for dt, code in ((torch.bfloat16, orc.BF16), (torch.float16, orc.F16)):

@@ -64,7 +64,7 @@ def fake(monkeypatch):
     monkeypatch.setattr(drv.TTDriver, "get_current_stream", lambda self, d=None: 0x1234)
     for k in (K.add_kernel, K.add_kernel_loop, K.sin_kernel, K.matmul_kernel_tma, K.matmul_kernel_fused, K._attn_fwd,
               K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel, K.unary_kernel, K.binary_kernel,
-              K.cast_kernel, K.reduce1d_kernel):
+              K.cast_kernel, K.reduce1d_kernel, K.binary_const_kernel):
         k._cache.clear()
     return lib
 
@@ -309,3 +309,15 @@ def test_reduce1d_binds_with_tritons_accumulate_types(fake):
                  "int64": "I64", "float64": "F64", "uint8": "U8", "uint16": "U16", "uint32": "U32", "uint64": "U64"}[name]
         assert re.search(rf"TT_{short} = {code}\b", header), name
         assert getattr(orc, short) == code
+
+
+def test_constant_operand_kernel_binds(fake):
+    x, o = FakeTensor((5000, ), torch.float32), FakeTensor((5000, ), torch.float32)
+    K.binary_const_kernel[(5, )](x, o, 5000, BLOCK_SIZE=1024, OP="sub", C=3.5, FLIP=True)
+    name, a = fake.calls[-1]
+    assert name == "tt_binary_const_kernel" and a[0] == rt.BINARY_OPS["sub"] and a[2:4] == (3.5, 1) and a[5:7] == (5000, 1024)
+    K.binary_const_kernel[(5, )](x, x, 5000, BLOCK_SIZE=1024, OP="mul", C=2)          # in place, FLIP defaults to False
+    name, a = fake.calls[-1]
+    assert a[1] == a[4] and a[2:4] == (2.0, 0)
+    with pytest.raises(rt.Unsupported):
+        K.binary_const_kernel[(5, )](x, o, 5000, BLOCK_SIZE=1024, OP="pow", C=2.0)

@@ -77,3 +77,31 @@ def test_trunci_keeps_low_bits():
     x = np.array([0, 1, -1, 127, 128, 255, 256, 32767, 32768, 65535, 65536, -32769, 2**31 - 1, -2**31], dtype=np.int32)
     assert np.array_equal(orc.trunci(x, 16), x.astype(np.int16))
     assert np.array_equal(orc.trunci(x, 8), x.astype(np.int8))
+
+
+@pytest.mark.parametrize("op,ref", [("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)])
+@pytest.mark.parametrize("c", [2.0, -0.75, 0.0, np.inf])
+def test_constant_operand_forms_equal_numpy_float32(op, ref, c):
+    # x OP c and c OP x against numpy's own float32 arithmetic (not the oracle's formula); in place as well
+    cf = np.float32(c)
+    with np.errstate(all="ignore"):
+        assert _same(orc.binary_const(op, X, c), ref(X, cf).astype(np.float32))
+        assert _same(orc.binary_const(op, X, c, flip=True), ref(cf, X).astype(np.float32))
+        buf = X.copy()
+        assert orc.binary_const(op, buf, c, out=buf) is buf and _same(buf, ref(X, cf).astype(np.float32))
+    # and it is the two-operand oracle with a constant second array
+    assert _same(orc.binary_const(op, X, c), orc.binary(op, X, np.full_like(X, cf)))
+
+
+def test_constant_operand_max_min_and_one_element_per_program():
+    for op in ("maximum", "minimum"):
+        for c in (0.5, np.nan, -0.0):
+            assert _same(orc.binary_const(op, X, c), orc.binary(op, X, np.full_like(X, np.float32(c))))
+            assert _same(orc.binary_const(op, X, c, flip=True), orc.binary(op, np.full_like(X, np.float32(c)), X))
+    # test_core.py::test_load_store_same_ptr: 65536 programs, one element each, x * 2 in place
+    x = np.ones(65536, np.float32)
+    orc.binary_const("mul", x, 2.0, block=1, grid=65536, out=x)
+    assert np.all(x == 2.0)
+    y = np.ones(10, np.float32)
+    orc.binary_const("mul", y, 2.0, block=1, grid=4, out=y)       # a smaller grid touches its own elements only
+    assert np.array_equal(y, [2, 2, 2, 2, 1, 1, 1, 1, 1, 1])

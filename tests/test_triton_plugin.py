@@ -374,3 +374,55 @@ def test_offline_compile_tool_accepts_the_tenstorrent_target(tmp_path, monkeypat
     assert {"add_kernel.ttir", "add_kernel.ttamd", "add_kernel.json"} <= made
     record = json.loads(next((tmp_path / "cache").rglob("add_kernel.ttamd")).read_text())
     assert record["kernel"] == "add_kernel" and record["arch"] == "gfx950"
+
+
+# --- a constant operand, and the one-element-per-program form of test_core.py::test_load_store_same_ptr ---
+@triton.jit
+def kernel_same_ptr(in_out_ptr):
+    pid = tl.program_id(axis=0)
+    x = tl.load(in_out_ptr + pid)
+    out = x * 2
+    tl.store(in_out_ptr + pid, out)
+
+
+@triton.jit
+def user_rsub_const(x_ptr, y_ptr, n, BLOCK: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    offs = pid * BLOCK + tl.arange(0, BLOCK)
+    m = offs < n
+    tl.store(y_ptr + offs, 3.5 - tl.load(x_ptr + offs, mask=m), mask=m)
+
+
+def test_constant_operand_forms_are_recognised(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    m = json.loads(_compile(kernel_same_ptr, {"in_out_ptr": "*fp32"}, {}).kernel)["match"]
+    assert m == {"kernel": "binary_const_kernel", "op": "mul", "inputs": ["in_out_ptr"], "output": "in_out_ptr", "n": None,
+                 "n_const": None, "block": 1, "c": 2.0, "flip": False}
+    m = json.loads(_compile(user_rsub_const, {"x_ptr": "*fp32", "y_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"},
+                            {"BLOCK": 1024}).kernel)["match"]
+    assert (m["kernel"], m["op"], m["inputs"], m["output"], m["n"], m["block"], m["c"], m["flip"]) == \
+        ("binary_const_kernel", "sub", ["x_ptr"], "y_ptr", "n", 1024, 3.5, True)
+
+
+@pytest.mark.gpu
+def test_load_store_same_ptr_runs(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton_tenstorrent_amd import runtime as rt
+    ttc.register()
+    try:
+        for _ in range(20):                                  # the upstream test repeats the launch 1000 times
+            x = torch.ones((65536, ), device="cuda", dtype=torch.float32)
+            kernel_same_ptr[(65536, )](x, num_warps=16)
+            assert torch.all(x == 2)
+        assert rt.last_kernel_name() == "ew_mulc_f32"
+        x = torch.ones(100, device="cuda")
+        kernel_same_ptr[(40, )](x)                           # 40 programs touch 40 elements
+        assert torch.all(x[:40] == 2) and torch.all(x[40:] == 1)
+        a = torch.randn(70001, device="cuda")
+        y = torch.full((70001 + 3, ), -7.0, device="cuda")
+        user_rsub_const[(triton.cdiv(70001, 1024), )](a, y, 70001, BLOCK=1024)
+        assert rt.last_kernel_name() == "ew_subc_f32" and torch.equal(y[:70001], 3.5 - a) and torch.all(y[70001:] == -7.0)
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None

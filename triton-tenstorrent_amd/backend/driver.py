@@ -233,6 +233,19 @@ def _bind_binary(lib, cur, consts, grid, stream):
                                 out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
 
 
+def _bind_binary_const(lib, cur, consts, grid, stream):
+    """out[i] = x[i] OP C, or C OP x[i] with FLIP: a binary operation of ConvertComputeOps.cpp:162-167 against a
+    constant of the kernel."""
+    x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
+    n = int(cur.scalar("n_elements"))
+    cur.done()
+    if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
+        raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "binary_const_kernel computes in fp32")
+    return lib.tt_binary_const_kernel(_op_code(rt.BINARY_OPS, consts, "binary_const_kernel"), x.data_ptr(), float(consts["C"]),
+                                      int(bool(consts.get("FLIP", False))), out.data_ptr(), n, int(consts["BLOCK_SIZE"]),
+                                      grid, stream)
+
+
 def _bind_cast(lib, cur, consts, grid, stream):
     """out[i] = x[i].to(out dtype): arith.truncf / arith.trunci (ConvertComputeOps.cpp:181-182)."""
     x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
@@ -381,7 +394,10 @@ def _bind_matched(match: dict, lib, cur, consts, grid, stream):
             raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "tensor arguments must live on the GPU")
         _contiguous_1d(t)
     cur.keep.extend(tensors)
-    n = int(match["n_const"] if match.get("n") is None else vals[match["n"]])
+    if match.get("n") is not None:
+        n = int(vals[match["n"]])
+    else:
+        n = int(match["n_const"]) if match.get("n_const") is not None else None     # None: one element per program
     block = int(match["block"])
     ptrs = [t.data_ptr() for t in tensors]
     if match["kernel"] == "reduce1d_kernel":
@@ -389,6 +405,11 @@ def _bind_matched(match: dict, lib, cur, consts, grid, stream):
             raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"the kernel reads {block} elements, its input holds {tensors[0].numel()}")
         return lib.tt_reduce1d_kernel(rt.REDUCE_OPS[match["op"]], ptrs[0], ptrs[1], block, match["in_dtype"],
                                       match["acc_dtype"], match["out_dtype"], int(match["propagate_nan"]), grid, stream)
+    if match["kernel"] == "binary_const_kernel":
+        if match.get("n") is None and match.get("n_const") is None:      # one element per program: n is the grid
+            n = int(grid[0])
+        return lib.tt_binary_const_kernel(rt.BINARY_OPS[match["op"]], ptrs[0], float(match["c"]), int(match["flip"]), ptrs[1],
+                                          n, block, grid, stream)
     if match["kernel"] == "muladd_kernel":
         return lib.tt_muladd_kernel(ptrs[0], ptrs[1], ptrs[2], ptrs[3], n, block, grid, stream)
     if match["kernel"] == "add_kernel":
@@ -408,6 +429,7 @@ KERNEL_TABLE: dict[str, Callable] = {
     "unary_kernel": _bind_unary,
     "binary_kernel": _bind_binary,
     "cast_kernel": _bind_cast,
+    "binary_const_kernel": _bind_binary_const,
     "reduce1d_kernel": _bind_reduce1d,
     "matmul_kernel_tma": _bind_matmul_tma,
     "matmul_kernel_tma_fp8_scaled": _bind_matmul_tma,

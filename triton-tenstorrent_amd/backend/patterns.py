@@ -125,8 +125,15 @@ def match_streaming(ttir: str) -> dict | None:
     if out_arg is None:
         return None
     inputs = []
-    for o in operands:
+    const_operand = None       # (position, value) of a splat constant among the operands of a binary operation
+    for pos, o in enumerate(operands):
         d = defs.get(o)
+        if d and d[0] == "arith.constant" and op in BINARY and const_operand is None and len(operands) == 2:
+            cm = re.match(r"\s*dense<([^>]+)>\s*:\s*tensor<\d+xf32>", d[2])
+            if not cm:
+                return None
+            const_operand = (pos, float(cm.group(1)))
+            continue
         if not d or d[0] != "tt.load" or len(d[1]) < 2 or d[1][1] != mask:
             return None
         a, offs = pointer_arg(d[1][0])
@@ -190,13 +197,20 @@ def match_streaming(ttir: str) -> dict | None:
             if len(inputs) != 1:
                 return None
             kernel, opname = "unary_kernel", UNARY[op]
+        elif const_operand is not None:
+            if len(inputs) != 1:
+                return None
+            kernel, opname = "binary_const_kernel", BINARY[op]
         else:
             if len(inputs) != 2:
                 return None
             kernel, opname = "binary_kernel", BINARY[op]
     strip = lambda a: a.lstrip("%")
-    return {"kernel": kernel, "op": opname, "inputs": [strip(a) for a in inputs], "output": strip(out_arg),
-            "n": strip(n_src) if n_const is None else None, "n_const": n_const, "block": block}
+    rec = {"kernel": kernel, "op": opname, "inputs": [strip(a) for a in inputs], "output": strip(out_arg),
+           "n": strip(n_src) if n_const is None else None, "n_const": n_const, "block": block}
+    if kernel == "binary_const_kernel":
+        rec.update(c=const_operand[1], flip=const_operand[0] == 0)
+    return rec
 
 
 _ELEM = {"f32": 0, "i32": 1, "bf16": 2, "f16": 3, "i16": 5, "i8": 6, "i64": 7, "f64": 8}
@@ -334,3 +348,70 @@ def match_reduce1d(ttir: str) -> dict | None:
     return {"kernel": "reduce1d_kernel", "op": op, "inputs": [strip(x_arg)], "output": strip(st[2][0]), "n": None,
             "n_const": block, "block": block, "in_dtype": in_dt, "acc_dtype": acc_dt, "out_dtype": out_dt,
             "propagate_nan": nan, "tie_break_left": tie}
+
+
+def match_per_program(ttir: str) -> dict | None:
+    """The one-element-per-program form of test_core.py::test_load_store_same_ptr:
+
+        pid = program_id(0); x = load(p + pid); store(q + pid, x OP constant)
+
+    (p and q may be the same argument) -> ``binary_const_kernel`` with BLOCK = 1 and n = the grid, or None."""
+    parsed = _body(ttir)
+    if parsed is None:
+        return None
+    _, args, lines = parsed
+    arg_types = dict(args)
+    defs, order = {}, []
+    for raw in lines:
+        line = _LOC.sub("", raw).strip()
+        if not line:
+            continue
+        m = _OP.match(line)
+        if not m:
+            return None
+        res, op, rest = m.groups()
+        operands = _SSA.findall(rest.split(" : ")[0])
+        order.append((res, op, operands, rest))
+        if res:
+            defs[res] = (op, operands, rest)
+    kinds = [o[1] for o in order]
+    compute = [o for o in order if o[1] in BINARY]
+    if sorted(k for k in kinds if k not in BINARY) != sorted(["tt.get_program_id", "tt.addptr", "tt.load", "arith.constant",
+                                                             "tt.addptr", "tt.store", "tt.return"]) and \
+            sorted(k for k in kinds if k not in BINARY) != sorted(["tt.get_program_id", "tt.addptr", "tt.load", "arith.constant",
+                                                                 "tt.store", "tt.return"]):
+        return None
+    if len(compute) != 1:
+        return None
+    res, op, operands, _ = compute[0]
+    if len(operands) != 2:
+        return None
+
+    def pointer_arg(ssa):      # %p = tt.addptr %arg, %pid with %pid = tt.get_program_id x
+        d = defs.get(ssa)
+        if not d or d[0] != "tt.addptr" or len(d[1]) != 2 or d[1][0] not in arg_types:
+            return None
+        pid = defs.get(d[1][1])
+        if not pid or pid[0] != "tt.get_program_id" or not pid[2].lstrip().startswith("x"):
+            return None
+        return d[1][0]
+
+    x_arg = c = flip = None
+    for pos, o in enumerate(operands):
+        d = defs.get(o)
+        if d and d[0] == "tt.load" and len(d[1]) == 1:
+            x_arg = pointer_arg(d[1][0])
+        elif d and d[0] == "arith.constant":
+            cm = re.match(r"\s*([-+0-9.eE]+(?:inf|nan)?)\s*:\s*f32", d[2])
+            if not cm:
+                return None
+            c, flip = float(cm.group(1)), pos == 0
+    st = next(o for o in order if o[1] == "tt.store")
+    if x_arg is None or c is None or len(st[2]) != 2 or st[2][1] != res:
+        return None
+    out_arg = pointer_arg(st[2][0])
+    if out_arg is None or arg_types[x_arg] != "!tt.ptr<f32>" or arg_types[out_arg] != "!tt.ptr<f32>":
+        return None
+    strip = lambda a: a.lstrip("%")
+    return {"kernel": "binary_const_kernel", "op": BINARY[op], "inputs": [strip(x_arg)], "output": strip(out_arg), "n": None,
+            "n_const": None, "block": 1, "c": c, "flip": flip}

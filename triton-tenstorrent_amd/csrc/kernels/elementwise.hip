@@ -74,6 +74,54 @@ __device__ __forceinline__ void binary_body(const T *__restrict__ x, const T *__
   }
 }
 
+// out[i] = x[i] OP c, or c OP x[i] when flip is set; x and out may be the same buffer (every element is read and
+// written by one thread), so no __restrict__ here
+template <typename Op, int UNROLL>
+__device__ __forceinline__ void binary_const_body(const float *x, float c, int flip, float *out, uint32_t n) {
+  using V = Vec4<float>::type;
+  const uint32_t nvec = n >> 2;
+  const V *xv = reinterpret_cast<const V *>(x);
+  V *ov = reinterpret_cast<V *>(out);
+  const uint32_t base = blockIdx.x * (kThreads * UNROLL);
+  const uint32_t i = base + threadIdx.x;
+  auto f = [&](float v) { return flip ? Op::apply(c, v) : Op::apply(v, c); };
+  if (base + kThreads * UNROLL <= nvec) {
+    V a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * kThreads);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      V r;
+      r.x = f(a[u].x);
+      r.y = f(a[u].y);
+      r.z = f(a[u].z);
+      r.w = f(a[u].w);
+      __builtin_nontemporal_store(r, ov + i + u * kThreads);
+    }
+  } else {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t j = i + u * kThreads;
+      if (j < nvec) {
+        V a = xv[j], r;
+        r.x = f(a.x);
+        r.y = f(a.y);
+        r.z = f(a.z);
+        r.w = f(a.w);
+        ov[j] = r;
+      }
+    }
+    const uint32_t t = (nvec << 2) + threadIdx.x;
+    if (t < n) out[t] = f(x[t]);
+  }
+}
+template <typename Op>
+__device__ __forceinline__ void binary_const_scalar_body(const float *x, float c, int flip, float *out, uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride)
+    out[i] = flip ? Op::apply(c, x[i]) : Op::apply(x[i], c);
+}
+
 template <typename T, typename Op>
 __device__ __forceinline__ void binary_scalar_body(const T *x, const T *y, T *out, uint32_t n) {
   const uint32_t stride = gridDim.x * kThreads;
@@ -335,6 +383,23 @@ EW_UNARY(sqrt, SqrtOp)
                                                                         float *out, uint32_t n) {          \
     binary_scalar_body<float, Op>(x, y, out, n);                                                           \
   }
+// one operand a constant: ew_<op>c_f32
+#define EW_BINARY_CONST(name, Op)                                                                              \
+  __global__ __launch_bounds__(kThreads) void ew_##name##c_f32(const float *x, float c, int flip, float *out,  \
+                                                               uint32_t n) {                                   \
+    binary_const_body<Op, 4>(x, c, flip, out, n);                                                              \
+  }                                                                                                            \
+  __global__ __launch_bounds__(kThreads) void ew_##name##c_f32_unaligned(const float *x, float c, int flip,    \
+                                                                         float *out, uint32_t n) {             \
+    binary_const_scalar_body<Op>(x, c, flip, out, n);                                                          \
+  }
+EW_BINARY_CONST(add, AddOp)
+EW_BINARY_CONST(sub, SubOp)
+EW_BINARY_CONST(mul, MulOp)
+EW_BINARY_CONST(div, DivOp)
+EW_BINARY_CONST(max, MaxOp)
+EW_BINARY_CONST(min, MinOp)
+
 EW_BINARY(sub, SubOp)
 EW_BINARY(mul, MulOp)
 EW_BINARY(div, DivOp)

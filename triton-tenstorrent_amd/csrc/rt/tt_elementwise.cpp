@@ -160,6 +160,25 @@ int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_
   return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 4);
 }
 
+int tt_binary_const_kernel(int32_t op, const void *x, float c, int32_t flip, void *out, int32_t n_elements,
+                           int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream) {
+  static const char *const names[] = {"add", "sub", "mul", "div", "max", "min"};
+  if (!props()) return fail(RT_ERR_NOT_INIT, "binary_const_kernel: call rt_init first");
+  if (op < 0 || op >= (int)(sizeof(names) / sizeof(names[0])))
+    return fail(RT_ERR_UNSUPPORTED, "binary_const_kernel: op %d (tt_binary_op has 0..5)", op);
+  uint32_t n_eff = 0;
+  int rc = check_1d("binary_const_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !out) return fail(RT_ERR_INVALID, "binary_const_kernel: null tensor pointer");
+  bool al = aligned16(x) && aligned16(out);
+  char name[48];
+  snprintf(name, sizeof(name), "ew_%sc_f32%s", names[op], al ? "" : "_unaligned");
+  int32_t fl = flip ? 1 : 0;
+  void *args[] = {&x, &c, &fl, &out, &n_eff};
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 5);
+}
+
 int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE, int32_t in_dtype,
                    int32_t out_dtype, const uint32_t grid[3], void *stream) {
   if (!props()) return fail(RT_ERR_NOT_INIT, "cast_kernel: call rt_init first");

@@ -52,6 +52,19 @@ def binary(op: str, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
     return out
 
 
+binary_const_kernel = PrebuiltKernel("binary_const_kernel", ["x_ptr", "output_ptr", "n_elements", "BLOCK_SIZE", "OP", "C", "FLIP"],
+                                     ["BLOCK_SIZE", "OP", "C", "FLIP"], defaults={"FLIP": False})
+
+
+def binary_const(op: str, x: torch.Tensor, c: float, flip: bool = False, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``x OP c`` (``c OP x`` with ``flip``) for ``op`` in add, sub, mul, div, maximum, minimum; fp32.  ``out`` may be
+    ``x`` itself (test_core.py::test_load_store_same_ptr updates its buffer in place)."""
+    out = torch.empty_like(x) if out is None else out
+    n = out.numel()
+    binary_const_kernel[lambda meta: (cdiv(n, meta["BLOCK_SIZE"]), )](x, out, n, BLOCK_SIZE=1024, OP=op, C=float(c), FLIP=flip)
+    return out
+
+
 def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     """fp32 -> bf16 / fp16 (round to nearest even) or int32 -> int16 / int8 (low bits kept)."""
     out = torch.empty(x.shape, device=x.device, dtype=dtype)
