@@ -138,6 +138,15 @@ def main() -> int:
             print("bench.py: GEMM output failed its parity spot check", file=sys.stderr)
             return 1
         del a, b, c, ad, bd, cd
+        # shapes that are not whole 256x256x128 macro tiles run the same kernel's clamping instantiation
+        ragged = {}
+        for (m_, n_, k_) in ((8000, 8192, 8192), (8192, 8192, 8160)):
+            a = (torch.randn(m_, k_, device="cuda") / math.sqrt(k_)).to(torch.bfloat16)
+            b = (torch.randn(k_, n_, device="cuda") / math.sqrt(k_)).to(torch.bfloat16)
+            avg_ms, per, _ = _events_time(lambda: K.matmul_tma(a, b), max(3, steps // 4), 2, stream)
+            ragged[f"{m_}x{n_}x{k_}"] = {"kernel": rt.last_kernel_name(), "TFLOPs": round(2.0 * m_ * n_ * k_ / (avg_ms * 1e-3) / 1e12, 1)}
+            del a, b
+        extra["gemm_bf16_ragged_shapes"] = ragged
 
     # ---------------- elementwise streaming, N = 2^28 ----------------------
     n_el = 1 << 28
@@ -279,6 +288,17 @@ def main() -> int:
                                                   "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
         rooflines["attn_fwd_causal_4x32x4096x128"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "attn_tile_d128")
         del q, k, v
+        # the other instantiations of the same kernel, for the record (few launches each; not roofline lines)
+        others = {}
+        for (z, h, s_, d, causal) in ((4, 32, 4096, 128, False), (4, 32, 4064, 128, True), (4, 32, 4096, 64, True),
+                                      (4, 32, 4096, 32, True), (2, 16, 4096, 256, True)):
+            q, k, v = (torch.randn(z, h, s_, d, device="cuda").to(torch.bfloat16) for _ in range(3))
+            avg_ms, per, _ = _events_time(lambda: K.attention(q, k, v, causal, 1.0 / math.sqrt(d)), max(3, steps // 4), 2, stream)
+            fl = 4.0 * z * h * s_ * s_ * d * (0.5 if causal else 1.0)
+            others[f"{z}x{h}x{s_}x{d}_{'causal' if causal else 'full'}"] = {"kernel": rt.last_kernel_name(),
+                                                                          "TFLOPs": round(fl / (avg_ms * 1e-3) / 1e12, 1)}
+            del q, k, v
+        extra["attn_fwd_other_shapes"] = others
 
     # ---------------- CPU baseline: the oracle on a bounded sample ---------
     cpu_baseline = None
