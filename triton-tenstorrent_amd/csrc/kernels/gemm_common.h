@@ -113,22 +113,21 @@ __device__ __forceinline__ void tile_of_pid(int pid, int num_pid_m, int num_pid_
 }
 
 // erf-form GELU, 0.5*x*(1+erf(x/sqrt(2))).  erf by Abramowitz & Stegun 7.1.26,
-// 1 - (a1 t + ... + a5 t^5) exp(-z^2) with t = 1/(1 + p z): absolute error <= 1.5e-7,
-// branch-free, one rcp and one exp2 instead of the library routine's ~40 operations (the
-// epilogue runs on 256 accumulators per lane with the matrix pipe idle).
+// erf(z) = 1 - (a1 t + ... + a5 t^5) exp(-z^2) for z >= 0 with t = 1/(1 + p z): absolute error <= 1.5e-7,
+// branch-free, one rcp and one exp2 instead of the library routine's ~40 operations (the epilogue runs on
+// 256 accumulators per lane with the matrix pipe idle).  Written out in x itself, with z = |x|/sqrt(2),
+//   gelu(x) = 0.5 (x + |x| erf(z)) = max(x, 0) - |x| * (0.5 (a1 t + ... + a5 t^5)) * exp2(-x^2 * 0.5 log2(e))
+// so the scaling by 1/sqrt(2), the sign and the halving cost nothing: 11 VALU operations, rcp and exp2.
 __device__ __forceinline__ float gelu_erf(float x) {
-  const float z = x * 0.70710678118654752440f;
-  const float az = __builtin_fabsf(z);
-  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, az, 1.0f));
-  float p = __builtin_fmaf(1.061405429f, t, -1.453152027f);
-  p = __builtin_fmaf(p, t, 1.421413741f);
-  p = __builtin_fmaf(p, t, -0.284496736f);
-  p = __builtin_fmaf(p, t, 0.254829592f);
+  const float ax = __builtin_fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f * 0.70710678118654752440f, ax, 1.0f));
+  float p = __builtin_fmaf(0.5f * 1.061405429f, t, 0.5f * -1.453152027f);
+  p = __builtin_fmaf(p, t, 0.5f * 1.421413741f);
+  p = __builtin_fmaf(p, t, 0.5f * -0.284496736f);
+  p = __builtin_fmaf(p, t, 0.5f * 0.254829592f);
   p = p * t;
-  const float e = __builtin_amdgcn_exp2f(-az * az * 1.44269504088896340736f);
-  const float erf_abs = __builtin_fmaf(-p, e, 1.0f);
-  const float erf_z = __builtin_copysignf(erf_abs, z);
-  return 0.5f * x * (1.0f + erf_z);
+  const float e = __builtin_amdgcn_exp2f((x * -0.72134752044448170368f) * x);
+  return __builtin_fmaf(-ax, p * e, __builtin_fmaxf(x, 0.0f));
 }
 
 // Epilogue on one fp32 accumulator value destined for C[m,n]; returns the fp32
