@@ -473,14 +473,17 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
   // ---- epilogue ----
   if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
   uint16_t *orow = a.o + (base + my_q) * a.ldo;
+  const float inv_l = 1.0f / l_i;
 #pragma unroll
   for (int t = 0; t < DT; ++t)
 #pragma unroll
     for (int r4 = 0; r4 < 4; ++r4) {
       const int d = t * 32 + r4 * 8 + hi * 4;
       typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-      u32x2_t pk = {pack_bf16x2(acc[t][r4 * 4 + 0] / l_i, acc[t][r4 * 4 + 1] / l_i),
-                    pack_bf16x2(acc[t][r4 * 4 + 2] / l_i, acc[t][r4 * 4 + 3] / l_i)};
+      // one division per query, then multiplications: within one fp32 unit in the last place of acc / l_i, far
+      // below the bf16 rounding that follows (a full division is ten instructions, and there are 4*D of them)
+      u32x2_t pk = {pack_bf16x2(acc[t][r4 * 4 + 0] * inv_l, acc[t][r4 * 4 + 1] * inv_l),
+                    pack_bf16x2(acc[t][r4 * 4 + 2] * inv_l, acc[t][r4 * 4 + 3] * inv_l)};
       *(u32x2_t *)(orow + d) = pk;
     }
 }
