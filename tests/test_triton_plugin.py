@@ -426,3 +426,40 @@ def test_load_store_same_ptr_runs(tmp_path, monkeypatch):
         from triton.backends import backends
         backends.pop("tenstorrent", None)
         triton.runtime.driver._active = None
+
+
+# --- autotune and do_bench through the plugin's device interface (driver.py:390-442 of the reference) ---
+@triton.autotune(configs=[triton.Config({"BLOCK_SIZE": 512}), triton.Config({"BLOCK_SIZE": 1024}),
+                          triton.Config({"BLOCK_SIZE": 2048})], key=["n_elements"])
+@triton.jit
+def add_kernel_autotuned(x_ptr, y_ptr, output_ptr, n_elements, BLOCK_SIZE: tl.constexpr):
+    pid = tl.program_id(axis=0)
+    block_start = pid * BLOCK_SIZE
+    offsets = block_start + tl.arange(0, BLOCK_SIZE)
+    mask = offsets < n_elements
+    x = tl.load(x_ptr + offsets, mask=mask)
+    y = tl.load(y_ptr + offsets, mask=mask)
+    tl.store(output_ptr + offsets, x + y, mask=mask)
+
+
+@pytest.mark.gpu
+def test_autotune_and_do_bench_through_the_plugin(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton_tenstorrent_amd import runtime as rt
+    ttc.register()
+    try:
+        n = 1 << 22
+        x, y = torch.rand(n, device="cuda"), torch.rand(n, device="cuda")
+        out = torch.empty_like(x)
+        grid = lambda meta: (triton.cdiv(n, meta["BLOCK_SIZE"]), )
+        add_kernel_autotuned[grid](x, y, out, n)             # times the three configurations with the driver's benchmarker
+        assert torch.equal(out, x + y) and rt.last_kernel_name() == "ew_add_f32"
+        assert add_kernel_autotuned.best_config.kwargs["BLOCK_SIZE"] in (512, 1024, 2048)
+        assert len(add_kernel_autotuned.cache) == 1
+        # do_bench drives Event / synchronize / the cache-clearing buffer of the device interface
+        ms = triton.testing.do_bench(lambda: add_kernel_autotuned[grid](x, y, out, n), warmup=5, rep=20)
+        assert 0.0 < ms < 5.0, ms                                             # 48 MiB of traffic: a few tens of microseconds
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None
