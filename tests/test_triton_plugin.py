@@ -463,3 +463,55 @@ def test_autotune_and_do_bench_through_the_plugin(tmp_path, monkeypatch):
         from triton.backends import backends
         backends.pop("tenstorrent", None)
         triton.runtime.driver._active = None
+
+
+@pytest.mark.gpu
+def test_triton_jit_launches_the_fused_matmul_muladd_and_attention(tmp_path, monkeypatch):
+    """The remaining example kernels as @triton.jit sources through Triton's own JIT: descriptors, scalars and
+    constexprs reach the launcher as Triton passes them."""
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton.tools.tensor_descriptor import TensorDescriptor
+    from oracle import oracle as orc
+    from triton_tenstorrent_amd import runtime as rt
+    from triton_tenstorrent_amd.examples import triton_kernels as tk
+    from util import bits
+    ttc.register()
+    try:
+        n = 70001
+        x, y, z = (torch.randn(n, device="cuda") for _ in range(3))
+        out = torch.empty_like(x)
+        tk.muladd_kernel[(triton.cdiv(n, 1024), )](x, y, z, out, n, BLOCK_SIZE=1024)
+        assert rt.last_kernel_name() == "ew_muladd_f32"
+        want = orc.muladd(x.cpu().numpy(), y.cpu().numpy(), z.cpu().numpy())
+        assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        # fused matmul: fp16, full bias added in fp16 after the cast
+        M, N, Kd = 256, 384, 128
+        a = (torch.randn(M, Kd, device="cuda") / 8).to(torch.float16)
+        b = torch.randn(Kd, N, device="cuda").to(torch.float16)
+        bias = torch.randn(M, N, device="cuda").to(torch.float16)
+        c = torch.empty(M, N, device="cuda", dtype=torch.float16)
+        descs = [TensorDescriptor.from_tensor(t, blk) for t, blk in ((a, [64, 64]), (b, [64, 64]), (c, [64, 64]), (bias, [64, 64]))]
+        tk.matmul_kernel_fused[(M // 64 * (N // 64), )](*descs, M, N, Kd, BLOCK_SIZE_M=64, BLOCK_SIZE_N=64, BLOCK_SIZE_K=64,
+                                                        GROUP_SIZE_M=1, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+        assert rt.last_kernel_name().startswith("gemm_") and rt.last_kernel_name().endswith("_epi1")
+        c0 = (a.double() @ b.double()).to(torch.float16)
+        assert torch.all((c.float() - (c0 + bias).float()).abs() <= 1e-2 * (c0 + bias).float().abs() + 2e-2)
+        # attention, causal and not, through 2-D descriptors over [Z*H*N_CTX, D]
+        Z, H, S, D = 1, 2, 256, 64
+        q, k, v = (torch.randn(Z, H, S, D, device="cuda").to(torch.bfloat16) for _ in range(3))
+        o = torch.empty_like(q)
+        Mlse = torch.empty(Z, H, S, device="cuda", dtype=torch.float32)
+        for causal in (True, False):
+            dq, dk, dv, do = (TensorDescriptor(t, shape=[Z * H * S, D], strides=[D, 1], block_shape=blk)
+                              for t, blk in ((q, [64, D]), (k, [64, D]), (v, [64, D]), (o, [64, D])))
+            tk._attn_fwd[(S // 64, Z * H, 1)](0.125, Mlse, Z, H, dq, dk, dv, do, S, HEAD_DIM=D, BLOCK_M=64, BLOCK_N=64,
+                                              FP8_OUTPUT=False, STAGE=3 if causal else 1, warp_specialize=False,
+                                              IS_HOPPER=False)
+            assert rt.last_kernel_name() == "attn_tile_d64"
+            wo, wM = orc.attn_fwd(bits(q), bits(k), bits(v), 0.125, causal=causal, BLOCK_M=64, BLOCK_N=64)
+            assert np.max(np.abs(o.float().cpu().numpy() - orc.from_bf16(wo))) <= 2e-2
+            assert np.max(np.abs(Mlse.cpu().numpy() - wM)) <= 1e-3
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None
