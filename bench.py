@@ -193,6 +193,8 @@ def main() -> int:
         avg_ms, per, _ = _events_time(lambda: K.cast_kernel[egrid](xs, ob, n_el, BLOCK_SIZE=1024), max(3, steps // 4), 2, stream)
         ops["truncf_bf16"] = round((4 + 2) * n_el / (avg_ms * 1e-3) / 1e9, 1)
         del ob
+        avg_ms, per, _ = _events_time(lambda: K.copy_kernel[egrid](xs, outs, n_el, BLOCK_SIZE=1024), max(3, steps // 4), 2, stream)
+        ops["copy"] = round(2 * 4 * n_el / (avg_ms * 1e-3) / 1e9, 1)
         extra["elementwise_ops_2p28_GBs"] = ops
         del xs, ys, outs
     if want("add0"):

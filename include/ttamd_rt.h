@@ -218,6 +218,12 @@ TTAMD_API int tt_binary_const_kernel(int32_t op, const void *x, float c, int32_t
                            int32_t BLOCK_SIZE, const uint32_t grid[3], void *stream);
 TTAMD_API int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
                    int32_t in_dtype, int32_t out_dtype, const uint32_t grid[3], void *stream);
+/* out[i] = x[i] for i < n_elements: the masked block loaded and stored back unchanged, the kernel that
+ * test_launch.py::test_memory_leak launches in the reference's CI (.github/workflows/integration-tests-cpu.yml:106;
+ * masked load and store: cpu/lib/TritonCPUToLLVM/MaskedOpsToLLVM.cpp:33-114).  dtype is any tt_dtype; the copy is
+ * by bytes.  x and out must be aligned to the element and must not overlap unless they are equal. */
+TTAMD_API int tt_copy_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE, int32_t dtype,
+                   const uint32_t grid[3], void *stream);
 
 /* kernel(X, Z, BLOCK): x = tl.load(X + tl.arange(0, BLOCK)); tl.store(Z, tl.<op>(x, axis=0))
  * The single-block reductions the reference's CI runs on its cpu/ path

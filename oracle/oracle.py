@@ -258,6 +258,19 @@ def binary_const(op: str, x: np.ndarray, c: float, *, flip: bool = False, block:
     return out
 
 
+def copy(x: np.ndarray, out: np.ndarray, n: int, *, block: int = 1024, grid: int | None = None) -> np.ndarray:
+    """The masked block moved unchanged: program p of ``grid`` stores out[i] = x[i] for the i of
+    [p*block, (p+1)*block) with i < n, and every other element of ``out`` keeps what it held
+    (masked load and store, cpu/lib/TritonCPUToLLVM/MaskedOpsToLLVM.cpp:33-114).  Any element type; bits move."""
+    grid = cdiv(max(n, 0), block) if grid is None else grid
+    x, out = x.reshape(-1), out.reshape(-1)
+    for p in range(grid):
+        lo, hi = p * block, min((p + 1) * block, n)
+        if lo < hi:
+            out[lo:hi] = x[lo:hi]
+    return out
+
+
 def trunci(x: np.ndarray, bits: int, *, block: int = 1024, grid: int | None = None) -> np.ndarray:
     """arith.trunci int32 -> int16 / int8 (ConvertComputeOps.cpp:182)."""
     x = np.ascontiguousarray(x, dtype=np.int32)

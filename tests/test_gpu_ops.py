@@ -148,3 +148,36 @@ def test_full_size_streaming_properties():
     del r
     q = K.unary("sqrt", x)
     assert float(((q * q - x).abs() / x).max()) <= 2 * 2.0 ** -23
+
+
+@pytest.mark.parametrize("dt", [torch.uint8, torch.int8, torch.int16, torch.bfloat16, torch.float16, torch.int32, torch.float32,
+                                torch.int64, torch.float64, torch.float8_e4m3fn])
+def test_copy_exact(dt):
+    """Bits move unchanged for every element width, every length around the vector and workgroup boundaries, and
+    operands off the 16-byte grid; what lies past the masked range keeps its contents."""
+    width = torch.empty(0, dtype=dt).element_size()
+    g = torch.Generator().manual_seed(5)
+    raw = torch.randint(0, 256, ((70001 + 64) * width, ), generator=g, dtype=torch.uint8)       # every bit pattern, NaNs included
+    for n in (1, 15, 16, 17, 4095, 4096, 4097, 16384, 16385, 70001):
+        x = raw[:n * width].cuda().view(dt)
+        out = torch.zeros(n + 8, dtype=torch.uint8).repeat_interleave(width).view(dt).cuda()
+        K.copy_kernel[(-(-n // 1024), )](x, out, n, BLOCK_SIZE=1024)
+        assert rt.last_kernel_name() == "ew_copy_b128"
+        want = np.zeros((n + 8) * width, dtype=np.uint8)
+        orc.copy(raw[:n * width].numpy(), want, n * width, block=1024 * width)
+        assert np.array_equal(out.view(torch.uint8).cpu().numpy(), want), (dt, n)
+    # off the 16-byte grid: one element in
+    n = 70001
+    src = raw[:(n + 1) * width].cuda().view(dt)[1:]
+    dst = torch.zeros((n + 2) * width, dtype=torch.uint8).cuda().view(dt)
+    K.copy_kernel[(-(-n // 1024), )](src, dst[1:], n, BLOCK_SIZE=1024)
+    assert rt.last_kernel_name() == f"ew_copy_b{8 * width}_unaligned"
+    got = dst.view(torch.uint8).cpu()
+    assert torch.equal(got[width:(n + 1) * width], raw[width:(n + 1) * width]) and not got[:width].any() and not got[(n + 1) * width:].any()
+    # a grid shorter than the data: three programs move 3072 elements
+    out = torch.zeros(n * width, dtype=torch.uint8).cuda().view(dt)
+    K.copy_kernel[(3, )](raw[:n * width].cuda().view(dt), out, n, BLOCK_SIZE=1024)
+    got = out.view(torch.uint8).cpu()
+    assert torch.equal(got[:3072 * width], raw[:3072 * width]) and not got[3072 * width:].any()
+    assert torch.equal(K.copy(x).view(torch.uint8), x.view(torch.uint8))
+

@@ -64,7 +64,7 @@ def fake(monkeypatch):
     monkeypatch.setattr(drv.TTDriver, "get_current_stream", lambda self, d=None: 0x1234)
     for k in (K.add_kernel, K.add_kernel_loop, K.sin_kernel, K.matmul_kernel_tma, K.matmul_kernel_fused, K._attn_fwd,
               K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel, K.unary_kernel, K.binary_kernel,
-              K.cast_kernel, K.reduce1d_kernel, K.binary_const_kernel):
+              K.cast_kernel, K.reduce1d_kernel, K.binary_const_kernel, K.copy_kernel):
         k._cache.clear()
     return lib
 
@@ -321,3 +321,14 @@ def test_constant_operand_kernel_binds(fake):
     assert a[1] == a[4] and a[2:4] == (2.0, 0)
     with pytest.raises(rt.Unsupported):
         K.binary_const_kernel[(5, )](x, o, 5000, BLOCK_SIZE=1024, OP="pow", C=2.0)
+
+
+def test_copy_kernel_binds(fake):
+    for dt, code in ((torch.float32, rt.TT_F32), (torch.int8, rt.TT_I8), (torch.int64, rt.TT_I64), (torch.bfloat16, rt.TT_BF16)):
+        x, o = FakeTensor((5000, ), dt), FakeTensor((5000, ), dt)
+        K.copy_kernel[(5, )](x, o, 5000, BLOCK_SIZE=1024)
+        name, a = fake.calls[-1]
+        assert name == "tt_copy_kernel" and a[2:5] == (5000, 1024, code)
+    with pytest.raises(rt.InvalidLaunch):
+        K.copy_kernel[(5, )](FakeTensor((5000, ), torch.float32), FakeTensor((5000, ), torch.int32), 5000, BLOCK_SIZE=1024)
+

@@ -105,3 +105,17 @@ def test_constant_operand_max_min_and_one_element_per_program():
     y = np.ones(10, np.float32)
     orc.binary_const("mul", y, 2.0, block=1, grid=4, out=y)       # a smaller grid touches its own elements only
     assert np.array_equal(y, [2, 2, 2, 2, 1, 1, 1, 1, 1, 1])
+
+
+def test_copy_moves_the_masked_block_and_nothing_else():
+    """Pinned by what a masked copy must do: the first min(n, grid*block) elements are the source's, bit for bit
+    (NaN payloads included), the rest of the destination is untouched; a ragged last block and a short grid."""
+    rng = np.random.default_rng(11)
+    for dt in (np.uint8, np.int16, np.float32, np.int64):
+        x = rng.integers(0, 255, 5000 * np.dtype(dt).itemsize, dtype=np.uint8).view(dt)
+        for n, block, grid in ((5000, 1024, None), (4097, 1024, None), (5000, 1024, 3), (10, 16, 10), (0, 16, 1)):
+            out = np.full(5000, 7, dtype=dt)
+            orc.copy(x, out, n, block=block, grid=grid)
+            moved = min(n, (orc.cdiv(n, block) if grid is None else grid) * block)
+            assert out[:moved].tobytes() == x[:moved].tobytes() and np.all(out[moved:] == 7), (dt, n, block, grid)
+

@@ -428,6 +428,122 @@ def test_load_store_same_ptr_runs(tmp_path, monkeypatch):
         triton.runtime.driver._active = None
 
 
+# --- the kernels of test_launch.py, which the reference's CI runs on its cpu/ path
+# (.github/workflows/integration-tests-cpu.yml:106): an empty kernel under the launch hooks and a masked copy whose
+# bound is a constant of the kernel, launched in a loop under tracemalloc ---
+@triton.jit
+def copy_first_ten(src_ptr, dst_ptr, count, BLOCK: tl.constexpr):
+    count = 10
+    idx = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    keep = idx < count
+    v = tl.load(src_ptr + idx, keep)
+    tl.store(dst_ptr + (idx + tl.zeros([BLOCK], tl.int32)), v, keep)
+
+
+@triton.jit
+def user_copy(src_ptr, dst_ptr, n, BLOCK: tl.constexpr):
+    offs = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+    tl.store(dst_ptr + offs, tl.load(src_ptr + offs, mask=offs < n), mask=offs < n)
+
+
+def _describe_launch(grid, kernel, args):
+    return {"grid": grid, "value": args["x"]}
+
+
+@triton.jit(launch_metadata=_describe_launch)
+def does_nothing(x):
+    pass
+
+
+def test_copy_and_empty_kernels_are_recognised(tmp_path, monkeypatch):
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    m = json.loads(_compile(copy_first_ten, {"src_ptr": "*fp32", "dst_ptr": "*fp32", "count": "i32", "BLOCK": "constexpr"},
+                            {"BLOCK": 16}).kernel)["match"]
+    assert m == {"kernel": "copy_kernel", "op": None, "inputs": ["src_ptr"], "output": "dst_ptr", "n": None, "n_const": 10,
+                 "block": 16, "dtype": 0}
+    for ty, code in (("*i8", 6), ("*u8", 6), ("*bf16", 2), ("*i64", 7), ("*fp64", 8), ("*u16", 5)):
+        m = json.loads(_compile(user_copy, {"src_ptr": ty, "dst_ptr": ty, "n": "i32", "BLOCK": "constexpr"},
+                                {"BLOCK": 256}).kernel)["match"]
+        assert (m["kernel"], m["n"], m["block"], m["dtype"]) == ("copy_kernel", "n", 256, code), ty
+    k = _compile(does_nothing, {"x": "i32"}, {})
+    assert json.loads(k.kernel)["match"] == {"kernel": "empty_kernel"}
+
+    @triton.jit
+    def copy_between_types(src_ptr, dst_ptr, n, BLOCK: tl.constexpr):     # the store widens: neither a copy nor a narrowing cast
+        offs = tl.program_id(0) * BLOCK + tl.arange(0, BLOCK)
+        tl.store(dst_ptr + offs, tl.load(src_ptr + offs, mask=offs < n), mask=offs < n)
+
+    with pytest.raises(RuntimeError, match="no prebuilt gfx950 implementation"):
+        _compile(copy_between_types, {"src_ptr": "*fp16", "dst_ptr": "*fp32", "n": "i32", "BLOCK": "constexpr"}, {"BLOCK": 256})
+
+
+@pytest.mark.gpu
+def test_launch_hooks_and_no_leak_through_the_jit(tmp_path, monkeypatch):
+    import gc
+    import tracemalloc
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton_tenstorrent_amd import runtime as rt
+    ttc.register()
+    seen = []
+
+    def first(launch_metadata):
+        md = launch_metadata.get()
+        assert md["grid"] == (1, 3, 2) and md["value"] == 6
+        seen.append("first")
+
+    def second(launch_metadata):
+        seen.append("second")
+
+    def after(launch_metadata):
+        seen.append("after")
+
+    try:
+        triton.knobs.runtime.launch_enter_hook.add(first)
+        triton.knobs.runtime.launch_enter_hook.add(second)
+        triton.knobs.runtime.launch_exit_hook.add(after)
+        try:
+            does_nothing[(1, 3, 2)](6)
+        finally:
+            triton.knobs.runtime.launch_enter_hook.remove(first)
+            triton.knobs.runtime.launch_enter_hook.remove(second)
+            triton.knobs.runtime.launch_exit_hook.remove(after)
+        assert seen == ["first", "second", "after"]
+        does_nothing[(1, 3, 2)](6)
+        assert seen == ["first", "second", "after"]                    # removed hooks stay removed
+
+        inp, out = torch.randn(10, device="cuda"), torch.randn(10, device="cuda")
+        tracemalloc.start()
+        try:
+            copy_first_ten[(10, )](inp, out, 10, BLOCK=16)
+            gc.collect()
+            begin, _ = tracemalloc.get_traced_memory()
+            for _ in range(100):
+                copy_first_ten[(10, )](inp, out, 10, BLOCK=16)
+            gc.collect()
+            end, _ = tracemalloc.get_traced_memory()
+        finally:
+            tracemalloc.stop()
+        assert end - begin < 30000                                     # the upstream test's bound
+        assert torch.equal(out, inp) and rt.last_kernel_name() == "ew_copy_b128"
+
+        # the bound is the kernel's constant, not the argument: 10 of 64 elements move
+        src = torch.arange(64, device="cuda", dtype=torch.int16)
+        dst = torch.full((64, ), -1, device="cuda", dtype=torch.int16)
+        copy_first_ten[(4, )](src, dst, 64, BLOCK=16)
+        assert torch.equal(dst[:10], src[:10]) and torch.all(dst[10:] == -1)
+        with pytest.raises(Exception, match="holds fewer"):
+            copy_first_ten[(1, )](src[:4], dst, 64, BLOCK=16)
+
+        big = torch.randint(-2**62, 2**62, (70001, ), device="cuda", dtype=torch.int64)
+        got = torch.zeros(70001 + 5, device="cuda", dtype=torch.int64)
+        user_copy[(triton.cdiv(70001, 512), )](big, got, 70001, BLOCK=512)
+        assert torch.equal(got[:70001], big) and not got[70001:].any()
+    finally:
+        from triton.backends import backends
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver._active = None
+
+
 # --- autotune and do_bench through the plugin's device interface (driver.py:390-442 of the reference) ---
 @triton.autotune(configs=[triton.Config({"BLOCK_SIZE": 512}), triton.Config({"BLOCK_SIZE": 1024}),
                           triton.Config({"BLOCK_SIZE": 2048})], key=["n_elements"])

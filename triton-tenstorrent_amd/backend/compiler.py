@@ -20,7 +20,7 @@ from types import ModuleType
 from typing import Dict, Tuple
 
 from .driver import BINARY_EXT, KERNEL_TABLE, GPUTarget, TTDriver
-from .patterns import match_per_program, match_reduce1d, match_streaming
+from .patterns import match_empty, match_per_program, match_reduce1d, match_streaming
 
 try:
     from triton.backends.compiler import BaseBackend, Language
@@ -161,7 +161,7 @@ class TTBackend(BaseBackend):
         if name not in KERNEL_TABLE:
             # not one of the example kernels by name: a kernel of the masked-block elementwise form is
             # bound by what its IR says it does (one operation of the reference's opcode set)
-            match = match_streaming(text) or match_reduce1d(text) or match_per_program(text)
+            match = match_streaming(text) or match_reduce1d(text) or match_per_program(text) or match_empty(text)
             if match is None:
                 raise RuntimeError(f"kernel '{name}' has no prebuilt gfx950 implementation; this backend runs "
                                    f"{sorted(KERNEL_TABLE)}, and elementwise kernels of the masked-block form with "

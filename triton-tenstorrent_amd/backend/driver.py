@@ -255,6 +255,22 @@ def _bind_cast(lib, cur, consts, grid, stream):
                               _torch_dtype_code(out), grid, stream)
 
 
+def _bind_copy(lib, cur, consts, grid, stream):
+    """out[i] = x[i] for i < n_elements: a masked block loaded and stored back unchanged, any element type
+    (the kernel of test_launch.py::test_memory_leak, .github/workflows/integration-tests-cpu.yml:106)."""
+    x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
+    n = int(cur.scalar("n_elements"))
+    cur.done()
+    if x.dtype != out.dtype:
+        raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"copy_kernel moves one element type, got {x.dtype} and {out.dtype}")
+    return lib.tt_copy_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), _torch_dtype_code(x), grid, stream)
+
+
+def _bind_empty(lib, cur, consts, grid, stream):
+    """A kernel with an empty body: the launch hooks run, nothing is sent to the device."""
+    return rt.RT_OK
+
+
 _FLOATS = (rt.TT_F32, rt.TT_BF16, rt.TT_F16, rt.TT_F64)
 _UNSIGNED = (rt.TT_U8, rt.TT_U16, rt.TT_U32, rt.TT_U64)
 _NARROW = (rt.TT_I8, rt.TT_I16, rt.TT_U8, rt.TT_U16, rt.TT_BF16, rt.TT_F16)
@@ -388,6 +404,8 @@ def _bind_matched(match: dict, lib, cur, consts, grid, stream):
     and BLOCK from the IR."""
     vals = cur.named()
     cur.done()
+    if match["kernel"] == "empty_kernel":
+        return rt.RT_OK
     tensors = [vals[n] for n in match["inputs"]] + [vals[match["output"]]]
     for t in tensors:
         if not hasattr(t, "data_ptr") or not t.is_cuda:
@@ -410,6 +428,13 @@ def _bind_matched(match: dict, lib, cur, consts, grid, stream):
             n = int(grid[0])
         return lib.tt_binary_const_kernel(rt.BINARY_OPS[match["op"]], ptrs[0], float(match["c"]), int(match["flip"]), ptrs[1],
                                           n, block, grid, stream)
+    if match["kernel"] == "copy_kernel":
+        if tensors[0].dtype != tensors[1].dtype:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "copy_kernel moves one element type")
+        touched = min(max(n, 0), int(grid[0]) * block)
+        if min(t.numel() for t in tensors) < touched:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"the kernel moves {touched} elements, a tensor holds fewer")
+        return lib.tt_copy_kernel(ptrs[0], ptrs[1], n, block, match["dtype"], grid, stream)
     if match["kernel"] == "muladd_kernel":
         return lib.tt_muladd_kernel(ptrs[0], ptrs[1], ptrs[2], ptrs[3], n, block, grid, stream)
     if match["kernel"] == "add_kernel":
@@ -430,6 +455,8 @@ KERNEL_TABLE: dict[str, Callable] = {
     "binary_kernel": _bind_binary,
     "cast_kernel": _bind_cast,
     "binary_const_kernel": _bind_binary_const,
+    "copy_kernel": _bind_copy,
+    "empty_kernel": _bind_empty,
     "reduce1d_kernel": _bind_reduce1d,
     "matmul_kernel_tma": _bind_matmul_tma,
     "matmul_kernel_tma_fp8_scaled": _bind_matmul_tma,

@@ -29,6 +29,8 @@ UNARY = {"math.absf": "abs", "math.ceil": "ceil", "math.cos": "cos", "math.exp":
 BINARY = {"arith.addf": "add", "arith.subf": "sub", "arith.mulf": "mul", "arith.divf": "div",
           "arith.maximumf": "maximum", "arith.minimumf": "minimum"}
 CASTS = {"arith.truncf", "arith.trunci"}
+# element types a copy moves, as tt_dtype codes (unsigned integers arrive as the signed type of their width)
+_COPY_ELEM = {"f32": 0, "i32": 1, "bf16": 2, "f16": 3, "f8E4M3FN": 4, "i16": 5, "i8": 6, "i64": 7, "f64": 8}
 _PLUMBING = {"tt.get_program_id", "arith.constant", "arith.muli", "tt.make_range", "tt.splat", "arith.addi",
              "arith.cmpi", "tt.addptr", "tt.load", "tt.store", "tt.return"}
 
@@ -95,9 +97,15 @@ def match_streaming(ttir: str) -> dict | None:
             return None
         if res:
             defs[res] = (op, operands, rest)
-    if len(store) != 1 or len(compute) not in (1, 2):
+    if len(store) != 1 or len(compute) not in (0, 1, 2):
         return None
-    if len(compute) == 2:
+    if not compute:
+        # the loaded block stored back unchanged: the copy kernel of test_launch.py::test_memory_leak
+        # (.github/workflows/integration-tests-cpu.yml:106)
+        if len(store[0][0]) != 3:
+            return None
+        res, op, operands = store[0][0][1], "copy", [store[0][0][1]]
+    elif len(compute) == 2:
         # x * y + z, contracted to one fused multiply-add (01-vector-mul-add.py:30-57; enable_fp_fusion)
         (mres, mop, mops, _), (ares, aop, aops, _) = compute
         if mop != "arith.mulf" or aop != "arith.addf" or mres not in aops or len(aops) != 2:
@@ -145,15 +153,21 @@ def match_streaming(ttir: str) -> dict | None:
     if not md or md[0] != "arith.cmpi" or not md[2].lstrip().startswith("slt") or md[1][0] != offsets:
         return None
     ns = defs.get(md[1][1])
-    if not ns or ns[0] != "tt.splat":
-        return None
-    n_src = ns[1][0] if ns[1] else None
-    n_const = None
-    if n_src not in arg_types:                 # n_elements folded to a constant (the value 1)
-        c = defs.get(n_src)
-        if not c or c[0] != "arith.constant":
+    n_src, n_const = None, None
+    if ns and ns[0] == "arith.constant":       # the bound is a constant of the kernel: dense<N> : tensor<BLOCKxi32>
+        cm = re.match(r"\s*dense<(-?\d+)>\s*:\s*tensor<\d+xi32>", ns[2])
+        if not cm:
             return None
-        n_const = int(re.match(r"\s*(-?\d+)", c[2]).group(1))
+        n_const = int(cm.group(1))
+    elif ns and ns[0] == "tt.splat":
+        n_src = ns[1][0] if ns[1] else None
+        if n_src not in arg_types:             # n_elements folded to a constant (the value 1)
+            c = defs.get(n_src)
+            if not c or c[0] != "arith.constant":
+                return None
+            n_const = int(re.match(r"\s*(-?\d+)", c[2]).group(1))
+    else:
+        return None
     # offsets = splat(pid * BLOCK) + make_range(0, BLOCK), either order
     od = defs.get(offsets)
     if not od or od[0] != "arith.addi" or len(od[1]) != 2:
@@ -176,7 +190,12 @@ def match_streaming(ttir: str) -> dict | None:
     # element types
     in_types = {arg_types[a] for a in inputs}
     out_type = arg_types[out_arg]
-    if op == "muladd":
+    if op == "copy":
+        elem = re.fullmatch(r"!tt\.ptr<(\w+)>", out_type)
+        if in_types != {out_type} or len(inputs) != 1 or not elem or elem.group(1) not in _COPY_ELEM:
+            return None
+        kernel, opname = "copy_kernel", None
+    elif op == "muladd":
         if in_types != {"!tt.ptr<f32>"} or out_type != "!tt.ptr<f32>" or len(inputs) != 3:
             return None
         kernel, opname = "muladd_kernel", None
@@ -210,7 +229,19 @@ def match_streaming(ttir: str) -> dict | None:
            "n": strip(n_src) if n_const is None else None, "n_const": n_const, "block": block}
     if kernel == "binary_const_kernel":
         rec.update(c=const_operand[1], flip=const_operand[0] == 0)
+    if kernel == "copy_kernel":
+        rec.update(dtype=_COPY_ELEM[elem.group(1)])
     return rec
+
+
+def match_empty(ttir: str) -> dict | None:
+    """A kernel whose body is ``tt.return`` alone (``def kernel(x): pass``, the kernel the hook tests of
+    test_launch.py launch, .github/workflows/integration-tests-cpu.yml:106): nothing to run on the device."""
+    parsed = _body(ttir)
+    if parsed is None:
+        return None
+    body = [l for l in (_LOC.sub("", raw).strip() for raw in parsed[2]) if l]
+    return {"kernel": "empty_kernel"} if body == ["tt.return"] else None
 
 
 _ELEM = {"f32": 0, "i32": 1, "bf16": 2, "f16": 3, "i16": 5, "i8": 6, "i64": 7, "f64": 8}

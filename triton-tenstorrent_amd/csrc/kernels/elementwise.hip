@@ -266,6 +266,39 @@ template <typename Op> __device__ __forceinline__ void unary_scalar_body(const f
   for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = Op::apply(x[i]);
 }
 
+// ---- copy: a masked load stored back unchanged ---------------------------------------
+// Bytes, not elements: with both pointers on 16-byte boundaries every lane moves 16-byte vectors whatever the
+// element type is, and the last workgroup moves the bytes past the last whole vector one at a time.
+template <int UNROLL>
+__device__ __forceinline__ void copy_vec_body(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
+                                              uint64_t nbytes) {
+  using V = Vec4<uint32_t>::type;
+  const uint32_t nvec = (uint32_t)(nbytes >> 4);
+  const V *xv = reinterpret_cast<const V *>(x);
+  V *ov = reinterpret_cast<V *>(out);
+  const uint32_t base = blockIdx.x * (kThreads * UNROLL);
+  const uint32_t i = base + threadIdx.x;
+  if (base + kThreads * UNROLL <= nvec) {
+    V a[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) a[u] = __builtin_nontemporal_load(xv + i + u * kThreads);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) __builtin_nontemporal_store(a[u], ov + i + u * kThreads);
+  } else {
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const uint32_t j = i + u * kThreads;
+      if (j < nvec) ov[j] = xv[j];
+    }
+    const uint64_t t = ((uint64_t)nvec << 4) + threadIdx.x;
+    if (threadIdx.x < 16 && t < nbytes) out[t] = x[t];
+  }
+}
+template <typename T> __device__ __forceinline__ void copy_scalar_body(const T *x, T *out, uint32_t n) {
+  const uint32_t stride = gridDim.x * kThreads;
+  for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = x[i];
+}
+
 // ---- narrowing conversions (arith.truncf, arith.trunci) ---------------------------
 // One element per lane and pass, grid-stride: 4-byte loads and 1- or 2-byte stores coalesce per
 // wavefront; these are conversions at the edge of a pipeline, not streaming hot spots.
@@ -454,5 +487,17 @@ __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restric
       out[i] = MulAdd::apply(x[i], y[i], z[i]);
   }
 }
+
+__global__ __launch_bounds__(kThreads) void ew_copy_b128(const uint8_t *x, uint8_t *out, uint64_t nbytes) {
+  copy_vec_body<4>(x, out, nbytes);
+}
+#define EW_COPY_UNALIGNED(name, T)                                                     \
+  __global__ __launch_bounds__(kThreads) void name(const T *x, T *out, uint32_t n) {   \
+    copy_scalar_body<T>(x, out, n);                                                    \
+  }
+EW_COPY_UNALIGNED(ew_copy_b8_unaligned, uint8_t)
+EW_COPY_UNALIGNED(ew_copy_b16_unaligned, uint16_t)
+EW_COPY_UNALIGNED(ew_copy_b32_unaligned, uint32_t)
+EW_COPY_UNALIGNED(ew_copy_b64_unaligned, uint64_t)
 
 } // extern "C"

@@ -207,4 +207,32 @@ int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_S
   return launch("elementwise", name, dim3(streaming_grid(n_eff, false)), dim3(kThreads), 0, stream, args, 3);
 }
 
+int tt_copy_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE, int32_t dtype,
+                   const uint32_t grid[3], void *stream) {
+  if (!props()) return fail(RT_ERR_NOT_INIT, "copy_kernel: call rt_init first");
+  const int64_t width = dtype_size(dtype);
+  if (width <= 0) return fail(RT_ERR_UNSUPPORTED, "copy_kernel: dtype %d", dtype);
+  uint32_t n_eff = 0;
+  int rc = check_1d("copy_kernel", n_elements, BLOCK_SIZE, grid, &n_eff);
+  if (rc) return rc;
+  if (n_eff == 0) return RT_OK;
+  if (!x || !out) return fail(RT_ERR_INVALID, "copy_kernel: null tensor pointer");
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & (uintptr_t)(width - 1))
+    return fail(RT_ERR_INVALID, "copy_kernel: pointers must be aligned to the %lld-byte element", (long long)width);
+  if (aligned16(x) && aligned16(out)) {
+    uint64_t nbytes = (uint64_t)n_eff * (uint64_t)width;
+    // one workgroup per run of kThreads * kUnroll 16-byte vectors; the one after the last whole run takes the
+    // ragged end of the vectors and the bytes past the last vector
+    const uint64_t nvec = nbytes >> 4, per_wg = kThreads * kUnroll;
+    uint64_t wgs = nvec / per_wg;
+    if (wgs * per_wg < nvec || (nbytes & 15u)) ++wgs;
+    void *args[] = {&x, &out, &nbytes};
+    return launch("elementwise", "ew_copy_b128", dim3((uint32_t)wgs), dim3(kThreads), 0, stream, args, 3);
+  }
+  char name[48];
+  snprintf(name, sizeof(name), "ew_copy_b%d_unaligned", (int)width * 8);
+  void *args[] = {&x, &out, &n_eff};
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, false)), dim3(kThreads), 0, stream, args, 3);
+}
+
 } // extern "C"

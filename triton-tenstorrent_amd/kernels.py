@@ -73,6 +73,17 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+copy_kernel = PrebuiltKernel("copy_kernel", ["x_ptr", "output_ptr", "n_elements", "BLOCK_SIZE"], ["BLOCK_SIZE"])
+
+
+def copy(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``out[i] = x[i]``: the masked block loaded and stored back unchanged, any element type."""
+    out = torch.empty_like(x) if out is None else out
+    n = x.numel()
+    copy_kernel[lambda meta: (cdiv(n, meta["BLOCK_SIZE"]), )](x, out, n, BLOCK_SIZE=1024)
+    return out
+
+
 reduce1d_kernel = PrebuiltKernel("reduce1d_kernel", ["X", "Z", "BLOCK", "OP", "PROPAGATE_NAN"], ["BLOCK", "OP", "PROPAGATE_NAN"],
                                  defaults={"PROPAGATE_NAN": False})
 

@@ -94,6 +94,7 @@ SYMBOLS = {
     "tt_binary_kernel": (C.c_int, [_i32, _vp, _vp, _vp, _i32, _i32, _G, _vp]),
     "tt_binary_const_kernel": (C.c_int, [_i32, _vp, _f32, _i32, _vp, _i32, _i32, _G, _vp]),
     "tt_cast_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _G, _vp]),
+    "tt_copy_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _G, _vp]),
     "tt_reduce1d_kernel": (C.c_int, [_i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_fused": (C.c_int, [_DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
