@@ -346,6 +346,33 @@ def test_fast_path_strided_rows_and_epilogues():
     assert rt.last_kernel_name() == "gemm_tile_bf16_epi4" and close_bf16(decode(cr), ref, RTOL, ATOL)
 
 
+# Shapes whose macro tiles do not fill the last round of the persistent grid: the kernel finishes the tail as
+# half tiles, two workgroups per tile.  With 256 CUs: 272 tiles = one round + 16 (dealt in groups of 8 tiles),
+# 289 = one round + 33 (dealt in pairs), 64 and 15 tiles = tail only.
+@pytest.mark.parametrize("M,N,K_", [(4352, 4096, 256), (4352, 4352, 128), (2048, 2048, 256), (768, 1280, 640)])
+def test_fast_path_half_tile_tail(M, N, K_):
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-4, 5, (M, K_), generator=g).to(torch.bfloat16).cuda()
+    b = torch.randint(-4, 5, (K_, N), generator=g).to(torch.bfloat16).cuda()
+    c = K.matmul_tma(a, b)
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi0"
+    assert torch.equal(c, (a.float() @ b.float()).to(torch.bfloat16))       # small integers: every sum is exact in fp32
+    # random operands against the oracle, with the GELU epilogue (row bias indexed by the half tile's columns)
+    a, b = _ab(M, N, K_, seed=M * 3 + N)
+    bias = (torch.randn(N, generator=g) * 0.02)
+    cg = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda(), epilogue="gelu")
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi2"
+    ref = orc.from_bf16(orc.matmul(bits(a), bits(b), bias=bias.numpy(), epi=orc.EPI_BIAS_ROW_GELU, acc64=True))
+    assert close_bf16(decode(cg), ref, RTOL, ATOL)
+    # strided C with a sentinel beside it: the half tiles store their own rows only
+    cbuf = torch.full((M, N + 8), 7.5, dtype=torch.float16, device="cuda")
+    ah, bh = a.to(torch.float16).cuda(), b.to(torch.float16).cuda()
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (ah, bh, cbuf[:, :N]))
+    K.matmul_kernel_tma[((M // 128) * (N // 128), )](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert rt.last_kernel_name() == "gemm_tile_f16_epi0" and torch.all(cbuf[:, N:] == 7.5)
+    _check(cbuf[:, :N].cpu(), ah.cpu(), bh.cpu())
+
+
 def test_full_size_8192_properties():
     """BASELINE's 8192^3: checked through size-independent properties -- B = I gives C = A
     bit for bit, linearity in A, and sampled rows against fp64 on the host."""

@@ -176,3 +176,19 @@ def test_full_size_tiled_identity_and_scaling():
     ref = (a[rows].double() @ b.double()).float()
     got = K.untilize(c1, n, n, 32, 32)[rows].float()
     assert torch.all((got - ref).abs() <= 1e-2 * ref.abs() + 1e-4)
+
+
+@pytest.mark.parametrize("M,N,K_", [(4352, 4096, 256), (4352, 4352, 128), (1024, 2048, 384)])
+def test_tiled_fast_kernel_half_tile_tail(M, N, K_):
+    """Macro-tile counts that leave a short last round (272 and 289 tiles on 256 CUs) or no whole round at all
+    (32): the tail runs as half tiles.  Small integers, so the result is exact whatever the order."""
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-3, 4, (M, K_), generator=g).to(torch.float16)
+    b = torch.randint(-3, 4, (K_, N), generator=g).to(torch.float16)
+    for act in ("", "leaky_relu"):
+        ct = K.matmul_tiled(K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, K_, activation=act)
+        assert rt.last_kernel_name() == f"gemm_tiled_f16_epi{3 if act else 0}"
+        want = a.cuda().float() @ b.cuda().float()
+        want = torch.where(want >= 0, want, 0.01 * want) if act else want
+        assert torch.equal(K.untilize(ct, M, N, 32, 32), want.to(torch.float16))
+

@@ -102,8 +102,16 @@ struct Ring {
 // contiguous, i.e. exactly 32 of this kernel's 64-byte LDS rows, so only the global addresses
 // of the copies and of the result change: a thread's offset inside a slab, the distance
 // between slabs and between K steps.  LDS layout, fragments and MFMA schedule are the same.
-template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false>
+//
+// MB: 32-row blocks of C per wavefront.  4 is the 256x256 macro tile described above.  With 2 a workgroup
+// computes a 128x256 HALF of a macro tile (each wavefront 64x128: 2x4 accumulators, two A slabs and six
+// copies per step, eight MFMAs per sub-step), used for the tail of the persistent loop: when the macro
+// tiles left over after the last whole round of the grid would keep at most half of the workgroups busy,
+// the kernel runs body<MB=4> over the whole rounds and then body<MB=2> over the halves of the tail tiles,
+// two workgroups per tile, instead of leaving half of the chip idle for a whole tile's time.
+template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
+  static_assert(MB == 4 || (MB == 2 && SPLIT_TAIL && !RAGGED), "half tiles exist for the tail of the plain kernels only");
   // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
   // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
   // real M and N (the padding of C is never written, as under the reference's store mask).
@@ -115,7 +123,39 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
-  const int total = tiles_m * tiles_n;
+  const int total_tiles = tiles_m * tiles_n;
+  // Work items of this pass: macro tiles (MB == 4) or halves of the tail's macro tiles (MB == 2).
+  int total = total_tiles, first_tile = 0, tail_tiles = 0;
+  if constexpr (SPLIT_TAIL) {
+    const int whole = total_tiles / (int)gridDim.x * (int)gridDim.x;
+    tail_tiles = total_tiles - whole;
+    const bool split = tail_tiles > 0 && 2 * tail_tiles <= (int)gridDim.x;
+    if (MB == 4) {
+      total = split ? whole : total_tiles;
+    } else {
+      total = split ? 2 * tail_tiles : 0;
+      first_tile = whole;
+    }
+  }
+  // item -> macro tile and which half of it.  Workgroup ids go round-robin over the 8 XCDs and tile_of gives
+  // tile t to XCD t % 8's run of ids, so halves are dealt in groups of 16 items over 8 tiles: both halves of
+  // a tile then stay on the XCD that tile's neighbours ran on.
+  auto item_tile = [&](int item, int &tm, int &tn, int &half) {
+    if constexpr (MB == 4) {
+      half = 0;
+      tile_of(item, tiles_m, tiles_n, tm, tn);
+    } else {
+      int j;
+      if (tail_tiles % 8 == 0) {
+        j = (item >> 4) * 8 + (item & 7);
+        half = (item >> 3) & 1;
+      } else {
+        j = item >> 1;
+        half = item & 1;
+      }
+      tile_of(first_tile + j, tiles_m, tiles_n, tm, tn);
+    }
+  };
   const int nk_real = Kf / BK;                                    // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
@@ -142,7 +182,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
   // ---- LDS -> fragments ----
   const int l32 = lane & 31, hi = lane >> 5;
-  const int a_base = (wm * 128 + l32) * 64;
+  const int a_base = (wm * (32 * MB) + l32) * 64;
   const int a_x = (l32 >> 2) & 3;
   int a_pos[2]; // sub-step s: logical chunk 2s + hi
 #pragma unroll
@@ -161,20 +201,20 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // Fragment registers: two sets (even / odd sub-steps).  B fragments are kept as their
   // two transposed halves (k 0-3 and k 4-7 of the lane's group).
   struct Frags {
-    vec a[4];
+    vec a[MB];
     union { s16x4 h[2]; vec v; } b[4];
   };
   Frags f0, f1;
-  f32x16 acc[4][4]; // [m-tile][n-tile]
+  f32x16 acc[MB][4]; // [m-tile][n-tile]
 
   // The 12 LDS reads of one sub-step, in the order the MFMAs will want them:
-  // b0.lo b0.hi a0 b1.lo b1.hi b2.lo b2.hi b3.lo b3.hi a1 a2 a3
+  // b0.lo b0.hi a0 b1.lo b1.hi b2.lo b2.hi b3.lo b3.hi a1 a2 a3        (MB == 2: the first ten)
   auto rd = [&](Frags &f, const uint8_t *stage, int s, int r) {
     switch (r) {
     case 2: f.a[0] = *(const vec *)(stage + a_pos[s]); break;
     case 9: f.a[1] = *(const vec *)(stage + a_pos[s] + 2048); break;
-    case 10: f.a[2] = *(const vec *)(stage + a_pos[s] + 4096); break;
-    case 11: f.a[3] = *(const vec *)(stage + a_pos[s] + 6144); break;
+    case 10: if constexpr (MB == 4) f.a[2] = *(const vec *)(stage + a_pos[s] + 4096); break;
+    case 11: if constexpr (MB == 4) f.a[3] = *(const vec *)(stage + a_pos[s] + 6144); break;
     default: {
       const int rr = r < 2 ? r : r - 1; // 0..7 over the b reads
       const int j = rr >> 1, h = rr & 1;
@@ -183,7 +223,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     }
     }
   };
-  // MFMA number n (0..15) of a sub-step, m-tile major: needs a[n/4], b[n%4]
+  // MFMA number n (0..4*MB-1) of a sub-step, m-tile major: needs a[n/4], b[n%4]
   auto mm = [&](Frags &f, int n) {
     const int i = n >> 2, j = n & 3;
     acc[i][j] = X::run(f.b[j].v, f.a[i], acc[i][j]);
@@ -213,9 +253,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   Voffs vo_cur, vo_nxt;
   const uint32_t z_voff = (uint32_t)tid * 16;
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
-    int tm, tn;
-    tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
-    ap = A + (TILED ? (int64_t)tm * (BM / 32) * ntk * 2048 : (int64_t)tm * BM * g.lda * 2);
+    int tm, tn, half;
+    item_tile(min(t, total - 1), tm, tn, half);
+    const int64_t row0 = (int64_t)tm * BM + half * 128;
+    ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
     if constexpr (RAGGED) {
       const int last_row = Mf - 1 - tm * BM;                  // >= 0
@@ -231,7 +272,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                    : (uint32_t)(((int64_t)b_k * g.ldb + cc * 8) * 2);
     }
   };
-  // copy number i (0..3: A slabs, 4..7: B slabs) of step kk into `stage`; kk may run past
+  // copy number i (0..MB-1: A slabs, MB..MB+3: B slabs) of step kk into `stage`; kk may run past
   // nk into the next tile
   auto dma_single = [&](int kk, uint8_t *stage, int i) {
     const bool over = kk >= nk;
@@ -246,12 +287,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - 4) * b_slab;
         dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - 4) * 4096);
       }
-    } else if (i < 4) {
+    } else if (i < MB) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
-      dma_one(bp + (i - 4) * b_slab, b_voff, stage + A_BYTES + (i - 4) * 4096);
+      dma_one(bp + (i - MB) * b_slab, b_voff, stage + A_BYTES + (i - MB) * 4096);
     }
   };
 
@@ -265,34 +306,62 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   auto step = [&](auto I_, int k) {
     constexpr int I = decltype(I_)::value;
     uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R], *prv = ring.s[(I + R - 1) % R];
-    // sub-step 0: MFMAs on f0; sub-step 1's fragments ride along (two reads per MFMA);
-    // second half of the refill of the stage freed one step ago
-#pragma unroll
-    for (int n = 0; n < 16; ++n) {
-      if (n < 6) {
-        rd(f1, cur, 1, 2 * n);
-        rd(f1, cur, 1, 2 * n + 1);
+    if constexpr (MB == 4) {
+      // sub-step 0: MFMAs on f0; sub-step 1's fragments ride along (two reads per MFMA);
+      // second half of the refill of the stage freed one step ago
+  #pragma unroll
+      for (int n = 0; n < 16; ++n) {
+        if (n < 6) {
+          rd(f1, cur, 1, 2 * n);
+          rd(f1, cur, 1, 2 * n + 1);
+        }
+        if ((n & 3) == 1) dma_single(k - 1 + R, prv, 4 + (n >> 2));
+        mm(f0, n);
+        FENCE();
       }
-      if ((n & 3) == 1) dma_single(k - 1 + R, prv, 4 + (n >> 2));
-      mm(f0, n);
+      // All of this wave's reads of stage I have returned, and so has its share of the
+      // copy into stage I+1 (the 16 younger copies may still be in flight).  After the
+      // barrier that holds for every wave: I+1 may be read, I may be overwritten.
+      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       FENCE();
-    }
-    // All of this wave's reads of stage I have returned, and so has its share of the
-    // copy into stage I+1 (the 16 younger copies may still be in flight).  After the
-    // barrier that holds for every wave: I+1 may be read, I may be overwritten.
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    FENCE();
-    // sub-step 1: MFMAs on f1; the next stage's sub-step 0 fragments; first half of the
-    // refill of stage I with step k+R
-#pragma unroll
-    for (int n = 0; n < 16; ++n) {
-      if (n < 6) {
-        rd(f0, nxt, 0, 2 * n);
-        rd(f0, nxt, 0, 2 * n + 1);
+      // sub-step 1: MFMAs on f1; the next stage's sub-step 0 fragments; first half of the
+      // refill of stage I with step k+R
+  #pragma unroll
+      for (int n = 0; n < 16; ++n) {
+        if (n < 6) {
+          rd(f0, nxt, 0, 2 * n);
+          rd(f0, nxt, 0, 2 * n + 1);
+        }
+        if ((n & 3) == 1) dma_single(k + R, cur, n >> 2);
+        mm(f1, n);
+        FENCE();
       }
-      if ((n & 3) == 1) dma_single(k + R, cur, n >> 2);
-      mm(f1, n);
+    } else {
+      // Half tiles: the same step with eight MFMAs per sub-step, ten fragment reads (two per MFMA over the
+      // first five) and six copies: the four B slabs of step k-1+R in sub-step 0, the two A slabs of step
+      // k+R in sub-step 1.  At the barrier the two youngest steps' copies (12) may still be in flight.
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {
+        if (n < 5) {
+          rd(f1, cur, 1, 2 * n);
+          rd(f1, cur, 1, 2 * n + 1);
+        }
+        if (n & 1) dma_single(k - 1 + R, prv, MB + (n >> 1));
+        mm(f0, n);
+        FENCE();
+      }
+      asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       FENCE();
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {
+        if (n < 5) {
+          rd(f0, nxt, 0, 2 * n);
+          rd(f0, nxt, 0, 2 * n + 1);
+        }
+        if ((n & 3) == 1) dma_single(k + R, cur, n >> 2);
+        mm(f1, n);
+        FENCE();
+      }
     }
   };
 
@@ -305,18 +374,22 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #pragma unroll
   for (int s = 0; s < R; ++s)
 #pragma unroll
-    for (int i = 0; i < (s == R - 1 ? 4 : 8); ++i) dma_single(s, ring.s[s], i);
-  static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume 8 copies per step and 4 stages");
-  asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
+    for (int i = 0; i < (s == R - 1 ? MB : MB + 4); ++i) dma_single(s, ring.s[s], i);
+  static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
+  // everything issued but step 0's own MB + 4 copies may still be in flight: 2 * (MB + 4) + MB
+  if constexpr (MB == 4)
+    asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
+  else
+    asm volatile("s_waitcnt vmcnt(14) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-  for (int r = 0; r < 12; ++r) rd(f0, ring.s[0], 0, r);
+  for (int r = 0; r < 8 + MB; ++r) rd(f0, ring.s[0], 0, r);
 
   for (; t < total; t += gridDim.x) {
-    int tm, tn;
-    tile_of(t, tiles_m, tiles_n, tm, tn);
-    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    int tm, tn, half;
+    item_tile(t, tm, tn, half);
+    const int64_t m0 = (int64_t)tm * BM + half * 128, n0 = (int64_t)tn * BN;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
 
@@ -337,7 +410,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
     // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
     //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
-    const int64_t m = m0 + wm * 128 + l32;
+    const int64_t m = m0 + wm * (32 * MB) + l32;
     // A row bias depends on n only: its 64 values for this lane are fetched once, all loads in flight
     // together, instead of one dependent load per use in the loop below.
     constexpr bool ROW_BIAS = EPI == EPI_BIAS_ROW || EPI == EPI_BIAS_ROW_GELU;
@@ -352,7 +425,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                                                  : n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4));
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MB; ++i) {
       const int64_t mi = m + i * 32;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -390,7 +463,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the trailing refetches must land before the LDS is released
-  if (g.probe && blockIdx.x == 0 && tid == 0) {
+  if (MB == 4 && g.probe && blockIdx.x == 0 && tid == 0) {
     g.probe[0] = (unsigned long long)(clock64() - probe_c0);
     g.probe[1] = (unsigned long long)(wall_clock64() - probe_w0);
   }
@@ -407,7 +480,8 @@ extern "C" {
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, OUT, EPI>(g, ring);                                                              \
+    fast::body<IN, OUT, EPI, false, false, 4, true>(g, ring);                                       \
+    fast::body<IN, OUT, EPI, false, false, 2, true>(g, ring);                                       \
   }
 #define GEMM_TILE_ALL_EPI(prefix, IN, OUT)             \
   GEMM_TILE(prefix##_epi0, IN, OUT, EPI_NONE)           \
@@ -446,7 +520,8 @@ GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<DT_F16, DT_F16, EPI, true>(g, ring);                                                 \
+    fast::body<DT_F16, DT_F16, EPI, true, false, 4, true>(g, ring);                                 \
+    fast::body<DT_F16, DT_F16, EPI, true, false, 2, true>(g, ring);                                 \
   }
 GEMM_TILED(gemm_tiled_f16_epi0, EPI_NONE)
 GEMM_TILED(gemm_tiled_f16_epi3, EPI_LEAKY_RELU)

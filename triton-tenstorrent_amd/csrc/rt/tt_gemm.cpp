@@ -11,6 +11,16 @@ using namespace ttamd;
 
 namespace {
 
+// Workgroups of the persistent macro-tile kernels: one per CU, or one per tile when there are fewer tiles.
+// The plain kernels (`splits`) finish a tail of at most grid/2 macro tiles as half tiles on twice the
+// workgroups, so a problem of at most CUs/2 tiles is launched with two workgroups per tile.
+uint32_t persistent_grid(int64_t tiles, bool splits) {
+  const int64_t cus = props()->multiprocessor_count;
+  if (tiles >= cus) return (uint32_t)cus;
+  if (splits && 2 * tiles <= cus && !env_int("TTAMD_GEMM_NO_SPLIT", 0)) return (uint32_t)(2 * tiles);
+  return (uint32_t)tiles;
+}
+
 int check_desc(const char *who, const char *what, const tt_desc2d *d, int64_t rows, int64_t cols) {
   if (!d) return fail(RT_ERR_INVALID, "%s: null %s descriptor", who, what);
   if (!d->base) return fail(RT_ERR_INVALID, "%s: %s descriptor has a null base", who, what);
@@ -111,7 +121,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
              epi);
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    const uint32_t wgs = persistent_grid(tiles, fast_shape);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
     // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
     static unsigned long long *probe_buf = nullptr;
@@ -234,7 +244,7 @@ int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t 
       aligned16(c_ptr) && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const bool whole = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    const uint32_t wgs = persistent_grid(tiles, whole);
     char name[48];
     snprintf(name, sizeof(name), "gemm_tiled%s_f16_epi%d", whole ? "" : "ragged", leaky_relu ? 3 : 0);
     return launch("gemm", name, dim3(wgs), dim3(256), 0, stream, args, 1);
