@@ -497,16 +497,30 @@ def test_launch_hooks_and_no_leak_through_the_jit(tmp_path, monkeypatch):
     def after(launch_metadata):
         seen.append("after")
 
+    def load_start(module, function, name, metadata_group, hash):
+        seen.append(("load start", name, repr(function)))
+
+    def load_end(module, function, name, metadata_group, hash):
+        seen.append(("load end", name))
+
     try:
         triton.knobs.runtime.launch_enter_hook.add(first)
         triton.knobs.runtime.launch_enter_hook.add(second)
         triton.knobs.runtime.launch_exit_hook.add(after)
+        triton.knobs.runtime.kernel_load_start_hook.add(load_start)
+        triton.knobs.runtime.kernel_load_end_hook.add(load_end)
         try:
             does_nothing[(1, 3, 2)](6)
         finally:
             triton.knobs.runtime.launch_enter_hook.remove(first)
             triton.knobs.runtime.launch_enter_hook.remove(second)
             triton.knobs.runtime.launch_exit_hook.remove(after)
+            triton.knobs.runtime.kernel_load_start_hook.remove(load_start)
+            triton.knobs.runtime.kernel_load_end_hook.remove(load_end)
+        # the load hooks bracket load_binary on the first launch (test_launch.py::test_load_hook), then the launch hooks
+        assert seen[0][:2] == ("load start", "does_nothing") and seen[1] == ("load end", "does_nothing")
+        assert "BoundKernel empty_kernel" in repr(seen[0][2]) or seen[0][2] == "None"
+        del seen[:2]
         assert seen == ["first", "second", "after"]
         does_nothing[(1, 3, 2)](6)
         assert seen == ["first", "second", "after"]                    # removed hooks stay removed
