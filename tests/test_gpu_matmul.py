@@ -373,6 +373,21 @@ def test_fast_path_half_tile_tail(M, N, K_):
     _check(cbuf[:, :N].cpu(), ah.cpu(), bh.cpu())
 
 
+@pytest.mark.parametrize("M,N,K_", [(4300, 4096, 160), (4225, 4104, 96), (2000, 2056, 224), (4481, 4096, 64)])
+def test_ragged_fast_path_half_tile_tail(M, N, K_):
+    """The clamping instantiation with a short last round: 272 and 289 macro tiles, 72 (tail only), and 288 with a
+    last row of tiles that holds one row of C, so every lower half there lies past the matrix and stores nothing."""
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-4, 5, (M, K_), generator=g).to(torch.bfloat16).cuda()
+    b = torch.randint(-4, 5, (K_, N), generator=g).to(torch.bfloat16).cuda()
+    cbuf = torch.full((M + 1, N + 8), 7.5, dtype=torch.bfloat16, device="cuda")
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, cbuf[:M, :N]))
+    K.matmul_kernel_tma[(-(-M // 128) * -(-N // 128), )](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert rt.last_kernel_name() == "gemm_ragged_bf16_epi0"
+    assert torch.equal(cbuf[:M, :N], (a.float() @ b.float()).to(torch.bfloat16))
+    assert torch.all(cbuf[M:] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
+
+
 def test_full_size_8192_properties():
     """BASELINE's 8192^3: checked through size-independent properties -- B = I gives C = A
     bit for bit, linearity in A, and sampled rows against fp64 on the host."""

@@ -192,3 +192,15 @@ def test_tiled_fast_kernel_half_tile_tail(M, N, K_):
         want = torch.where(want >= 0, want, 0.01 * want) if act else want
         assert torch.equal(K.untilize(ct, M, N, 32, 32), want.to(torch.float16))
 
+
+@pytest.mark.parametrize("M,N,K_", [(4300, 4090, 100), (4481, 4000, 40)])
+def test_tiled_clamping_kernel_half_tile_tail(M, N, K_):
+    """The same for the clamping instantiation: 272 and 288 macro tiles, the second with a last row of tiles
+    whose lower halves lie wholly past the matrix."""
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-3, 4, (M, K_), generator=g).to(torch.float16)
+    b = torch.randint(-3, 4, (K_, N), generator=g).to(torch.float16)
+    ct = K.matmul_tiled(K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, K_)
+    assert rt.last_kernel_name() == "gemm_tiledragged_f16_epi0"
+    assert torch.equal(K.untilize(ct, M, N, 32, 32), (a.cuda().float() @ b.cuda().float()).to(torch.float16))
+

@@ -108,10 +108,11 @@ struct Ring {
 // copies per step, eight MFMAs per sub-step), used for the tail of the persistent loop: when the macro
 // tiles left over after the last whole round of the grid would keep at most half of the workgroups busy,
 // the kernel runs body<MB=4> over the whole rounds and then body<MB=2> over the halves of the tail tiles,
-// two workgroups per tile, instead of leaving half of the chip idle for a whole tile's time.
+// two workgroups per tile, instead of leaving half of the chip idle for a whole tile's time.  (RAGGED: a
+// half tile that lies wholly past the last row computes the other half's rows again and stores nothing.)
 template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
-  static_assert(MB == 4 || (MB == 2 && SPLIT_TAIL && !RAGGED), "half tiles exist for the tail of the plain kernels only");
+  static_assert(MB == 4 || (MB == 2 && SPLIT_TAIL), "half tiles exist for the tail pass only");
   // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
   // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
   // real M and N (the padding of C is never written, as under the reference's store mask).
@@ -255,14 +256,17 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
     int tm, tn, half;
     item_tile(min(t, total - 1), tm, tn, half);
-    const int64_t row0 = (int64_t)tm * BM + half * 128;
+    int64_t row0 = (int64_t)tm * BM + half * 128;
+    // RAGGED: a lower half that starts past the last row has nothing to fetch or store; it is pointed at the
+    // upper half's rows (which exist) and its stores all fall to the clipping
+    if (RAGGED && MB == 2 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
     if constexpr (RAGGED) {
-      const int last_row = Mf - 1 - tm * BM;                  // >= 0
+      const int last_row = Mf - 1 - (int)row0;                // >= 0
       const int last_chunk = (Nf - tn * BN) / 8 - 1;          // >= 0: the fetchable N is a multiple of 8
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < MB; ++i) {
         const int r = min(i * 64 + a_row, last_row);
         vo.a[i] = TILED ? (uint32_t)((((int64_t)(r >> 5) * ntk << 10) + (r & 31) * 32 + a_chunk * 8) * 2)
                         : (uint32_t)(((int64_t)r * g.lda + a_chunk * 8) * 2);
@@ -280,12 +284,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if constexpr (RAGGED) {
       const bool zero = k >= nk_real;                         // a padding step: both operands are zeros
       const Voffs &vo = over ? vo_nxt : vo_cur;
-      if (i < 4) {
+      if (i < MB) {
         const uint8_t *ap = zero ? zero_page : (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
         dma_one(ap, zero ? z_voff : vo.a[i], stage + i * 4096);
       } else {
-        const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - 4) * b_slab;
-        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - 4) * 4096);
+        const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - MB) * b_slab;
+        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - MB) * 4096);
       }
     } else if (i < MB) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
@@ -501,7 +505,8 @@ GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, OUT, EPI, false, true>(g, ring);                                                 \
+    fast::body<IN, OUT, EPI, false, true, 4, true>(g, ring);                                        \
+    fast::body<IN, OUT, EPI, false, true, 2, true>(g, ring);                                        \
   }
 #define GEMM_TILE_RAGGED_ALL_EPI(prefix, IN, OUT)             \
   GEMM_TILE_RAGGED(prefix##_epi0, IN, OUT, EPI_NONE)           \
@@ -534,7 +539,8 @@ GEMM_TILED(gemm_tiled_f16_epi3, EPI_LEAKY_RELU)
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<DT_F16, DT_F16, EPI, true, true>(g, ring);                                           \
+    fast::body<DT_F16, DT_F16, EPI, true, true, 4, true>(g, ring);                                  \
+    fast::body<DT_F16, DT_F16, EPI, true, true, 2, true>(g, ring);                                  \
   }
 GEMM_TILED_RAGGED(gemm_tiledragged_f16_epi0, EPI_NONE)
 GEMM_TILED_RAGGED(gemm_tiledragged_f16_epi3, EPI_LEAKY_RELU)

@@ -121,7 +121,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
              epi);
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = persistent_grid(tiles, fast_shape);
+    const uint32_t wgs = persistent_grid(tiles, true);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
     // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
     static unsigned long long *probe_buf = nullptr;
@@ -244,7 +244,7 @@ int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t 
       aligned16(c_ptr) && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const bool whole = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = persistent_grid(tiles, whole);
+    const uint32_t wgs = persistent_grid(tiles, true);
     char name[48];
     snprintf(name, sizeof(name), "gemm_tiled%s_f16_epi%d", whole ? "" : "ragged", leaky_relu ? 3 : 0);
     return launch("gemm", name, dim3(wgs), dim3(256), 0, stream, args, 1);
