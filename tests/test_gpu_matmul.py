@@ -448,6 +448,18 @@ def test_fp8_fast_path_small_integers_bit_exact_and_permutations():
     assert torch.equal(K.matmul_fp8_scaled(x8, p8, 0.5, 4.0).cpu().float(), (x @ p) * 2)
 
 
+@pytest.mark.parametrize("M,N,K_", [(4352, 4096, 256), (4352, 4352, 256), (2048, 2048, 512), (4300, 4096, 192), (4481, 4112, 128)])
+def test_fp8_fast_path_half_tile_tail(M, N, K_):
+    """fp8 with a short last round of macro tiles (272, 289, 64 tiles on 256 CUs; the last two shapes take the
+    clamping instantiation, the very last with lower halves that lie wholly past the matrix).  Small integers: exact."""
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randint(-4, 5, (M, K_), generator=g).float()
+    b = torch.randint(-4, 5, (K_, N), generator=g).float()
+    c = K.matmul_fp8_scaled(a.to(torch.float8_e4m3fn).cuda(), b.to(torch.float8_e4m3fn).cuda(), 0.5, 4.0)
+    assert rt.last_kernel_name() == ("gemm_tile_fp8_bf16" if M % 256 == 0 and N % 256 == 0 and K_ % 256 == 0 else "gemm_ragged_fp8_bf16")
+    assert torch.equal(c, ((a.cuda() @ b.cuda()) * 2).to(torch.bfloat16))
+
+
 def test_fp8_full_size_8192_properties():
     n = 8192
     g = torch.Generator(device="cuda").manual_seed(0)

@@ -91,6 +91,52 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int &tm
   tn = (id % in_group) / gsz;
 }
 
+// Work items of one pass of a kernel that finishes a short last round as half tiles: the macro-tile pass
+// (MB == 4) takes the whole rounds of the grid, or every tile when the tail is not worth splitting; the
+// half-tile pass (MB == 2) takes the two 128-row halves of each tail tile.
+struct PassItems {
+  int total;       // items of this pass
+  int first_tile;  // MB == 2: id of the first tail tile
+  int tail_tiles;
+};
+template <int MB, bool SPLIT_TAIL>
+__device__ __forceinline__ PassItems pass_items(int total_tiles) {
+  PassItems p = {total_tiles, 0, 0};
+  if constexpr (SPLIT_TAIL) {
+    const int whole = total_tiles / (int)gridDim.x * (int)gridDim.x;
+    p.tail_tiles = total_tiles - whole;
+    const bool split = p.tail_tiles > 0 && 2 * p.tail_tiles <= (int)gridDim.x;
+    if (MB == 4) {
+      p.total = split ? whole : total_tiles;
+    } else {
+      p.total = split ? 2 * p.tail_tiles : 0;
+      p.first_tile = whole;
+    }
+  }
+  return p;
+}
+// item -> macro tile and which half of it.  Workgroup ids go round-robin over the 8 XCDs and tile_of gives
+// tile t to XCD t % 8's run of ids, so halves are dealt in groups of 16 items over 8 tiles: both halves of
+// a tile then stay on the XCD that tile's neighbours ran on.
+template <int MB>
+__device__ __forceinline__ void item_tile(const PassItems &p, int item, int tiles_m, int tiles_n, int &tm, int &tn,
+                                          int &half) {
+  if constexpr (MB == 4) {
+    half = 0;
+    tile_of(item, tiles_m, tiles_n, tm, tn);
+  } else {
+    int j;
+    if (p.tail_tiles % 8 == 0) {
+      j = (item >> 4) * 8 + (item & 7);
+      half = (item >> 3) & 1;
+    } else {
+      j = item >> 1;
+      half = item & 1;
+    }
+    tile_of(p.first_tile + j, tiles_m, tiles_n, tm, tn);
+  }
+}
+
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
 
 struct Ring {
@@ -125,38 +171,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
   const int total_tiles = tiles_m * tiles_n;
-  // Work items of this pass: macro tiles (MB == 4) or halves of the tail's macro tiles (MB == 2).
-  int total = total_tiles, first_tile = 0, tail_tiles = 0;
-  if constexpr (SPLIT_TAIL) {
-    const int whole = total_tiles / (int)gridDim.x * (int)gridDim.x;
-    tail_tiles = total_tiles - whole;
-    const bool split = tail_tiles > 0 && 2 * tail_tiles <= (int)gridDim.x;
-    if (MB == 4) {
-      total = split ? whole : total_tiles;
-    } else {
-      total = split ? 2 * tail_tiles : 0;
-      first_tile = whole;
-    }
-  }
-  // item -> macro tile and which half of it.  Workgroup ids go round-robin over the 8 XCDs and tile_of gives
-  // tile t to XCD t % 8's run of ids, so halves are dealt in groups of 16 items over 8 tiles: both halves of
-  // a tile then stay on the XCD that tile's neighbours ran on.
-  auto item_tile = [&](int item, int &tm, int &tn, int &half) {
-    if constexpr (MB == 4) {
-      half = 0;
-      tile_of(item, tiles_m, tiles_n, tm, tn);
-    } else {
-      int j;
-      if (tail_tiles % 8 == 0) {
-        j = (item >> 4) * 8 + (item & 7);
-        half = (item >> 3) & 1;
-      } else {
-        j = item >> 1;
-        half = item & 1;
-      }
-      tile_of(first_tile + j, tiles_m, tiles_n, tm, tn);
-    }
-  };
+  const PassItems items = pass_items<MB, SPLIT_TAIL>(total_tiles);
+  const int total = items.total;
   const int nk_real = Kf / BK;                                    // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
@@ -255,7 +271,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const uint32_t z_voff = (uint32_t)tid * 16;
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
     int tm, tn, half;
-    item_tile(min(t, total - 1), tm, tn, half);
+    item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, half);
     int64_t row0 = (int64_t)tm * BM + half * 128;
     // RAGGED: a lower half that starts past the last row has nothing to fetch or store; it is pointed at the
     // upper half's rows (which exist) and its stores all fall to the clipping
@@ -393,7 +409,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
   for (; t < total; t += gridDim.x) {
     int tm, tn, half;
-    item_tile(t, tm, tn, half);
+    item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, half);
     const int64_t m0 = (int64_t)tm * BM + half * 128, n0 = (int64_t)tn * BN;
 #pragma unroll
     for (int i = 0; i < MB; ++i)

@@ -37,13 +37,16 @@ typedef __attribute__((address_space(3))) void lds_void;
 // RAGGED (M any, N a multiple of 16, K a multiple of 64): as in the 16-bit kernel, fetches past the edges are
 // clamped into the matrix, K is padded to whole turns of the ring with steps copied from a page of zeros, and
 // the stores are clipped.
-template <int OUT_DT, bool RAGGED = false>
+// MB = 2: the half-tile pass over the tail of the persistent loop, as in the 16-bit kernel: a workgroup computes a
+// 128x256 half of a macro tile, each wavefront 64x128 (2x4 accumulators), two A slabs and six copies per step.
+template <int OUT_DT, bool RAGGED = false, int MB = 4>
 __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
-  const int total = tiles_m * tiles_n;
+  const fast::PassItems items = fast::pass_items<MB, true>(tiles_m * tiles_n);
+  const int total = items.total;
   const int nk_real = g.K / BK;                                   // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
@@ -62,7 +65,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
   // ---- LDS -> fragments ----
   const int l32 = lane & 31, hi = lane >> 5;
-  const int a_base = (wm * 128 + l32) * 64;
+  const int a_base = (wm * (32 * MB) + l32) * 64;
   const int a_x = (l32 >> 2) & 3;
   int a_pos[2];
 #pragma unroll
@@ -77,13 +80,13 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   const uint8_t *B = (const uint8_t *)g.b;
 
   struct Frags {
-    union { i32x4 q[2]; i32x8 v; } a[4];
+    union { i32x4 q[2]; i32x8 v; } a[MB];
     union { i32x2 d[4]; i32x8 v; } b[4];
   };
   Frags f0, f1;
-  f32x16 acc[4][4];
+  f32x16 acc[MB][4];
 
-  // the 24 LDS reads of one step in the order the MFMAs want them:
+  // the 24 LDS reads of one step in the order the MFMAs want them (MB == 2: the first 20):
   // b0 (4 reads) a0 (2) b1 (4) b2 (4) b3 (4) a1 (2) a2 (2) a3 (2)
   auto rd = [&](Frags &f, const uint8_t *stage, int r) {
     auto rb = [&](int j, int q) {
@@ -112,15 +115,19 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   Voffs vo_cur, vo_nxt;
   const uint32_t z_voff = (uint32_t)tid * 16;
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
-    int tm, tn;
-    fast::tile_of(min(t, total - 1), tiles_m, tiles_n, tm, tn);
-    ap = A + (int64_t)tm * BM * g.lda;
+    int tm, tn, half;
+    fast::item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, half);
+    int64_t row0 = (int64_t)tm * BM + half * 128;
+    // RAGGED: a lower half that starts past the last row is pointed at the upper half's rows; its stores all
+    // fall to the clipping
+    if (RAGGED && MB == 2 && row0 >= g.M) row0 = (int64_t)tm * BM;
+    ap = A + row0 * g.lda;
     bp = B + (int64_t)tn * BN;
     if constexpr (RAGGED) {
-      const int last_row = g.M - 1 - tm * BM;
+      const int last_row = g.M - 1 - (int)row0;
       const int last_chunk = (g.N - tn * BN) / 16 - 1;        // N is a multiple of 16
 #pragma unroll
-      for (int i = 0; i < 4; ++i) vo.a[i] = (uint32_t)((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 16);
+      for (int i = 0; i < MB; ++i) vo.a[i] = (uint32_t)((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 16);
       vo.b = (uint32_t)((int64_t)b_k * g.ldb + min(b_chunk, last_chunk) * 16);
     }
   };
@@ -130,19 +137,19 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     if constexpr (RAGGED) {
       const bool zero = k >= nk_real;
       const Voffs &vo = over ? vo_nxt : vo_cur;
-      if (i < 4) {
+      if (i < MB) {
         const uint8_t *ap = zero ? fast::zero_page : (over ? a_nxt : a_cur) + (int64_t)k * BK;
         dma_one(ap, zero ? z_voff : vo.a[i], stage + i * 4096);
       } else {
-        const uint8_t *bp = zero ? fast::zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - 4) * b_slab;
-        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - 4) * 4096);
+        const uint8_t *bp = zero ? fast::zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - MB) * b_slab;
+        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - MB) * 4096);
       }
-    } else if (i < 4) {
+    } else if (i < MB) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * BK;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
-      dma_one(bp + (i - 4) * b_slab, b_voff, stage + A_BYTES + (i - 4) * 4096);
+      dma_one(bp + (i - MB) * b_slab, b_voff, stage + A_BYTES + (i - MB) * 4096);
     }
   };
 
@@ -156,17 +163,32 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     // every wave's reads of stage I have returned (they fed `c`), and this wave's share of the
     // copy into stage I+1 has landed (the 16 younger copies may still be in flight); after the
     // barrier that holds for all waves: I+1 may be read, I may be overwritten
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    FENCE();
-#pragma unroll
-    for (int n = 1; n < 16; ++n) {
-      if (n <= 12) {
-        rd(p, nxt, 2 * (n - 1));
-        rd(p, nxt, 2 * (n - 1) + 1);
-      }
-      if (n & 1) dma_single(k + R, cur, n >> 1); // one copy per two MFMAs: thin enough not to stall issue
-      mm(c, n);
+    if constexpr (MB == 4) {
+      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       FENCE();
+#pragma unroll
+      for (int n = 1; n < 16; ++n) {
+        if (n <= 12) {
+          rd(p, nxt, 2 * (n - 1));
+          rd(p, nxt, 2 * (n - 1) + 1);
+        }
+        if (n & 1) dma_single(k + R, cur, n >> 1); // one copy per two MFMAs: thin enough not to stall issue
+        mm(c, n);
+        FENCE();
+      }
+    } else {
+      // half tiles: 8 MFMAs, 20 fragment reads (three per MFMA) and 6 copies per step; the two youngest
+      // steps' copies (12) may still be in flight at the barrier
+      asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      FENCE();
+#pragma unroll
+      for (int n = 1; n < 8; ++n) {
+#pragma unroll
+        for (int r = 3 * (n - 1); r < 3 * n && r < 20; ++r) rd(p, nxt, r);
+        if (n <= 6) dma_single(k + R, cur, n - 1);
+        mm(c, n);
+        FENCE();
+      }
     }
   };
 
@@ -178,17 +200,21 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 #pragma unroll
   for (int s = 0; s < R; ++s)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dma_single(s, ring.s[s], i);
-  asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
+    for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i);
+  // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
+  if constexpr (MB == 4)
+    asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-  for (int r = 0; r < 24; ++r) rd(f0, ring.s[0], r);
+  for (int r = 0; r < 16 + 2 * MB; ++r) rd(f0, ring.s[0], r);
 
   for (; t < total; t += gridDim.x) {
-    int tm, tn;
-    fast::tile_of(t, tiles_m, tiles_n, tm, tn);
-    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    int tm, tn, half;
+    fast::item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, half);
+    const int64_t m0 = (int64_t)tm * BM + half * 128, n0 = (int64_t)tn * BN;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
     for (int k = 0; k < nk; k += R) {
@@ -206,9 +232,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     }
     // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
     //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
-    const int64_t m = m0 + wm * 128 + l32;
+    const int64_t m = m0 + wm * (32 * MB) + l32;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < MB; ++i) {
       const int64_t mi = m + i * 32;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -252,7 +278,8 @@ extern "C" {
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                    \
-    fast8::body<OUT>(g, ring);                                                                       \
+    fast8::body<OUT, false, 4>(g, ring);                                                             \
+    fast8::body<OUT, false, 2>(g, ring);                                                             \
   }
 
 GEMM_TILE_FP8(gemm_tile_fp8_bf16, DT_BF16)
@@ -266,7 +293,8 @@ GEMM_TILE_FP8(gemm_tile_fp8_fp8, DT_FP8)
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                    \
-    fast8::body<OUT, true>(g, ring);                                                                 \
+    fast8::body<OUT, true, 4>(g, ring);                                                              \
+    fast8::body<OUT, true, 2>(g, ring);                                                              \
   }
 GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16, DT_BF16)
 GEMM_RAGGED_FP8(gemm_ragged_fp8_f16, DT_F16)

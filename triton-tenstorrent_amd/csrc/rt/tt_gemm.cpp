@@ -148,7 +148,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   const bool fp8_ragged = !fp8_shape && N % 16 == 0 && K % 64 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24);
   if (full_grid && fp8_io && (fp8_shape || fp8_ragged) && fp8_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = (uint32_t)std::min<int64_t>(tiles, props()->multiprocessor_count);
+    const uint32_t wgs = persistent_grid(tiles, true);
     void *fargs[] = {&g};
     char fp8_name[48];
     snprintf(fp8_name, sizeof(fp8_name), "gemm_%s_fp8_%s", fp8_shape ? "tile" : "ragged",
