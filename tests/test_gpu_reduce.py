@@ -18,7 +18,9 @@ TORCH_OF = {orc.I8: torch.int8, orc.I16: torch.int16, orc.I32: torch.int32, orc.
             orc.U16: torch.uint16, orc.U32: torch.uint32, orc.U64: torch.uint64}
 NP_OF = {orc.I8: np.int8, orc.I16: np.int16, orc.I32: np.int32, orc.I64: np.int64, orc.U8: np.uint8, orc.U16: np.uint16,
          orc.U32: np.uint32, orc.U64: np.uint64}
-SHAPES = [1, 32, 64, 128, 512, 1000, 4096, 1 << 20]    # 32..512: test_core.py::test_reduce1d; 2^20: Triton's largest tensor
+# 32..512: test_core.py::test_reduce1d; 2^20: Triton's largest tensor; 131072 and up: from 128 KiB of input on the
+# block is shared between workgroups (131072 int8 is the first such size, 131075 and 1048575 leave a ragged end)
+SHAPES = [1, 32, 64, 128, 512, 1000, 4096, 131072, 131075, 1048575, 1 << 20]
 
 
 def _acc_for(op, dt):
@@ -104,3 +106,32 @@ def test_error_paths_return_codes():
     assert "reduce1d" in rt.last_error()
     assert call(0, 64, rt.TT_F32, rt.TT_F32, rt.TT_F32, g=(C.c_uint32 * 3)(7, 1, 1)) == rt.RT_OK   # every program stores the same
     torch.cuda.synchronize()
+
+
+def test_large_blocks_across_workgroups_streams_and_repeats():
+    """A block of 128 KiB and more is folded by several workgroups through a per-stream buffer of partial results:
+    repeated launches on one stream, launches on two streams at once, an operand off the 16-byte grid (one
+    workgroup) and the one-workgroup switch all give the same exact answers."""
+    rng = np.random.default_rng(3)
+    x = rng.integers(-2**31, 2**31 - 1, (1 << 20) + 4, dtype=np.int64).astype(np.int32)
+    xg = torch.from_numpy(x).cuda()
+    want = {op: orc.reduce1d(x[:1 << 20], op, orc.I32) for op in ("sum", "argmax", "xor_sum", "min")}
+    for _ in range(5):
+        for op, w in want.items():
+            assert K.reduce1d(op, xg[:1 << 20]).cpu().numpy()[0] == w, op
+    off = xg[1:(1 << 20) + 1]                                          # 4 bytes off a 16-byte boundary
+    for op in want:
+        assert K.reduce1d(op, off).cpu().numpy()[0] == orc.reduce1d(x[1:(1 << 20) + 1], op, orc.I32), op
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    y = torch.from_numpy(x[::-1].copy()).cuda()
+    torch.cuda.synchronize()
+    outs = []
+    for i in range(20):
+        with torch.cuda.stream(s1):
+            outs.append((K.reduce1d("sum", xg[:1 << 20]), want["sum"]))
+        with torch.cuda.stream(s2):
+            outs.append((K.reduce1d("argmax", y[4:]), orc.reduce1d(np.ascontiguousarray(x[::-1][4:]), "argmax", orc.I32)))
+    torch.cuda.synchronize()
+    for got, w in outs:
+        assert got.cpu().numpy()[0] == w
+

@@ -3,7 +3,7 @@
 // that the reference's CI runs on its cpu/ path (.github/workflows/integration-tests-cpu.yml:105,
 // test_core.py::test_reduce1d; lowering of the cross-lane steps: cpu/lib/TritonCPUToLLVM/TargetInfo.cpp:95-225).
 //
-// One workgroup of 1024 lanes: each lane folds a strided share of the elements, 64 lanes fold with
+// One workgroup of 1024 lanes (up to 256 of them for blocks of 128 KiB and more, see reduce_body): each lane folds a strided share of the elements, 64 lanes fold with
 // __shfl_xor, the sixteen wavefronts fold through LDS, lane 0 stores.  Integers are carried in 64 bits
 // (sum and xor wrap, so truncating the 64-bit result to the accumulator width of the IR gives that
 // width's wraparound result; min/max compare exactly); f16/bf16/f32 are carried in fp32, f64 in fp64.
@@ -124,20 +124,31 @@ template <typename C> __device__ __forceinline__ void store_value(void *z, int o
 // low out_bytes of the 64-bit result is that accumulator's wraparound result, truncated as the IR does.
 template <typename T, int op>
 __device__ __forceinline__ void reduce_body(const T *__restrict__ x, void *__restrict__ z, int n, int nan_mode,
-                                            int out_bytes, int out_kind) {
+                                            int out_bytes, int out_kind, void *scratch, unsigned *counter) {
   using C = typename Carry<T>::type;
   __shared__ Pair<C> part[kLanes / 64];
   const int tid = threadIdx.x;
+  const int G = (int)gridDim.x, b = (int)blockIdx.x;
   Pair<C> p{C(0), -1};
   // 16-byte loads when X is 16-byte aligned: kAhead of them per lane are issued before the first fold
   // waits on one; the ragged end (and an unaligned X) goes element by element.
+  // With more than one workgroup (large blocks on an aligned X) the vectors are dealt in contiguous runs, the
+  // ragged end goes to the last workgroup, every workgroup leaves its partial result in `scratch`, and the one
+  // that finishes last folds the partials in workgroup order and stores.
   constexpr int kPer = 16 / (int)sizeof(T);
-  int done = 0;
-  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15u) == 0;
+  int lo = 0, hi = n;
+  if (G > 1) {
+    const int nvec = n / kPer, per = (nvec + G - 1) / G;
+    lo = min(b * per, nvec) * kPer;
+    hi = b == G - 1 ? n : min((b + 1) * per, nvec) * kPer;
+  }
+  int done = lo;
+  if (vec) {
     const uint4 *xv = reinterpret_cast<const uint4 *>(x);
-    const int nvec = n / kPer;
-    int j = tid;
-    for (; j + (kAhead - 1) * kLanes < nvec; j += kAhead * kLanes) {
+    const int vend = hi / kPer;
+    int j = lo / kPer + tid;
+    for (; j + (kAhead - 1) * kLanes < vend; j += kAhead * kLanes) {
       union { uint4 q; T e[kPer]; } v[kAhead];
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) v[u].q = xv[j + u * kLanes];
@@ -147,21 +158,57 @@ __device__ __forceinline__ void reduce_body(const T *__restrict__ x, void *__res
         for (int e = 0; e < kPer; ++e)
           p = fold<op>(nan_mode != 0, p, Pair<C>{widen<T>(v[u].e[e]), (j + u * kLanes) * kPer + e});
     }
-    for (; j < nvec; j += kLanes) {
-      union { uint4 q; T e[kPer]; } v;
-      v.q = xv[j];
+    if (j < vend) {   // fewer than kAhead vectors left for this lane: again all loads first
+      union { uint4 q; T e[kPer]; } v[kAhead];
 #pragma unroll
-      for (int e = 0; e < kPer; ++e) p = fold<op>(nan_mode != 0, p, Pair<C>{widen<T>(v.e[e]), j * kPer + e});
+      for (int u = 0; u < kAhead - 1; ++u)
+        if (j + u * kLanes < vend) v[u].q = xv[j + u * kLanes];
+#pragma unroll
+      for (int u = 0; u < kAhead - 1; ++u)
+        if (j + u * kLanes < vend) {
+#pragma unroll
+          for (int e = 0; e < kPer; ++e)
+            p = fold<op>(nan_mode != 0, p, Pair<C>{widen<T>(v[u].e[e]), (j + u * kLanes) * kPer + e});
+        }
     }
-    done = nvec * kPer;
+    done = vend * kPer;
   }
-  for (int i = done + tid; i < n; i += kLanes) p = fold<op>(nan_mode != 0, p, Pair<C>{widen<T>(x[i]), i});
+  for (int i = done + tid; i < hi; i += kLanes) p = fold<op>(nan_mode != 0, p, Pair<C>{widen<T>(x[i]), i});
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) p = fold<op>(nan_mode != 0, p, shuffle_xor(p, m));
   if ((tid & 63) == 0) part[tid >> 6] = p;
   __syncthreads();
-  if (tid == 0) {
+  if (tid == 0)
     for (int w = 1; w < kLanes / 64; ++w) p = fold<op>(nan_mode != 0, p, part[w]);
+  if (G > 1) {
+    // the workgroup's result goes to its slot; the workgroup that takes the last ticket folds all the slots,
+    // one per lane, the same way
+    __shared__ int last;
+    volatile Pair<C> *slots = (volatile Pair<C> *)scratch;
+    if (tid == 0) {
+      slots[b].v = p.v;
+      slots[b].i = p.i;
+      __threadfence();                                   // the partial is visible before the ticket is taken
+      last = atomicAdd(counter, 1u) == (unsigned)(G - 1);
+    }
+    __syncthreads();
+    if (!last) return;
+    __threadfence();
+    p = Pair<C>{C(0), -1};
+    if (tid < G) {
+      p.v = slots[tid].v;
+      p.i = slots[tid].i;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) p = fold<op>(nan_mode != 0, p, shuffle_xor(p, m));
+    if ((tid & 63) == 0) part[tid >> 6] = p;
+    __syncthreads();
+    if (tid == 0) {
+      for (int w = 1; w < kLanes / 64; ++w) p = fold<op>(nan_mode != 0, p, part[w]);
+      *counter = 0;                                      // ready for the next launch on this stream
+    }
+  }
+  if (tid == 0) {
     if (op == ARGMIN || op == ARGMAX) {
       if (out_bytes == 8) *(int64_t *)z = p.i;
       else *(int32_t *)z = p.i;
@@ -175,14 +222,15 @@ __device__ __forceinline__ void reduce_body(const T *__restrict__ x, void *__res
 
 #define REDUCE_KERNEL(name, T)                                                                                        \
   extern "C" __global__ __launch_bounds__(kLanes) void name(const void *x, void *z, int n, int op, int nan_mode,     \
-                                                             int out_bytes, int out_kind) {                          \
+                                                             int out_bytes, int out_kind, void *scratch,        \
+                                                             unsigned *counter) {                                    \
     switch (op) {                                                                                                     \
-    case SUM: reduce_body<T, SUM>((const T *)x, z, n, nan_mode, out_bytes, out_kind); break;                          \
-    case MIN: reduce_body<T, MIN>((const T *)x, z, n, nan_mode, out_bytes, out_kind); break;                          \
-    case MAX: reduce_body<T, MAX>((const T *)x, z, n, nan_mode, out_bytes, out_kind); break;                          \
-    case ARGMIN: reduce_body<T, ARGMIN>((const T *)x, z, n, nan_mode, out_bytes, out_kind); break;                    \
-    case ARGMAX: reduce_body<T, ARGMAX>((const T *)x, z, n, nan_mode, out_bytes, out_kind); break;                    \
-    default: reduce_body<T, XOR>((const T *)x, z, n, nan_mode, out_bytes, out_kind); break;                           \
+    case SUM: reduce_body<T, SUM>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
+    case MIN: reduce_body<T, MIN>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
+    case MAX: reduce_body<T, MAX>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
+    case ARGMIN: reduce_body<T, ARGMIN>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
+    case ARGMAX: reduce_body<T, ARGMAX>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
+    default: reduce_body<T, XOR>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
     }                                                                                                                 \
   }
 

@@ -1,9 +1,44 @@
 // tt_reduce1d_kernel: launch validation and kernel selection for the single-block reductions.
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <utility>
+
+#include <hip/hip_runtime.h>
+
 #include "tt_internal.h"
 
 using namespace ttamd;
 
 namespace {
+// A large block is reduced by several workgroups that leave partial results in a small device buffer (256 slots
+// of 16 bytes and an arrival counter).  Launches on one stream run in order and share one buffer; every
+// (device, stream) pair gets its own, allocated on first use and kept until the process ends.
+constexpr int kMaxGroups = 256;
+constexpr size_t kSlotBytes = 16, kCounterAt = kMaxGroups * kSlotBytes;
+void *partials_for(void *stream) {
+  static std::mutex mu;
+  static std::map<std::pair<int, void *>, void *> bufs;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lk(mu);
+  auto it = bufs.find({dev, stream});
+  if (it != bufs.end()) return it->second;
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing((hipStream_t)stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;   // no allocation while the stream records a graph: the caller takes one workgroup
+  }
+  void *p = nullptr;
+  if (hipMalloc(&p, kCounterAt + 256) != hipSuccess) return nullptr;
+  if (hipMemset(p, 0, kCounterAt + 256) != hipSuccess) {
+    (void)hipFree(p);
+    return nullptr;
+  }
+  bufs[{dev, stream}] = p;
+  return p;
+}
+
 struct TypeInfo { const char *kernel; int bytes; bool is_float; };
 bool type_info(int dt, TypeInfo *t) {
   switch (dt) {
@@ -60,7 +95,19 @@ extern "C" int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BL
                   "is not offered)", acc_dtype, out_dtype);
   }
   int32_t n = BLOCK, op_ = op, nan_ = propagate_nan ? 1 : 0, ob = out.bytes;
-  void *args[] = {(void *)&x, (void *)&z, &n, &op_, &nan_, &ob, &out_kind};
-  // Every program of the logical grid computes and stores the same value; one workgroup does it once.
-  return launch("reduce", in.kernel, dim3(1), dim3(1024), 0, stream, args, 7);
+  // Every program of the logical grid computes and stores the same value; it is computed once: by one workgroup,
+  // or, from 128 KiB of 16-byte aligned input on, by one workgroup per 16 KiB (256 at most) whose last finisher
+  // folds their partial results.
+  const int64_t bytes = (int64_t)BLOCK * in.bytes;
+  uint32_t groups = 1;
+  void *scratch = nullptr, *counter = nullptr;
+  if (bytes >= (128 << 10) && aligned16(x) && !env_int("TTAMD_REDUCE_ONE_GROUP", 0)) {
+    scratch = partials_for(stream);
+    if (scratch) {
+      groups = (uint32_t)std::min<int64_t>(kMaxGroups, bytes >> 14);
+      counter = (char *)scratch + kCounterAt;
+    }
+  }
+  void *args[] = {(void *)&x, (void *)&z, &n, &op_, &nan_, &ob, &out_kind, &scratch, &counter};
+  return launch("reduce", in.kernel, dim3(groups), dim3(1024), 0, stream, args, 9);
 }
