@@ -1,7 +1,6 @@
 """Launches are plain hipModuleLaunchKernel calls on the caller's stream with no allocation, memset or
 synchronisation inside, so a caller can record them into a HIP graph.  Each graph is replayed several times
 with eager work and synchronisations in between, and every replay is checked against the eager result."""
-import numpy as np
 import pytest
 import torch
 

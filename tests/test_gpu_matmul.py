@@ -9,7 +9,7 @@ from oracle import oracle as orc
 from triton_tenstorrent_amd import kernels as K
 from triton_tenstorrent_amd import runtime as rt
 from triton_tenstorrent_amd.tensor_descriptor import TensorDescriptor
-from util import ORC_DT, bits, close_bf16, decode, from_bits
+from util import ORC_DT, bits, close_bf16, decode
 
 pytestmark = pytest.mark.gpu
 RTOL, ATOL, PCC = 1e-2, 1e-4, 0.9999

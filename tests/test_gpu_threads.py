@@ -2,7 +2,6 @@
 tables are locked, errors and "last kernel" are per thread, so concurrent launches on distinct streams are safe."""
 import threading
 
-import numpy as np
 import pytest
 import torch
 
