@@ -143,7 +143,6 @@ def test_fast_attention_random_lengths_and_head_dims():
 
 
 def test_fast_attention_closed_forms_and_any_path_agreement():
-    import os
     from triton_tenstorrent_amd import runtime as rt
     q, k, v = _qkv(1, 2, 512, 128, seed=7)
     o, M = K.attention(q.cuda(), k.cuda(), v.cuda(), True, 0.3, return_lse=True)
