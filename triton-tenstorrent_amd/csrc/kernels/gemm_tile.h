@@ -447,40 +447,66 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                                          (RAGGED ? min(n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4, (int64_t)g.N - 4)
                                                  : n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4));
     }
+    // the four columns n .. n+3 of row mi that this lane holds for (i, j, r4), after scale, epilogue and rounding
+    auto packed = [&](int i, int j, int r4, int64_t mi, int64_t n) {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float x = acc[i][j][r4 * 4 + e] * g.scale;
+        if constexpr (EPI == EPI_BIAS_ROW_GELU)
+          v[e] = gelu_erf(x + brow[j][r4][e]);
+        else if constexpr (EPI == EPI_BIAS_ROW)
+          v[e] = x + brow[j][r4][e];
+        else
+          v[e] = apply_epilogue_ct<OUT_DT, EPI>(g, x, mi, n + e);
+      }
+      if constexpr (OUT_DT == DT_BF16)
+        return (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+      else
+        return (u32x2){(uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16),
+                       (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
+    };
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
       const int64_t mi = m + i * 32;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        if constexpr (!(RAGGED && TILED)) {
+          // The lane pair (l, l+32) holds columns 0-3 | 4-7 for r4 = 2q and 8-11 | 12-15 for r4 = 2q+1 of one row.
+          // Swapping the upper lanes' first group with the lower lanes' second (v_permlane32_swap: upper half of
+          // its first operand <-> lower half of its second) gives the lower lane columns 0-7 and the upper lane
+          // 8-15, so each lane stores 16 contiguous bytes: half the store instructions, each covering 32 bytes of
+          // a row (8 columns never straddle a 32x32 tile of a tile-major C, nor the edge of a clipped one, whose N
+          // is a multiple of 8).  Every lane takes part in the swap; clipped lanes only skip the store, and read a
+          // full bias, if there is one, at a clamped position.
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
-          if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // row-major: N is a multiple of 8, the four columns stand or fall together
-          float v[4];
+          for (int q = 0; q < 2; ++q) {
+            const int64_t nb = n0 + wn * 128 + j * 32 + q * 16;
+            const int64_t mb = RAGGED ? min(mi, (int64_t)g.M - 1) : mi;
+            const int64_t nl = nb + hi * 4, nh = nb + 8 + hi * 4;
+            u32x2 p0 = packed(i, j, 2 * q, mb, RAGGED ? min(nl, (int64_t)g.N - 4) : nl);
+            u32x2 p1 = packed(i, j, 2 * q + 1, mb, RAGGED ? min(nh, (int64_t)g.N - 4) : nh);
+            asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p0.x), "+v"(p1.x));
+            asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p0.y), "+v"(p1.y));
+            const int64_t n = nb + hi * 8;
+            if (RAGGED && (mi >= g.M || n >= g.N)) continue;
+            const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
+            *(u32x4 *)((uint16_t *)g.c + coff) = (u32x4){p0.x, p0.y, p1.x, p1.y};
+          }
+        } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float x = acc[i][j][r4 * 4 + e] * g.scale;
-            if constexpr (EPI == EPI_BIAS_ROW_GELU)
-              v[e] = gelu_erf(x + brow[j][r4][e]);
-            else if constexpr (EPI == EPI_BIAS_ROW)
-              v[e] = x + brow[j][r4][e];
-            else
-              v[e] = apply_epilogue_ct<OUT_DT, EPI>(g, x, mi, n + e);
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
+            if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // row-major: N is a multiple of 8, the four columns stand or fall together
+            const u32x2 pk = packed(i, j, r4, mi, n);
+            const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
+            if (TILED && RAGGED && n + 3 >= g.N) {               // N is anything here: the last group goes by element
+              for (int e = 0; e < 4 && n + e < g.N; ++e)
+                ((uint16_t *)g.c)[coff + e] = (uint16_t)(e & 1 ? pk[e >> 1] >> 16 : pk[e >> 1] & 0xffffu);
+              continue;
+            }
+            *(u32x2 *)((uint16_t *)g.c + coff) = pk;
           }
-          u32x2 pk;
-          if constexpr (OUT_DT == DT_BF16) {
-            pk = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-          } else {
-            pk = (u32x2){(uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16),
-                         (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
-          }
-          const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
-          if (TILED && RAGGED && n + 3 >= g.N) {               // N is anything here: the last group goes by element
-            for (int e = 0; e < 4 && n + e < g.N; ++e)
-              ((uint16_t *)g.c)[coff + e] = (uint16_t)(e & 1 ? pk[e >> 1] >> 16 : pk[e >> 1] & 0xffffu);
-            continue;
-          }
-          *(u32x2 *)((uint16_t *)g.c + coff) = pk;
         }
       }
     }

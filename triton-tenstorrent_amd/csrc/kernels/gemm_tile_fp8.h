@@ -238,28 +238,42 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
       const int64_t mi = m + i * 32;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        if constexpr (OUT_DT == DT_FP8) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
-          if (RAGGED && (mi >= g.M || n >= g.N)) continue;
-          float v[4];
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
+            if (RAGGED && (mi >= g.M || n >= g.N)) continue;
+            float v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][r4 * 4 + e] * g.scale;
-          if constexpr (OUT_DT == DT_FP8) {
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][r4 * 4 + e] * g.scale;
             // FP8_OUTPUT (09-persistent-matmul.py:116,173): four e4m3 codes, one 4-byte store
             const uint32_t q = (uint32_t)f32_to_fp8(v[0]) | ((uint32_t)f32_to_fp8(v[1]) << 8) |
                                ((uint32_t)f32_to_fp8(v[2]) << 16) | ((uint32_t)f32_to_fp8(v[3]) << 24);
             *(uint32_t *)((uint8_t *)g.c + mi * g.ldc + n) = q;
-            continue;
           }
-          u32x2 pk;
-          if constexpr (OUT_DT == DT_BF16) {
-            pk = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-          } else {
-            pk = (u32x2){(uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16),
-                         (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
+        } else {
+          // 16-byte stores as in the 16-bit kernel: the lane pair (l, l+32) exchanges its middle column groups
+          // (v_permlane32_swap), so the lower lane holds columns 0-7 and the upper lane 8-15 of each 16
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            u32x2 p[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              float v[4];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = acc[i][j][(2 * q + h) * 4 + e] * g.scale;
+              if constexpr (OUT_DT == DT_BF16)
+                p[h] = (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+              else
+                p[h] = (u32x2){(uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16),
+                               (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
+            }
+            asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p[0].x), "+v"(p[1].x));
+            asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p[0].y), "+v"(p[1].y));
+            const int64_t n = n0 + wn * 128 + j * 32 + q * 16 + hi * 8;
+            if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // N is a multiple of 16
+            *(u32x4 *)((uint16_t *)g.c + mi * g.ldc + n) = (u32x4){p[0].x, p[0].y, p[1].x, p[1].y};
           }
-          *(u32x2 *)((uint16_t *)g.c + mi * g.ldc + n) = pk;
         }
       }
     }
