@@ -72,13 +72,13 @@ def _events_time(fn, steps: int, warmup: int, stream: int, tag: str | None = Non
 # plain copy-like kernel of known size).  Not measured live: the counters need the profiler around the process.
 # profiles/bench_all_kernels_rocprofv3.md holds the raw readings and the commands.
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_tile_bf16_epi0": int((2 * 808858 + 187073) * 1024),
-    "gemm_tile_bf16_epi2": int((2 * 386044 + 119597) * 1024),
-    "gemm_tile_fp8_bf16": int((2 * 403126 + 174109) * 1024),
-    "gemm_tiled_f16_epi0": int((2 * 919114 + 141068) * 1024),
-    "attn_tile_d128": int((2 * 196920 + 133120) * 1024),
-    "ew_add_i32": int((2 * 1048596 + 1048576) * 1024),
-    "ew_sin_f32": int((2 * 524420 + 1048607) * 1024),
+    "gemm_tile_bf16_epi0": int((2 * 799244 + 165485) * 1024),
+    "gemm_tile_bf16_epi2": int((2 * 386055 + 119776) * 1024),
+    "gemm_tile_fp8_bf16": int((2 * 403806 + 160068) * 1024),
+    "gemm_tiled_f16_epi0": int((2 * 860650 + 141087) * 1024),
+    "attn_tile_d128": int((2 * 197059 + 133120) * 1024),
+    "ew_add_i32": int((2 * 1048594 + 1048576) * 1024),
+    "ew_sin_f32": int((2 * 524420 + 1048595) * 1024),
 }
 
 
