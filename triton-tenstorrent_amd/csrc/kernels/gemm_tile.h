@@ -294,10 +294,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   };
   // copy number i (0..MB-1: A slabs, MB..MB+3: B slabs) of step kk into `stage`; kk may run past
   // nk into the next tile
-  auto dma_single = [&](int kk, uint8_t *stage, int i) {
-    const bool over = kk >= nk;
+  // `inner` (RAGGED only): the caller knows that step kk belongs to this tile and carries data, so the choices
+  // between this tile and the next and between data and the page of zeros are not made at run time
+  auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_) {
+    constexpr bool inner = decltype(inner_)::value;
+    const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
-    if constexpr (RAGGED) {
+    if constexpr (RAGGED && inner) {
+      if (i < MB)
+        dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
+      else
+        dma_one(b_cur + (int64_t)k * b_kstep + (i - MB) * b_slab, vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
+    } else if constexpr (RAGGED) {
       const bool zero = k >= nk_real;                         // a padding step: both operands are zeros
       const Voffs &vo = over ? vo_nxt : vo_cur;
       if (i < MB) {
@@ -326,7 +334,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // queue, and its MFMAs stall with it.  (One per four MFMAs, at 1, 5, 9, 13, keeps the pipe
   // 77 % busy at 1.68 GHz, this placement 80 % at 1.63 GHz: the part is power-limited, so
   // most of a gain in issue efficiency is taken back by the clock.)
-  auto step = [&](auto I_, int k) {
+  auto step = [&](auto I_, int k, auto inner_) {
     constexpr int I = decltype(I_)::value;
     uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R], *prv = ring.s[(I + R - 1) % R];
     if constexpr (MB == 4) {
@@ -338,7 +346,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           rd(f1, cur, 1, 2 * n);
           rd(f1, cur, 1, 2 * n + 1);
         }
-        if (n >= 7 && n <= 13 && (n & 1)) dma_single(k - 1 + R, prv, 4 + ((n - 7) >> 1));
+        if (n >= 7 && n <= 13 && (n & 1)) dma_single(k - 1 + R, prv, 4 + ((n - 7) >> 1), inner_);
         mm(f0, n);
         FENCE();
       }
@@ -355,7 +363,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           rd(f0, nxt, 0, 2 * n);
           rd(f0, nxt, 0, 2 * n + 1);
         }
-        if (n >= 7 && n <= 13 && (n & 1)) dma_single(k + R, cur, (n - 7) >> 1);
+        if (n >= 7 && n <= 13 && (n & 1)) dma_single(k + R, cur, (n - 7) >> 1, inner_);
         mm(f1, n);
         FENCE();
       }
@@ -369,7 +377,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           rd(f1, cur, 1, 2 * n);
           rd(f1, cur, 1, 2 * n + 1);
         }
-        if (n & 1) dma_single(k - 1 + R, prv, MB + (n >> 1));
+        if (n & 1) dma_single(k - 1 + R, prv, MB + (n >> 1), inner_);
         mm(f0, n);
         FENCE();
       }
@@ -381,7 +389,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           rd(f0, nxt, 0, 2 * n);
           rd(f0, nxt, 0, 2 * n + 1);
         }
-        if ((n & 3) == 1) dma_single(k + R, cur, n >> 2);
+        if ((n & 3) == 1) dma_single(k + R, cur, n >> 2, inner_);
         mm(f1, n);
         FENCE();
       }
@@ -397,7 +405,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #pragma unroll
   for (int s = 0; s < R; ++s)
 #pragma unroll
-    for (int i = 0; i < (s == R - 1 ? MB : MB + 4); ++i) dma_single(s, ring.s[s], i);
+    for (int i = 0; i < (s == R - 1 ? MB : MB + 4); ++i) dma_single(s, ring.s[s], i, std::false_type{});
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
   // everything issued but step 0's own MB + 4 copies may still be in flight: 2 * (MB + 4) + MB
   if constexpr (MB == 4)
@@ -416,11 +424,21 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
 
-    for (int k = 0; k < nk; k += R) {
-      step(std::integral_constant<int, 0>{}, k);
-      step(std::integral_constant<int, 1>{}, k + 1);
-      step(std::integral_constant<int, 2>{}, k + 2);
-      step(std::integral_constant<int, 3>{}, k + 3);
+    int k = 0;
+    if constexpr (RAGGED) {
+      // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
+      for (; k + 2 * R <= nk_real; k += R) {
+        step(std::integral_constant<int, 0>{}, k, std::true_type{});
+        step(std::integral_constant<int, 1>{}, k + 1, std::true_type{});
+        step(std::integral_constant<int, 2>{}, k + 2, std::true_type{});
+        step(std::integral_constant<int, 3>{}, k + 3, std::true_type{});
+      }
+    }
+    for (; k < nk; k += R) {
+      step(std::integral_constant<int, 0>{}, k, std::false_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, std::false_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, std::false_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, std::false_type{});
     }
     // the ring already holds the next tile's first steps; move the tile window on
     a_cur = a_nxt;
