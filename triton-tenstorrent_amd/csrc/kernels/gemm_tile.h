@@ -278,9 +278,11 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if (RAGGED && MB == 2 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
-    if constexpr (RAGGED) {
-      const int last_row = Mf - 1 - (int)row0;                // >= 0
-      const int last_chunk = (Nf - tn * BN) / 8 - 1;          // >= 0: the fetchable N is a multiple of 8
+    {
+      // per-thread offsets of the tile's copies from ap / bp, one per A slab (RAGGED: rows and column chunks
+      // clamped into the matrix)
+      const int last_row = RAGGED ? Mf - 1 - (int)row0 : BM;  // >= 0
+      const int last_chunk = RAGGED ? (Nf - tn * BN) / 8 - 1 : 32;   // >= 0: the fetchable N is a multiple of 8
 #pragma unroll
       for (int i = 0; i < MB; ++i) {
         const int r = min(i * 64 + a_row, last_row);
@@ -294,13 +296,14 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   };
   // copy number i (0..MB-1: A slabs, MB..MB+3: B slabs) of step kk into `stage`; kk may run past
   // nk into the next tile
-  // `inner` (RAGGED only): the caller knows that step kk belongs to this tile and carries data, so the choices
-  // between this tile and the next and between data and the page of zeros are not made at run time
+  // `inner`: the caller knows that step kk belongs to this tile and carries data, so the choices between this
+  // tile and the next and (RAGGED) between data and the page of zeros are not made at run time, and a copy's
+  // source is one scalar address per operand and step plus the thread's offset for that slab
   auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_) {
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
-    if constexpr (RAGGED && inner) {
+    if constexpr (inner) {
       if (i < MB)
         dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
       else
@@ -425,14 +428,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
 
     int k = 0;
-    if constexpr (RAGGED) {
-      // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
-      for (; k + 2 * R <= nk_real; k += R) {
-        step(std::integral_constant<int, 0>{}, k, std::true_type{});
-        step(std::integral_constant<int, 1>{}, k + 1, std::true_type{});
-        step(std::integral_constant<int, 2>{}, k + 2, std::true_type{});
-        step(std::integral_constant<int, 3>{}, k + 3, std::true_type{});
-      }
+    // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
+    for (; k + 2 * R <= nk_real; k += R) {
+      step(std::integral_constant<int, 0>{}, k, std::true_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, std::true_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, std::true_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, std::true_type{});
     }
     for (; k < nk; k += R) {
       step(std::integral_constant<int, 0>{}, k, std::false_type{});

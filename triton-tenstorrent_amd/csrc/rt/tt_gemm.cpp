@@ -110,7 +110,8 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   // the problem (then the assignment of output to programs does not show in the result).
   const bool full_grid = (int64_t)grid[0] == num_pid_m * num_pid_n;
   const bool half_io = (in == TT_BF16 && out == TT_BF16) || (in == TT_F16 && out == TT_F16);
-  const bool fast_shape = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
+  // (leading strides below 2^23 elements: a thread's offset from its tile's first row is a 32-bit byte count)
+  const bool fast_shape = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128 && g.lda < (1 << 23) && g.ldb < (1 << 23);
   const bool fast_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 8 == 0 &&
                           g.ldb % 8 == 0 && g.ldc % 8 == 0;
   // The same kernel with clamped fetches, zero-padded K steps and clipped stores takes every other shape
