@@ -269,7 +269,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   struct Voffs { uint32_t a[4]; uint32_t b; };
   Voffs vo_cur, vo_nxt;
   const uint32_t z_voff = (uint32_t)tid * 16;
-  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
+  // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
+  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo, bool offsets = RAGGED) {
     int tm, tn, half;
     item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, half);
     int64_t row0 = (int64_t)tm * BM + half * 128;
@@ -278,7 +279,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if (RAGGED && MB == 2 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
-    {
+    if (RAGGED || offsets) {
       // per-thread offsets of the tile's copies from ap / bp, one per A slab (RAGGED: rows and column chunks
       // clamped into the matrix)
       const int last_row = RAGGED ? Mf - 1 - (int)row0 : BM;  // >= 0
@@ -402,8 +403,13 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // ---- fill the ring: steps 0..R-1 of the first tile ----
   int t = blockIdx.x;
   if (t >= total) return;
-  tile_bases(t, a_cur, b_cur, vo_cur);
-  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
+  tile_bases(t, a_cur, b_cur, vo_cur, true);
+  // no copy of the fill looks at the next tile.  RAGGED: where it lies is worked out before the last turns of each
+  // tile, so that its offsets are not held through the turns before; whole tiles: one tile ahead, at the end of a tile
+  a_nxt = a_cur;
+  b_nxt = b_cur;
+  vo_nxt = vo_cur;
+  if constexpr (!RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
   // steps 0..R-2 whole, and the first half of step R-1 (step 0's first sub-step issues the rest)
 #pragma unroll
   for (int s = 0; s < R; ++s)
@@ -435,6 +441,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       step(std::integral_constant<int, 2>{}, k + 2, std::true_type{});
       step(std::integral_constant<int, 3>{}, k + 3, std::true_type{});
     }
+    // the remaining turns copy the next tile's first steps (this tile's again when there is none: a harmless
+    // refetch); RAGGED: where that tile lies is worked out only now
+    if constexpr (RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
     for (; k < nk; k += R) {
       step(std::integral_constant<int, 0>{}, k, std::false_type{});
       step(std::integral_constant<int, 1>{}, k + 1, std::false_type{});
@@ -444,8 +453,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // the ring already holds the next tile's first steps; move the tile window on
     a_cur = a_nxt;
     b_cur = b_nxt;
-    vo_cur = vo_nxt;
-    {
+    if constexpr (RAGGED) {
+      vo_cur = vo_nxt;
+    } else {
+      // whole tiles: only the two addresses change from tile to tile; the tile after the next
       const int t2 = t + 2 * (int)gridDim.x;
       tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt, vo_nxt);
     }

@@ -114,7 +114,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   struct Voffs { uint32_t a[4]; uint32_t b; };   // RAGGED: a tile's per-thread offsets, clamped into the matrix
   Voffs vo_cur, vo_nxt;
   const uint32_t z_voff = (uint32_t)tid * 16;
-  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo) {
+  // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
+  auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo, bool offsets = RAGGED) {
     int tm, tn, half;
     fast::item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, half);
     int64_t row0 = (int64_t)tm * BM + half * 128;
@@ -123,18 +124,25 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     if (RAGGED && MB == 2 && row0 >= g.M) row0 = (int64_t)tm * BM;
     ap = A + row0 * g.lda;
     bp = B + (int64_t)tn * BN;
-    if constexpr (RAGGED) {
-      const int last_row = g.M - 1 - (int)row0;
-      const int last_chunk = (g.N - tn * BN) / 16 - 1;        // N is a multiple of 16
+    if (RAGGED || offsets) {
+      const int last_row = RAGGED ? g.M - 1 - (int)row0 : BM;
+      const int last_chunk = RAGGED ? (g.N - tn * BN) / 16 - 1 : 16;        // N is a multiple of 16
 #pragma unroll
       for (int i = 0; i < MB; ++i) vo.a[i] = (uint32_t)((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 16);
       vo.b = (uint32_t)((int64_t)b_k * g.ldb + min(b_chunk, last_chunk) * 16);
     }
   };
-  auto dma_single = [&](int kk, uint8_t *stage, int i) {
-    const bool over = kk >= nk;
+  // `inner`: step kk belongs to this tile and carries data (see the 16-bit kernel)
+  auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_) {
+    constexpr bool inner = decltype(inner_)::value;
+    const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
-    if constexpr (RAGGED) {
+    if constexpr (inner) {
+      if (i < MB)
+        dma_one(a_cur + (int64_t)k * BK, vo_cur.a[i], stage + i * 4096);
+      else
+        dma_one(b_cur + (int64_t)k * b_kstep + (i - MB) * b_slab, vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
+    } else if constexpr (RAGGED) {
       const bool zero = k >= nk_real;
       const Voffs &vo = over ? vo_nxt : vo_cur;
       if (i < MB) {
@@ -155,7 +163,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
   // One step (K += 64) on ring stage I: 16 MFMAs on `c` (read from stage I during the previous
   // step), the next stage's fragments into `p`, and the refill of stage I itself with step k+R.
-  auto step = [&](auto I_, int k, Frags &c, Frags &p) {
+  auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_) {
     constexpr int I = decltype(I_)::value;
     uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
     mm(c, 0);
@@ -172,7 +180,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
           rd(p, nxt, 2 * (n - 1));
           rd(p, nxt, 2 * (n - 1) + 1);
         }
-        if (n & 1) dma_single(k + R, cur, n >> 1); // one copy per two MFMAs: thin enough not to stall issue
+        if (n & 1) dma_single(k + R, cur, n >> 1, inner_); // one copy per two MFMAs: thin enough not to stall issue
         mm(c, n);
         FENCE();
       }
@@ -185,7 +193,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
       for (int n = 1; n < 8; ++n) {
 #pragma unroll
         for (int r = 3 * (n - 1); r < 3 * n && r < 20; ++r) rd(p, nxt, r);
-        if (n <= 6) dma_single(k + R, cur, n - 1);
+        if (n <= 6) dma_single(k + R, cur, n - 1, inner_);
         mm(c, n);
         FENCE();
       }
@@ -194,13 +202,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
   int t = blockIdx.x;
   if (t >= total) return;
-  tile_bases(t, a_cur, b_cur, vo_cur);
-  tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
+  tile_bases(t, a_cur, b_cur, vo_cur, true);
+  // no copy of the fill looks at the next tile.  RAGGED: where it lies is worked out before the last turns of each
+  // tile, so that its offsets are not held through the turns before; whole tiles: one tile ahead, at the end of a tile
+  a_nxt = a_cur;
+  b_nxt = b_cur;
+  vo_nxt = vo_cur;
+  if constexpr (!RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
   // fill the ring with steps 0..R-1
 #pragma unroll
   for (int s = 0; s < R; ++s)
 #pragma unroll
-    for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i);
+    for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
   // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
   if constexpr (MB == 4)
     asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -217,16 +230,29 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     for (int i = 0; i < MB; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
-    for (int k = 0; k < nk; k += R) {
-      step(std::integral_constant<int, 0>{}, k, f0, f1);
-      step(std::integral_constant<int, 1>{}, k + 1, f1, f0);
-      step(std::integral_constant<int, 2>{}, k + 2, f0, f1);
-      step(std::integral_constant<int, 3>{}, k + 3, f1, f0);
+    int k = 0;
+    // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
+    for (; k + 2 * R <= nk_real; k += R) {
+      step(std::integral_constant<int, 0>{}, k, f0, f1, std::true_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::true_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::true_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::true_type{});
+    }
+    // the remaining turns copy the next tile's first steps (this tile's again when there is none: a harmless
+    // refetch); RAGGED: where that tile lies is worked out only now
+    if constexpr (RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
+    for (; k < nk; k += R) {
+      step(std::integral_constant<int, 0>{}, k, f0, f1, std::false_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::false_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::false_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::false_type{});
     }
     a_cur = a_nxt;
     b_cur = b_nxt;
-    vo_cur = vo_nxt;
-    {
+    if constexpr (RAGGED) {
+      vo_cur = vo_nxt;
+    } else {
+      // whole tiles: only the two addresses change from tile to tile; the tile after the next
       const int t2 = t + 2 * (int)gridDim.x;
       tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt, vo_nxt);
     }

@@ -143,7 +143,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
 
   // fp8 fast path: e4m3 in, bf16/fp16 out, scale in the epilogue, K in steps of 64 through a 4-stage ring
   const bool fp8_io = in == TT_FP8E4M3 && (out == TT_BF16 || out == TT_F16 || out == TT_FP8E4M3) && epi == TT_EPI_NONE;
-  const bool fp8_shape = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
+  const bool fp8_shape = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256 && g.lda < (1 << 24) && g.ldb < (1 << 24);
   const bool fp8_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 16 == 0 && g.ldb % 16 == 0 &&
                          g.ldc % 4 == 0;
   const bool fp8_ragged = !fp8_shape && N % 16 == 0 && K % 64 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24);
