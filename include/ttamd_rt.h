@@ -238,7 +238,10 @@ TTAMD_API int tt_copy_kernel(const void *x, void *out, int32_t n_elements, int32
  * (tie_break_left; without it any such index is a legal result).  Float min / max drop NaN operands
  * (arith.minnumf / maxnumf) unless propagate_nan (arith.minimumf / maximumf); the index reductions
  * on NaN input return an index that depends on the fold order, as the reference's do.
- * Every program of the grid would store the same value; it is computed once. */
+ * Every program of the grid would store the same value; it is computed once.  Blocks of 128 KiB and more
+ * (16-byte aligned) are folded by several workgroups through a small device buffer that the library keeps
+ * per (device, stream): the first such call on a stream allocates it (never while the stream is recording a
+ * graph: one workgroup then does the work), and calls on different streams do not share it. */
 typedef enum tt_reduce_op {
   TT_REDUCE_SUM = 0, TT_REDUCE_MIN = 1, TT_REDUCE_MAX = 2, TT_REDUCE_ARGMIN = 3, TT_REDUCE_ARGMAX = 4,
   TT_REDUCE_XOR_SUM = 5
