@@ -67,3 +67,47 @@ def test_matmul_and_attention_in_a_graph():
         torch.cuda.synchronize()
         assert rt.last_kernel_name() is not None
         assert torch.equal(res["c"], eager["c"]) and torch.equal(res["o"], eager["o"]), rep
+
+
+def test_large_reduction_in_a_graph():
+    """A reduction of 128 KiB and more runs on several workgroups through a per-stream buffer that the first
+    call on a stream allocates.  Recorded on a stream that has no buffer yet it must not allocate (one workgroup
+    runs); recorded on a stream that has one, the multi-workgroup kernel goes into the graph and its arrival
+    counter is back at zero after every replay."""
+    n = 1 << 20
+    x = torch.randint(-2**31, 2**31 - 1, (n, ), device="cuda", dtype=torch.int64).to(torch.int32)
+    z = torch.zeros(1, device="cuda", dtype=torch.int32)
+    za = torch.zeros(1, device="cuda", dtype=torch.int32)
+
+    def work():
+        K.reduce1d_kernel[(1, )](x, z, BLOCK=n, OP="sum")
+        K.reduce1d_kernel[(1, )](x, za, BLOCK=n, OP="argmax")
+
+    # a fresh side stream: nothing may be allocated while it records
+    fresh = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    g1 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1, stream=fresh):
+        work()
+    # a side stream that has run the reduction before
+    warm = torch.cuda.Stream()
+    with torch.cuda.stream(warm):
+        work()
+    torch.cuda.synchronize()
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2, stream=warm):
+        work()
+    for rep in range(4):
+        x.copy_(torch.randint(-2**31, 2**31 - 1, (n, ), device="cuda", dtype=torch.int64).to(torch.int32))
+        torch.cuda.synchronize()
+        want_sum = int(x.sum(dtype=torch.int64).item()) & 0xffffffff
+        want_arg = int(torch.argmax(x).item())           # ties are as good as impossible in 2^20 draws from 2^32
+        for g in (g1, g2):
+            z.fill_(-7)
+            za.fill_(-7)
+            g.replay()
+            torch.cuda.synchronize()
+            assert int(z.item()) & 0xffffffff == want_sum and int(za.item()) == want_arg, rep
+        work()                                           # and eagerly, between the replays
+        torch.cuda.synchronize()
+        assert int(z.item()) & 0xffffffff == want_sum and int(za.item()) == want_arg
