@@ -16,8 +16,9 @@
  *
  * Pinning status (what independent check fixes each function) is listed in
  * oracle/README.md and exercised by tests/test_oracle_*.py:
- *   orc_block_range, orc_pid_decode, orc_tile_of_pid : brute-force coverage /
- *       bijection properties
+ *   orc_block_range, orc_pid_decode, orc_tile_of_pid, orc_tile_of_pid_pointer :
+ *       brute-force coverage / bijection properties, a literal transcription of
+ *       both sources' decode on a grid with a short last group
  *   orc_add_*      : closed form (numpy), bit-exact
  *   orc_sin_f32    : float64 libm sin rounded once to fp32
  *   orc_unary/binary_f32: numpy's float32 operations bit for bit where the operation is
@@ -204,6 +205,23 @@ ORC_API void orc_tile_of_pid(int pid, int num_pid_m, int num_pid_n, int group_m,
   int group_size_m = num_pid_m - first_pid_m;
   if (group_size_m > group_m) group_size_m = group_m;
   *pid_m = first_pid_m + (pid % group_size_m);
+  *pid_n = (pid % num_pid_in_group) / group_size_m;
+}
+
+/* The pointer-based matmul_kernel decodes its program id differently
+ * (examples/matmul/03-matrix-multiplication.py:273-282): the row inside a group
+ * is taken from the position inside the group, not from the program id itself:
+ *   pid_m = first_pid_m + ((pid % num_pid_in_group) % group_size_m).
+ * The two forms agree whenever group_id * num_pid_in_group is a multiple of
+ * group_size_m, i.e. always except in a last, shorter group. */
+ORC_API void orc_tile_of_pid_pointer(int pid, int num_pid_m, int num_pid_n, int group_m,
+                                     int *pid_m, int *pid_n) {
+  int num_pid_in_group = group_m * num_pid_n;
+  int group_id = pid / num_pid_in_group;
+  int first_pid_m = group_id * group_m;
+  int group_size_m = num_pid_m - first_pid_m;
+  if (group_size_m > group_m) group_size_m = group_m;
+  *pid_m = first_pid_m + ((pid % num_pid_in_group) % group_size_m);
   *pid_n = (pid % num_pid_in_group) / group_size_m;
 }
 
@@ -698,7 +716,8 @@ ORC_API int orc_matmul(const void *a, int64_t lda, const void *b, int64_t ldb, v
  * masked on k < K only (:340-342, 359-361), the store on m < M and n < N (:387-388).
  * acc is fp32 (:320), the activation acts on it before the cast (:370-374), and the
  * result is always cast to fp16 (:374).  The strides in the signature are not used
- * by the kernel (:251-253) and are not taken here.  Program order as orc_matmul.
+ * by the kernel (:251-253) and are not taken here.  Programs are split over workers
+ * as in orc_matmul; the program id is decoded by orc_tile_of_pid_pointer (:273-282).
  */
 ORC_API int orc_matmul_tiled(const void *a, const void *b, void *c, int32_t M, int32_t N, int32_t K,
                              int32_t BM, int32_t BN, int32_t BK, int32_t group_m, int32_t grid,
@@ -723,7 +742,7 @@ ORC_API int orc_matmul_tiled(const void *a, const void *b, void *c, int32_t M, i
     orc_block_range(grid, nw, w, &bs, &be);
     for (int64_t pid = bs; pid < be; ++pid) {
       int pid_m, pid_n;
-      orc_tile_of_pid((int)pid, num_pid_m, num_pid_n, group_m, &pid_m, &pid_n);
+      orc_tile_of_pid_pointer((int)pid, num_pid_m, num_pid_n, group_m, &pid_m, &pid_n);
       int64_t om = (int64_t)pid_m * BM, on = (int64_t)pid_n * BN;
       for (int i = 0; i < BM * BN; ++i) accf[i] = 0.0f;
       if (acc64) for (int i = 0; i < BM * BN; ++i) accd[i] = 0.0;

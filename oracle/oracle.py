@@ -53,6 +53,8 @@ def lib() -> C.CDLL:
         L.orc_pid_decode.restype = None
         L.orc_tile_of_pid.argtypes = [C.c_int] * 4 + [C.POINTER(C.c_int)] * 2
         L.orc_tile_of_pid.restype = None
+        L.orc_tile_of_pid_pointer.argtypes = [C.c_int] * 4 + [C.POINTER(C.c_int)] * 2
+        L.orc_tile_of_pid_pointer.restype = None
         for name in ("orc_add_f32", "orc_add_i32"):
             f = getattr(L, name)
             f.argtypes = [vp, vp, vp, i32, i32, i32, C.c_int]
@@ -154,6 +156,13 @@ def pid_decode(b: int, gx: int, gy: int) -> tuple[int, int, int]:
 def tile_of_pid(pid: int, num_pid_m: int, num_pid_n: int, group_m: int) -> tuple[int, int]:
     m, n = C.c_int(), C.c_int()
     lib().orc_tile_of_pid(pid, num_pid_m, num_pid_n, group_m, C.byref(m), C.byref(n))
+    return m.value, n.value
+
+
+def tile_of_pid_pointer(pid: int, num_pid_m: int, num_pid_n: int, group_m: int) -> tuple[int, int]:
+    """The pointer-based matmul_kernel's decode (03-matrix-multiplication.py:273-282)."""
+    m, n = C.c_int(), C.c_int()
+    lib().orc_tile_of_pid_pointer(pid, num_pid_m, num_pid_n, group_m, C.byref(m), C.byref(n))
     return m.value, n.value
 
 

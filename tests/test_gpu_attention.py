@@ -189,3 +189,25 @@ def test_full_size_attention_properties():
     del o, M
     o1 = K.attention(q, k, torch.ones_like(v), True, sm)
     assert (o1.float() - 1).abs().max() <= 1e-2
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("S,D,kernel", [(256, 128, "attn_tile_d128"), (256, 64, "attn_tile_d64"), (224, 128, "attn_ragged_d128"),
+                                        (128, 256, "attn_tile_d256"), (64, 16, "attn_any_d16")])
+def test_p_is_rounded_to_bf16_and_l_is_summed_before_the_cast(causal, S, D, kernel):
+    """06-fused-attention.py:65-83 on the constructed input of util.p_cast_case: a kernel that fed fp32 P into the
+    second product would put 0.2-1.7 where the last row of O is exactly 0, and one that summed l after the cast would
+    move M by 5e-3 (the bar is 1e-3)."""
+    from triton_tenstorrent_amd import runtime as rt
+    from util import from_bits, p_cast_case
+    q, k, v, sm, models = p_cast_case(S, D)
+    tq, tk, tv = (from_bits(t, torch.bfloat16) for t in (q, k, v))
+    o, M = K.attention(tq, tk, tv, causal, sm, return_lse=True)
+    assert rt.last_kernel_name() == kernel
+    wo, wM = models[("faithful", causal)]
+    o, M = decode(o)[0, 0], M.cpu().numpy()[0, 0]
+    assert np.all(np.abs(o - wo) <= 2.0 ** -8 * np.abs(wo) + O_ATOL) and np.max(np.abs(M - wM)) <= M_ATOL
+    assert np.all(o[-1] == 0.0)
+    bm = 32 if S % 64 else 64
+    ro, rM = orc.attn_fwd(q, k, v, sm, causal=causal, BLOCK_M=bm, BLOCK_N=min(bm, D))
+    assert np.all(np.abs(o - orc.from_bf16(ro)[0, 0]) <= 2.0 ** -8 * np.abs(wo) + O_ATOL) and np.max(np.abs(M - rM[0, 0])) <= M_ATOL

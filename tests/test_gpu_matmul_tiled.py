@@ -120,6 +120,31 @@ def test_partial_grid_and_errors():
         K.matmul_tiled(K.tilize(a, 48, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, 32, BLOCK_SIZE_M=48)
 
 
+def test_partial_grid_in_a_short_last_group_follows_the_pointer_decode():
+    """5x3 tiles in groups of 3: the last group has 2 rows and starts at an odd program id, where the row taken from
+    the position inside the group (03-matrix-multiplication.py:281) and the row taken from the program id itself
+    (the descriptor kernels) name different tiles.  12 of 15 programs: the oracle and the kernel must leave the same
+    three tiles of the result untouched."""
+    M, N, K_ = 160, 96, 64
+    a, b = _rand((M, K_), 12), _rand((K_, N), 13)
+    at, bt = K.tilize(a, 32, 32), K.tilize(b, 32, 32)
+    for grid in (10, 12, 14):
+        c = torch.full((15 * 1024, ), float("nan"), dtype=torch.float16, device="cuda")
+        K.matmul_kernel[(grid, )](at.cuda(), bt.cuda(), c, M, N, K_, K_, 1, N, 1, N, 1, GROUP_SIZE_M=3)
+        assert rt.last_kernel_name() == "gemm_anytiled_f16_f16"
+        ref = orc.matmul_tiled(_bits(at), _bits(bt), M, N, K_, group_m=3, grid=grid, acc64=True,
+                               out=np.full(15 * 1024, 0x7e00, dtype=np.uint16))
+        got = _bits(c.cpu())
+        untouched = np.isnan(_f16(ref))
+        assert np.array_equal(np.isnan(_f16(got)), untouched) and untouched.sum() == (15 - grid) * 1024
+        assert _close(_f16(got)[~untouched], _f16(ref)[~untouched])
+        if grid == 12:
+            # hand-worked: programs 9, 10, 11 are tiles (3,0), (4,0), (3,1); in the tile-major result tile (i,j) is
+            # block i*3 + j, so blocks 12 (4,0) and 9, 10 are written and 11, 13, 14 are not
+            blocks = {t for t in range(15) if not np.isnan(_f16(got[t * 1024:(t + 1) * 1024])).any()}
+            assert blocks == set(range(9)) | {9, 12, 10}
+
+
 @pytest.mark.parametrize("act", ["", "leaky_relu"])
 def test_fast_path_tiled(act):
     M, N, K_ = 512, 768, 256

@@ -99,3 +99,22 @@ def test_rejects_block_n_above_head_dim():
     q, k, v = _qkv(5, 1, 1, 64, 32)
     with pytest.raises(ValueError):
         orc.attn_fwd(q, k, v, 1.0, BLOCK_M=64, BLOCK_N=64)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("BM,BN", [(32, 32), (64, 32)])
+def test_p_is_rounded_to_bf16_and_l_is_summed_before_the_cast(causal, BM, BN):
+    """06-fused-attention.py:65-83: l_ij = sum(p) in fp32, then p.to(bf16) feeds the second dot.  On the constructed
+    input an oracle that left P in fp32 puts 0.2-1.7 into the last row of O where the source gives 0, and one that
+    summed l after the cast moves M by 5e-3."""
+    from util import p_cast_case
+    S, D = 64, 32
+    q, k, v, sm, models = p_cast_case(S, D)
+    o, M = orc.attn_fwd(q, k, v, sm, causal=causal, BLOCK_M=BM, BLOCK_N=BN)
+    o, M = orc.from_bf16(o)[0, 0], M[0, 0]
+    wo, wM = models[("faithful", causal)]
+    assert np.all(np.abs(o - wo) <= 2.0 ** -8 * np.abs(wo) + 2e-2) and np.max(np.abs(M - wM)) <= 1e-3
+    assert np.all(o[-1] == 0.0)
+    # the construction discriminates: each wrong reading is far outside those bars
+    assert np.min(np.abs(models[("p_not_rounded", causal)][0][-1])) > 0.2
+    assert abs(models[("l_after_cast", causal)][1][-1] - wM[-1]) > 4e-3

@@ -72,3 +72,20 @@ def test_partial_grid_leaves_other_tiles_untouched():
     out = np.full(4 * 32 * 32, 0x7e00, dtype=np.uint16)
     orc.matmul_tiled(orc.tilize(a.view(np.uint16), 32, 32), orc.tilize(b.view(np.uint16), 32, 32), M, N, 32, grid=3, out=out)
     assert np.all(out[3 * 1024:] == 0x7e00) and not np.any(out[:3 * 1024] == 0x7e00)
+
+
+def test_partial_grid_writes_the_tiles_the_pointer_decode_names():
+    """matmul_kernel takes its row from the position inside the group (03-matrix-multiplication.py:281); on 5x3 tiles
+    in groups of 3 the first 12 programs therefore write tiles (3,0), (4,0), (3,1) of the last group, not
+    (4,0), (3,0), (4,1) as the descriptor kernels' decode would."""
+    M, N, K = 160, 96, 32
+    rng = np.random.default_rng(5)
+    a = rng.integers(1, 4, (M, K)).astype(np.float16).view(np.uint16)
+    b = rng.integers(1, 4, (K, N)).astype(np.float16).view(np.uint16)
+    c = orc.matmul_tiled(orc.tilize(a, 32, 32), orc.tilize(b, 32, 32), M, N, K, group_m=3, grid=12)
+    written = {(t // 3, t % 3) for t in range(15) if c[t * 1024:(t + 1) * 1024].any()}
+    assert written == {(i, j) for i in range(3) for j in range(3)} | {(3, 0), (4, 0), (3, 1)}
+    want = a.view(np.float16).astype(np.float32) @ b.view(np.float16).astype(np.float32)
+    got = orc.untilize(c, M, N, 32, 32).view(np.float16).astype(np.float32)
+    for (i, j) in written:
+        assert np.array_equal(got[i * 32:(i + 1) * 32, j * 32:(j + 1) * 32], want[i * 32:(i + 1) * 32, j * 32:(j + 1) * 32])

@@ -53,3 +53,42 @@ def test_group_swizzle_is_a_bijection(npm, npn, g):
 def test_group_swizzle_walks_down_columns_inside_a_group():
     # with G=4 the first 4 pids share pid_n=0 and step pid_m
     assert [orc.tile_of_pid(p, 8, 8, 4) for p in range(5)] == [(0, 0), (1, 0), (2, 0), (3, 0), (0, 1)]
+
+
+def _decode_descriptor(pid, num_pid_m, num_pid_n, GROUP_SIZE_M):
+    """09-persistent-matmul.py:118-126, transcribed statement by statement."""
+    num_pid_in_group = GROUP_SIZE_M * num_pid_n
+    group_id = pid // num_pid_in_group
+    first_pid_m = group_id * GROUP_SIZE_M
+    group_size_m = min(num_pid_m - first_pid_m, GROUP_SIZE_M)
+    pid_m = first_pid_m + (pid % group_size_m)
+    pid_n = (pid % num_pid_in_group) // group_size_m
+    return pid_m, pid_n
+
+
+def _decode_pointer(pid, num_pid_m, num_pid_n, GROUP_SIZE_M):
+    """03-matrix-multiplication.py:276-282, transcribed statement by statement."""
+    num_pid_in_group = GROUP_SIZE_M * num_pid_n
+    group_id = pid // num_pid_in_group
+    first_pid_m = group_id * GROUP_SIZE_M
+    group_size_m = min(num_pid_m - first_pid_m, GROUP_SIZE_M)
+    pid_m = first_pid_m + ((pid % num_pid_in_group) % group_size_m)
+    pid_n = (pid % num_pid_in_group) // group_size_m
+    return pid_m, pid_n
+
+
+@pytest.mark.parametrize("npm,npn,g", [(5, 3, 3), (7, 5, 4), (64, 64, 8), (3, 9, 16), (9, 7, 5), (1, 1, 1)])
+def test_both_decodes_follow_their_sources(npm, npn, g):
+    for p in range(npm * npn):
+        assert orc.tile_of_pid(p, npm, npn, g) == _decode_descriptor(p, npm, npn, g)
+        assert orc.tile_of_pid_pointer(p, npm, npn, g) == _decode_pointer(p, npm, npn, g)
+    tiles = [orc.tile_of_pid_pointer(p, npm, npn, g) for p in range(npm * npn)]
+    assert sorted(tiles) == sorted(itertools.product(range(npm), range(npn)))
+
+
+def test_the_two_decodes_differ_in_a_short_last_group():
+    # 5 rows of tiles in groups of 3, 3 columns: the last group has 2 rows and starts at program 9, which is odd,
+    # so `pid % 2` and `(pid % 9) % 2` disagree (hand-worked: program 9 is the group's first -> row 3 by position)
+    assert orc.tile_of_pid_pointer(9, 5, 3, 3) == (3, 0) and orc.tile_of_pid(9, 5, 3, 3) == (4, 0)
+    assert orc.tile_of_pid_pointer(10, 5, 3, 3) == (4, 0) and orc.tile_of_pid(10, 5, 3, 3) == (3, 0)
+    assert orc.tile_of_pid_pointer(11, 5, 3, 3) == (3, 1) and orc.tile_of_pid(11, 5, 3, 3) == (4, 1)

@@ -63,7 +63,8 @@ __device__ __forceinline__ void gemm_any_body(const GemmArgs &g) {
   for (int64_t it = (int64_t)blockIdx.x * waves_per_block + wave; it < items; it += stride) {
     const int pid = (int)(it / spt), sub = (int)(it % spt);
     int pid_m, pid_n;
-    tile_of_pid(pid, g.num_pid_m, g.num_pid_n, g.group_m, pid_m, pid_n);
+    if constexpr (TILED) tile_of_pid_pointer(pid, g.num_pid_m, g.num_pid_n, g.group_m, pid_m, pid_n);
+    else tile_of_pid(pid, g.num_pid_m, g.num_pid_n, g.group_m, pid_m, pid_n);
     const int64_t m0 = (int64_t)pid_m * g.BM + (sub / sub_n) * 32;
     const int64_t n0 = (int64_t)pid_n * g.BN + (sub % sub_n) * 32;
     if (m0 >= g.M || n0 >= g.N) continue; // piece lies wholly in the padding (wave-uniform)

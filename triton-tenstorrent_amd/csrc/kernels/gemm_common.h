@@ -112,6 +112,19 @@ __device__ __forceinline__ void tile_of_pid(int pid, int num_pid_m, int num_pid_
   pid_n = (pid % num_pid_in_group) / group_size_m;
 }
 
+// The pointer-based matmul_kernel takes the row from the position inside the group
+// (examples/matmul/03-matrix-multiplication.py:281); the two decodes differ only in a last, shorter group.
+__device__ __forceinline__ void tile_of_pid_pointer(int pid, int num_pid_m, int num_pid_n, int group_m,
+                                                    int &pid_m, int &pid_n) {
+  int num_pid_in_group = group_m * num_pid_n;
+  int group_id = pid / num_pid_in_group;
+  int first_pid_m = group_id * group_m;
+  int group_size_m = min(num_pid_m - first_pid_m, group_m);
+  int in_group = pid % num_pid_in_group;
+  pid_m = first_pid_m + (in_group % group_size_m);
+  pid_n = in_group / group_size_m;
+}
+
 // erf-form GELU, 0.5*x*(1+erf(x/sqrt(2))).  erf by Abramowitz & Stegun 7.1.26,
 // erf(z) = 1 - (a1 t + ... + a5 t^5) exp(-z^2) for z >= 0 with t = 1/(1 + p z): absolute error <= 1.5e-7,
 // branch-free, one rcp and one exp2 instead of the library routine's ~40 operations (the epilogue runs on

@@ -62,7 +62,7 @@ def matmul_kernel(a_ptr, b_ptr, c_ptr, M, N, K, stride_am, stride_ak, stride_bk,
     width = GROUP_SIZE_M * num_pid_n
     first_pid_m = (pid // width) * GROUP_SIZE_M
     rows = min(num_pid_m - first_pid_m, GROUP_SIZE_M)
-    pid_m = first_pid_m + (pid % rows)
+    pid_m = first_pid_m + ((pid % width) % rows)
     pid_n = (pid % width) // rows
     num_k = tl.cdiv(K, BLOCK_SIZE_K)
     im = tl.arange(0, BLOCK_SIZE_M)
