@@ -124,6 +124,7 @@ def main() -> int:
                    "clock_mhz": props["clock_khz"] // 1000,
                    "peaks": {"hbm_GBs": PEAK_HBM_GBS, "bf16_TFLOPs": PEAK_BF16_TFLOPS, "fp8_TFLOPs": PEAK_FP8_TFLOPS}}
     rooflines: dict = {}
+    parity_failed = False
     torch.manual_seed(0)
 
     # ---------------- primary: persistent bf16 GEMM 8192^3 -----------------
@@ -269,7 +270,13 @@ def main() -> int:
         extra["gemm_gelu_4096x14336x4096"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
                                               "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
         rooflines["gemm_gelu_4096x14336x4096"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_tile_bf16_epi2")
-        del a, b, c, bias
+        # spot parity on the timed output: 64 random rows against float64 erf-GELU
+        rows = torch.randint(0, Mf, (64, ), device="cuda")
+        ref = torch.nn.functional.gelu(a[rows].double() @ b.double() + bias.double()).float()
+        ok = bool(torch.all((c[rows].float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4))
+        extra["gemm_gelu_4096x14336x4096"]["parity_rows_ok"] = ok
+        parity_failed |= not ok
+        del a, b, c, bias, ref
     if want("fp8"):
         xa = torch.randn(M, Kd, device="cuda")
         qa, sa = K.quantize_fp8(xa)
@@ -287,7 +294,15 @@ def main() -> int:
         extra["gemm_fp8_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4), "ms_min": round(min(per), 4),
                                   "TFLOPs": round(tf, 2)}
         rooflines["gemm_fp8_8192"] = _roof("mfma", tf, PEAK_FP8_TFLOPS, "TFLOP/s", "gemm_tile_fp8_bf16")
-        del qa, qb, c
+        # spot parity: 64 random rows against float64 on the dequantised operands; the absolute slack follows the
+        # output's rms, since fp8 products summed over K cancel to values no relative bound can hold
+        rows = torch.randint(0, M, (64, ), device="cuda")
+        ref = ((qa[rows].double() @ qb.double()) * (sa * sb)).float()
+        atol = 1e-4 * max(1.0, float(ref.square().mean().sqrt()))
+        ok = bool(torch.all((c[rows].float() - ref).abs() <= 1e-2 * ref.abs() + atol))
+        extra["gemm_fp8_8192"]["parity_rows_ok"] = ok
+        parity_failed |= not ok
+        del qa, qb, c, ref
     if want("tiled"):
         # the pointer-based matmul_kernel on tile-major fp16 buffers, 32x32x32 tiles, same 8192^3 problem
         at = K.tilize((torch.randn(M, Kd, device="cuda") / math.sqrt(Kd)).to(torch.float16), 32, 32)
@@ -300,18 +315,41 @@ def main() -> int:
         extra["gemm_tiled_f16_8192"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
                                         "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
         rooflines["gemm_tiled_f16_8192"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "gemm_tiled_f16_epi0")
-        del at, bt, ct
+        # spot parity: 64 random rows of the un-tiled result against float64 on the un-tiled operands
+        rows = torch.randint(0, M, (64, ), device="cuda")
+        a_rows = K.untilize(at, M, Kd, 32, 32)[rows].double()
+        ref = (a_rows @ K.untilize(bt, Kd, N, 32, 32).double()).float()
+        got = K.untilize(ct, M, N, 32, 32)[rows].float()
+        ok = bool(torch.all((got - ref).abs() <= 1e-2 * ref.abs() + 1e-4))
+        extra["gemm_tiled_f16_8192"]["parity_rows_ok"] = ok
+        parity_failed |= not ok
+        del at, bt, ct, ref, got, a_rows
     if want("attn"):
         Z, H, S, D = 4, 32, 4096, 128
         q, k, v = (torch.randn(Z, H, S, D, device="cuda").to(torch.bfloat16) for _ in range(3))
         sm = 1.0 / math.sqrt(D)
-        avg_ms, per, _ = _events_time(lambda: K.attention(q, k, v, True, sm), steps, warmup, stream, "attn_tile_d128")
+        o_buf = []
+
+        def attn_step():
+            o_buf[:] = [K.attention(q, k, v, True, sm)]
+
+        avg_ms, per, _ = _events_time(attn_step, steps, warmup, stream, "attn_tile_d128")
         fl = 4.0 * Z * H * S * S * D / 2  # lower triangle only
         tf = fl / (avg_ms * 1e-3) / 1e12
         extra["attn_fwd_causal_4x32x4096x128"] = {"kernel": rt.last_kernel_name(), "ms_avg": round(avg_ms, 4),
                                                   "ms_min": round(min(per), 4), "TFLOPs": round(tf, 2)}
         rooflines["attn_fwd_causal_4x32x4096x128"] = _roof("mfma", tf, PEAK_BF16_TFLOPS, "TFLOP/s", "attn_tile_d128")
-        del q, k, v
+        # spot parity on the last timed output: 64 random rows of two heads against float64 softmax attention
+        ok = True
+        for (z, h) in ((1, 7), (3, 31)):
+            rows = torch.randint(0, S, (64, ), device="cuda")
+            sc = (q[z, h, rows].double() @ k[z, h].double().T) * sm
+            sc = sc.masked_fill(rows[:, None] < torch.arange(S, device="cuda")[None, :], float("-inf"))
+            ref = torch.softmax(sc, -1) @ v[z, h].double()
+            ok &= bool((o_buf[0][z, h, rows].double() - ref).abs().max() <= 2e-2)
+        extra["attn_fwd_causal_4x32x4096x128"]["parity_rows_ok"] = ok
+        parity_failed |= not ok
+        del q, k, v, o_buf
         # the other instantiations of the same kernel, for the record (few launches each; not roofline lines)
         others = {}
         for (z, h, s_, d, causal) in ((4, 32, 4096, 128, False), (4, 32, 4064, 128, True), (4, 32, 4096, 64, True),
@@ -413,6 +451,9 @@ def main() -> int:
     extra["spinup_ms"] = SPINUP_MS
     extra["spinup_launches"] = dict(SPINUP_LAUNCHES)
     print(json.dumps(line))
+    if parity_failed:
+        print("bench.py: a timed output failed its parity spot check (see parity_rows_ok under 'extra')", file=sys.stderr)
+        return 1
     return 0
 
 

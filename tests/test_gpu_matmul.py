@@ -388,6 +388,45 @@ def test_ragged_fast_path_half_tile_tail(M, N, K_):
     assert torch.all(cbuf[M:] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
 
 
+def test_full_size_gelu_row_bias_4096x14336x4096():
+    """BASELINE's fused-epilogue shape, D = GELU(A.B + bias[N]) with M, N, K = 4096, 14336, 4096: 896 macro tiles on
+    256 CUs, i.e. three whole rounds and a tail that runs as half tiles, at 32 turns of the ring per tile.  Small
+    integers with an integer row bias are exact in fp32 whatever the order (the GELU of an integer >= 6 in magnitude
+    is the integer or 0 to bf16 precision, and in between the bar is the bf16 rounding of the exact value); random
+    operands on sampled rows and columns against float64 erf-GELU; a sentinel column block beside C."""
+    M, N, K_ = 4096, 14336, 4096
+    g = torch.Generator(device="cuda").manual_seed(21)
+    a = torch.randint(-2, 3, (M, K_), device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randint(-2, 3, (K_, N), device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randint(-3, 4, (N, ), device="cuda", generator=g).float()
+    c = K.matmul_fused(a, b, bias, epilogue="bias_row")
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi4"
+    want = a.float() @ b.float() + bias                      # |sums| < 2^24: exact in fp32 in any order
+    assert torch.equal(c, want.to(torch.bfloat16))
+    cg = K.matmul_fused(a, b, bias, epilogue="gelu")
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi2"
+    ref = torch.nn.functional.gelu(want.double())
+    assert bool(torch.all((cg.double() - ref).abs() <= RTOL * ref.abs() + ATOL))
+    del c, cg, want, ref
+    # random operands as BASELINE draws them, sampled rows and columns against float64
+    a = (torch.randn(M, K_, device="cuda", generator=g) / K_ ** 0.5).to(torch.bfloat16)
+    b = torch.randn(K_, N, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(N, device="cuda", generator=g) * 0.02
+    cbuf = torch.full((M, N + 8), 7.5, dtype=torch.bfloat16, device="cuda")
+    cg = cbuf[:, :N]
+    ad, bd, cd, biasd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, cg, bias.reshape(1, N)))
+    K.matmul_kernel_fused[((M // 128) * (N // 128), )](ad, bd, cd, biasd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False,
+                                                        EPILOGUE="gelu")
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi2"
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 2047, 2048, 3839, 3840, 3967, 3968, 4095, 1234], device="cuda")
+    ref = torch.nn.functional.gelu(a[rows].double() @ b.double() + bias.double())
+    assert bool(torch.all((cg[rows].double() - ref).abs() <= RTOL * ref.abs() + ATOL))
+    cols = torch.tensor([0, 7, 8, 255, 256, 14079, 14080, 14207, 14208, 14335, 9999], device="cuda")
+    ref = torch.nn.functional.gelu(a.double() @ b[:, cols].double() + bias[cols].double())
+    assert bool(torch.all((cg[:, cols].double() - ref).abs() <= RTOL * ref.abs() + ATOL))
+    assert torch.all(cbuf[:, N:] == 7.5)
+
+
 def test_full_size_8192_properties():
     """BASELINE's 8192^3: checked through size-independent properties -- B = I gives C = A
     bit for bit, linearity in A, and sampled rows against fp64 on the host."""

@@ -97,6 +97,27 @@ def test_tiled_matmul_random_shapes_exact_and_padding_untouched():
         assert torch.isnan(full[M:, :]).all() and torch.isnan(full[:, N:]).all(), (M, N, K_)
 
 
+@pytest.mark.parametrize("M,N,K_", [(70, 45, 50), (300, 333, 200), (256, 256, 1), (515, 260, 31), (64, 64, 161), (1000, 1000, 1000)])
+def test_tiled_matmul_ignores_what_the_padding_holds(M, N, K_):
+    """The source masks k >= K to zero and never stores rows >= M or columns >= N (03-matrix-multiplication.py:340-342,
+    359-361, 387-388), so the result must not depend on the padding of the tile-major buffers: here it is NaN in A
+    (rows past M, columns past K) and in B (rows past K, columns past N), and the result equals the zero-padded one
+    bit for bit and meets the bar against the oracle run on the same NaN-padded buffers."""
+    a, b = _rand((M, K_), 20), _rand((K_, N), 21)
+    Mp, Np, Kp = (K.cdiv(x, 32) * 32 for x in (M, N, K_))
+    an = torch.full((Mp, Kp), float("nan"), dtype=torch.float16); an[:M, :K_] = a
+    bn = torch.full((Kp, Np), float("nan"), dtype=torch.float16); bn[:K_, :N] = b
+    at, bt = K.tilize(an, 32, 32), K.tilize(bn, 32, 32)
+    for act in ("", "leaky_relu"):
+        ct = K.matmul_tiled(at.cuda(), bt.cuda(), M, N, K_, activation=act)
+        assert rt.last_kernel_name() == f"gemm_tiledragged_f16_epi{3 if act else 0}"
+        c0 = K.matmul_tiled(K.tilize(a, 32, 32).cuda(), K.tilize(b, 32, 32).cuda(), M, N, K_, activation=act)
+        got, got0 = (orc.untilize(_bits(t.cpu()), M, N, 32, 32) for t in (ct, c0))
+        assert np.array_equal(got, got0)
+        ref = orc.matmul_tiled(_bits(at), _bits(bt), M, N, K_, leaky_relu=bool(act), acc64=True)
+        assert _close(_f16(got), _f16(orc.untilize(ref, M, N, 32, 32)))
+
+
 def test_tiled_matmul_bf16_inputs_give_fp16():
     M, N, K_ = 64, 96, 128
     a, b = _rand((M, K_), 4, torch.bfloat16), _rand((K_, N), 5, torch.bfloat16)

@@ -259,6 +259,35 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                  : "memory", "m0");
   };
 
+  // TILED && RAGGED with K not a multiple of 32: the last tile of every K row of tiles holds columns (A) and rows
+  // (B) past K.  The source masks them to zero whatever the buffers hold there
+  // (03-matrix-multiplication.py:340-342, 359-361), so a thread clears, in the stage that received the last data
+  // step, the part of its OWN sixteen bytes of each slab that lies past K, once its copies have landed and before
+  // the barrier that opens the stage for reading.
+  const int k_tail = (TILED && RAGGED) ? g.K & 31 : 0;            // valid k of the last data step, 0 = all 32
+  auto clear_past_k = [&](uint8_t *stage) {
+    if constexpr (TILED && RAGGED) {
+      typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+      // A: this thread's chunk holds k = 8*a_chunk .. 8*a_chunk + 7 of one row, two per 32-bit word
+      const int ka = a_chunk * 8;
+      u32x4 keep;
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        keep[w] = (ka + 2 * w + 1 < k_tail) ? 0xffffffffu : (ka + 2 * w < k_tail) ? 0x0000ffffu : 0u;
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + i * 4096 + lds_wave + lane * 16);
+        *p = *p & keep;
+      }
+      // B: slab i holds k rows 8i .. 8i + 7, this thread's sixteen bytes lie in row 8i + b_k
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + A_BYTES + i * 4096 + lds_wave + lane * 16);
+        if (i * 8 + b_k >= k_tail) *p = (u32x4){0, 0, 0, 0};
+      }
+    }
+  };
+
   // The stream of steps this workgroup executes: tile after tile, nk steps each.
   // a_cur/b_cur point at the current tile's A rows / B columns, a_nxt/b_nxt at the next
   // tile's (or the current one again when there is none: a harmless refetch).
@@ -357,6 +386,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       // All of this wave's reads of stage I have returned, and so has its share of the
       // copy into stage I+1 (the 16 younger copies may still be in flight).  After the
       // barrier that holds for every wave: I+1 may be read, I may be overwritten.
+      if constexpr (TILED && RAGGED && !decltype(inner_)::value) {
+        if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
+          asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+          clear_past_k(nxt);
+        }
+      }
       asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       FENCE();
       // sub-step 1: MFMAs on f1; the next stage's sub-step 0 fragments; first half of the
@@ -384,6 +419,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         if (n & 1) dma_single(k - 1 + R, prv, MB + (n >> 1), inner_);
         mm(f0, n);
         FENCE();
+      }
+      if constexpr (TILED && RAGGED && !decltype(inner_)::value) {
+        if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
+          asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+          clear_past_k(nxt);
+        }
       }
       asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       FENCE();
@@ -417,6 +458,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     for (int i = 0; i < (s == R - 1 ? MB : MB + 4); ++i) dma_single(s, ring.s[s], i, std::false_type{});
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
   // everything issued but step 0's own MB + 4 copies may still be in flight: 2 * (MB + 4) + MB
+  if (TILED && RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    clear_past_k(ring.s[0]);
+  }
   if constexpr (MB == 4)
     asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
   else
