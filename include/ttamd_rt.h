@@ -106,7 +106,7 @@ TTAMD_API int rt_memset(void *dst, int value, size_t bytes, void *stream);
 
 /* Code objects.  rt_module_load takes a gfx950 code object image in memory
  * (device.load_library, backend/driver.py:72); rt_builtin_module returns one of
- * the images embedded in this library ("elementwise", "gemm", "attention"). */
+ * the images embedded in this library ("elementwise", "gemm", "attention", "reduce"). */
 TTAMD_API int rt_module_load(const void *image, size_t bytes, rt_module *out);
 TTAMD_API int rt_module_unload(rt_module m);
 TTAMD_API int rt_builtin_module(const char *which, rt_module *out);
@@ -240,8 +240,10 @@ TTAMD_API int tt_copy_kernel(const void *x, void *out, int32_t n_elements, int32
  * on NaN input return an index that depends on the fold order, as the reference's do.
  * Every program of the grid would store the same value; it is computed once.  Blocks of 128 KiB and more
  * (16-byte aligned) are folded by several workgroups through a small device buffer that the library keeps
- * per (device, stream): the first such call on a stream allocates it (never while the stream is recording a
- * graph: one workgroup then does the work), and calls on different streams do not share it. */
+ * per (device, stream): the first such call on a stream allocates it (hipMalloc, 4352 bytes), calls on
+ * different streams do not share it, and rt_release_stream frees it.  A call on a stream that is recording a
+ * graph never uses that buffer, whether it exists or not: it runs as one workgroup, so a recorded graph holds
+ * no address of the library's and may be replayed on any stream beside eager calls. */
 typedef enum tt_reduce_op {
   TT_REDUCE_SUM = 0, TT_REDUCE_MIN = 1, TT_REDUCE_MAX = 2, TT_REDUCE_ARGMIN = 3, TT_REDUCE_ARGMAX = 4,
   TT_REDUCE_XOR_SUM = 5
@@ -249,6 +251,21 @@ typedef enum tt_reduce_op {
 TTAMD_API int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
                        int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
                        const uint32_t grid[3], void *stream);
+/* Frees what the library allocated for `stream` on the current device (the buffer above), after waiting for the
+ * stream; call it before destroying a stream that ran large reductions.  No counterpart in the reference. */
+TTAMD_API int rt_release_stream(void *stream);
+/* The same reductions, same arguments and results, for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  It calls no hipMalloc / hipFree at any time: the partial results of a block folded by several
+ * workgroups live in a 4352-byte device array that is part of the library's own image (one copy on every GPU the
+ * library runs on, for the life of the process), and its kernels are resolved by rt_init.  BLOCK beyond 1048576
+ * elements is refused (RT_ERR_INVALID).  Every call on a GPU shares that GPU's array: calls that may run at the
+ * same time on one GPU (two streams, or two graphs replayed side by side) race and must be ordered by the
+ * caller; calls on one stream, eager or replayed, are ordered already.  Recorded into a graph it keeps the
+ * several-workgroup form (tt_reduce1d_kernel records one workgroup). */
+TTAMD_API int tt_reduce1d_kernel_noalloc(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
+                               int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
+                               const uint32_t grid[3], void *stream);
 
 /* matmul_kernel_tma(a_desc, b_desc, c_desc, M, N, K, BLOCK_SIZE_M, BLOCK_SIZE_N,
  *                   BLOCK_SIZE_K, GROUP_SIZE_M, FP8_OUTPUT, WARP_SPECIALIZE)

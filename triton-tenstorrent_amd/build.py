@@ -22,7 +22,8 @@ LIB = PKG / "lib" / "libttamd_rt.so"
 ARCH = "gfx950"
 
 CODE_OBJECTS = ["elementwise", "gemm", "attention", "reduce"]
-RT_SOURCES = ["ttamd_rt.cpp", "tt_elementwise.cpp", "tt_gemm.cpp", "tt_attention.cpp", "tt_reduce.cpp"]
+RT_SOURCES = ["ttamd_rt.cpp", "tt_elementwise.cpp", "tt_gemm.cpp", "tt_attention.cpp", "tt_reduce.cpp",
+              "tt_reduce_static.hip"]
 
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 on this target
 DEVICE_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -55,7 +56,9 @@ def build_code_object(name: str, extra: list[str] | None = None) -> Path:
 
 def build_runtime() -> Path:
     LIB.parent.mkdir(exist_ok=True)
-    cmd = [hipcc(), "-shared", "-fPIC", "-O2", "-std=c++17", "-fvisibility=hidden", "-Wall",
+    # tt_reduce_static.hip carries a __device__ array, so the library holds a small gfx950 image of its own
+    cmd = [hipcc(), "-shared", "-fPIC", "-O2", "-std=c++17", "-fvisibility=hidden", "-Wall", f"--offload-arch={ARCH}",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
            f"-I{ROOT / 'include'}", f"-I{CSRC / 'rt'}", f'-DTTAMD_CO_DIR="{BUILD}"',
            *[str(CSRC / "rt" / s) for s in RT_SOURCES], "-o", str(LIB)]
     _run(cmd)

@@ -189,7 +189,8 @@ __device__ __forceinline__ void reduce_body(const T *__restrict__ x, void *__res
       slots[b].v = p.v;
       slots[b].i = p.i;
       __threadfence();                                   // the partial is visible before the ticket is taken
-      last = atomicAdd(counter, 1u) == (unsigned)(G - 1);
+      // the counter wraps to zero by itself with the G-th ticket, so it is ready for the next launch that uses it
+      last = atomicInc(counter, (unsigned)(G - 1)) == (unsigned)(G - 1);
     }
     __syncthreads();
     if (!last) return;
@@ -203,10 +204,8 @@ __device__ __forceinline__ void reduce_body(const T *__restrict__ x, void *__res
     for (int m = 32; m >= 1; m >>= 1) p = fold<op>(nan_mode != 0, p, shuffle_xor(p, m));
     if ((tid & 63) == 0) part[tid >> 6] = p;
     __syncthreads();
-    if (tid == 0) {
+    if (tid == 0)
       for (int w = 1; w < kLanes / 64; ++w) p = fold<op>(nan_mode != 0, p, part[w]);
-      *counter = 0;                                      // ready for the next launch on this stream
-    }
   }
   if (tid == 0) {
     if (op == ARGMIN || op == ARGMAX) {
@@ -233,6 +232,12 @@ __device__ __forceinline__ void reduce_body(const T *__restrict__ x, void *__res
     default: reduce_body<T, XOR>((const T *)x, z, n, nan_mode, out_bytes, out_kind, scratch, counter); break; \
     }                                                                                                                 \
   }
+
+// Puts the arrival counter of a buffer of partial results back to zero (a kernel rather than a memset, so that it
+// can be recorded into a graph).
+extern "C" __global__ __launch_bounds__(64) void reduce1d_clear_counter(unsigned *counter) {
+  if (threadIdx.x == 0) *counter = 0u;
+}
 
 REDUCE_KERNEL(reduce1d_i8, int8_t)
 REDUCE_KERNEL(reduce1d_i16, int16_t)

@@ -27,6 +27,15 @@ inline size_t dtype_size(int dt) {
   default: return 0;
   }
 }
+// The buffer of partial results of a reduction shared between workgroups: 256 slots of 16 bytes, then the arrival
+// counter.
+constexpr int kReduceMaxGroups = 256;
+constexpr size_t kReduceCounterAt = kReduceMaxGroups * 16, kReduceScratchBytes = kReduceCounterAt + 256;
+int reduce1d_launch(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype, int32_t acc_dtype,
+                    int32_t out_dtype, int32_t propagate_nan, const uint32_t grid[3], void *stream,
+                    void *fixed_scratch);
+// Resolves the address of the static scratch array on the current device; called by rt_init.
+int static_scratch_setup(int device);
 // Integer environment knob read once per name (tuning sweeps only).
 int env_int(const char *name, int dflt);
 

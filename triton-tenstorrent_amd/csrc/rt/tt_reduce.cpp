@@ -13,29 +13,32 @@ using namespace ttamd;
 namespace {
 // A large block is reduced by several workgroups that leave partial results in a small device buffer (256 slots
 // of 16 bytes and an arrival counter).  Launches on one stream run in order and share one buffer; every
-// (device, stream) pair gets its own, allocated on first use and kept until the process ends.
-constexpr int kMaxGroups = 256;
-constexpr size_t kSlotBytes = 16, kCounterAt = kMaxGroups * kSlotBytes;
+// (device, stream) pair gets its own, allocated on first use and kept until rt_release_stream or the end of the
+// process.  A launch that is being recorded into a graph never takes this path (the graph could be replayed on
+// any stream, beside eager launches on the one it was recorded on, and the buffer's address would be baked in):
+// it runs as one workgroup, which needs no buffer.
+using ttamd::kReduceMaxGroups;
+using ttamd::kReduceCounterAt;
+std::mutex g_mu;
+std::map<std::pair<int, void *>, void *> g_bufs;
 void *partials_for(void *stream) {
-  static std::mutex mu;
-  static std::map<std::pair<int, void *>, void *> bufs;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  std::lock_guard<std::mutex> lk(mu);
-  auto it = bufs.find({dev, stream});
-  if (it != bufs.end()) return it->second;
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing((hipStream_t)stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
     (void)hipGetLastError();
-    return nullptr;   // no allocation while the stream records a graph: the caller takes one workgroup
+    return nullptr;
   }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lk(g_mu);
+  auto it = g_bufs.find({dev, stream});
+  if (it != g_bufs.end()) return it->second;
   void *p = nullptr;
-  if (hipMalloc(&p, kCounterAt + 256) != hipSuccess) return nullptr;
-  if (hipMemset(p, 0, kCounterAt + 256) != hipSuccess) {
+  if (hipMalloc(&p, ttamd::kReduceScratchBytes) != hipSuccess) return nullptr;
+  if (hipMemset(p, 0, ttamd::kReduceScratchBytes) != hipSuccess) {
     (void)hipFree(p);
     return nullptr;
   }
-  bufs[{dev, stream}] = p;
+  g_bufs[{dev, stream}] = p;
   return p;
 }
 
@@ -59,9 +62,11 @@ bool type_info(int dt, TypeInfo *t) {
 }
 } // namespace
 
-extern "C" int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
-                                  int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
-                                  const uint32_t grid[3], void *stream) {
+// Validation and launch shared by the two entry points.  `fixed_scratch`: null = the per-stream buffer (allocated on
+// first use, never while recording); otherwise the buffer to use, whose counter is put back to zero first.
+int ttamd::reduce1d_launch(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype, int32_t acc_dtype,
+                           int32_t out_dtype, int32_t propagate_nan, const uint32_t grid[3], void *stream,
+                           void *fixed_scratch) {
   if (!props()) return fail(RT_ERR_NOT_INIT, "reduce1d: call rt_init first");
   if (!grid) return fail(RT_ERR_INVALID, "reduce1d: null grid");
   if (!x || !z) return fail(RT_ERR_INVALID, "reduce1d: null pointer");
@@ -102,12 +107,42 @@ extern "C" int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BL
   uint32_t groups = 1;
   void *scratch = nullptr, *counter = nullptr;
   if (bytes >= (128 << 10) && aligned16(x) && !env_int("TTAMD_REDUCE_ONE_GROUP", 0)) {
-    scratch = partials_for(stream);
+    scratch = fixed_scratch ? fixed_scratch : partials_for(stream);
     if (scratch) {
-      groups = (uint32_t)std::min<int64_t>(kMaxGroups, bytes >> 14);
-      counter = (char *)scratch + kCounterAt;
+      groups = (uint32_t)std::min<int64_t>(kReduceMaxGroups, bytes >> 14);
+      counter = (char *)scratch + kReduceCounterAt;
     }
+  }
+  if (fixed_scratch && groups > 1) {
+    // the buffer outlives the call and is shared by every call on this device: start from a counter of zero
+    void *cargs[] = {&counter};
+    int rc = launch("reduce", "reduce1d_clear_counter", dim3(1), dim3(64), 0, stream, cargs, 1);
+    if (rc) return rc;
   }
   void *args[] = {(void *)&x, (void *)&z, &n, &op_, &nan_, &ob, &out_kind, &scratch, &counter};
   return launch("reduce", in.kernel, dim3(groups), dim3(1024), 0, stream, args, 9);
+}
+
+extern "C" int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
+                                  int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
+                                  const uint32_t grid[3], void *stream) {
+  return ttamd::reduce1d_launch(op, x, z, BLOCK, in_dtype, acc_dtype, out_dtype, propagate_nan, grid, stream, nullptr);
+}
+
+extern "C" int rt_release_stream(void *stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(RT_ERR_HIP, "rt_release_stream: no current device");
+  void *p = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_bufs.find({dev, stream});
+    if (it == g_bufs.end()) return RT_OK;
+    p = it->second;
+    g_bufs.erase(it);
+  }
+  hipError_t e = hipStreamSynchronize((hipStream_t)stream);
+  if (e != hipSuccess) return hip_fail(e, "rt_release_stream: hipStreamSynchronize");
+  e = hipFree(p);
+  if (e != hipSuccess) return hip_fail(e, "rt_release_stream: hipFree");
+  return RT_OK;
 }

@@ -171,6 +171,24 @@ int rt_init(int device) {
     m->builtin = true;
     s.builtin[im.name] = m;
   }
+  // every kernel the reductions can launch is resolved now, so that a later call, which may sit inside a graph
+  // capture, neither loads code nor allocates
+  static const char *const reduce_kernels[] = {"reduce1d_i8", "reduce1d_i16", "reduce1d_i32", "reduce1d_i64",
+                                               "reduce1d_u8", "reduce1d_u16", "reduce1d_u32", "reduce1d_u64",
+                                               "reduce1d_f32", "reduce1d_bf16", "reduce1d_f16", "reduce1d_f64",
+                                               "reduce1d_clear_counter"};
+  for (const char *name : reduce_kernels) {
+    rt_module_s *m = s.builtin["reduce"];
+    hipFunction_t fn = nullptr;
+    hipError_t e = hipModuleGetFunction(&fn, m->mod, name);
+    if (e != hipSuccess) return ttamd::hip_fail(e, (std::string("hipModuleGetFunction(") + name + ")").c_str());
+    auto *k = new rt_kernel_s();
+    k->fn = fn;
+    k->name = name;
+    m->kernels[name] = k;
+  }
+  int rc = ttamd::static_scratch_setup(device);
+  if (rc) return rc;
   s.device = device;
   s.inited = true;
   return RT_OK;

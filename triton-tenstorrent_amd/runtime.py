@@ -96,6 +96,8 @@ SYMBOLS = {
     "tt_cast_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_copy_kernel": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _G, _vp]),
     "tt_reduce1d_kernel": (C.c_int, [_i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
+    "tt_reduce1d_kernel_noalloc": (C.c_int, [_i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
+    "rt_release_stream": (C.c_int, [_vp]),
     "tt_matmul_kernel_tma": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_fused": (C.c_int, [_DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_matmul_kernel_tma_fp8_scaled": (C.c_int, [_DP, _DP, _DP, _i32, _i32, _i32, _f32, _f32, _i32, _i32, _i32, _i32, _G, _vp]),
