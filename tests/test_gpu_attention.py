@@ -211,3 +211,37 @@ def test_p_is_rounded_to_bf16_and_l_is_summed_before_the_cast(causal, S, D, kern
     bm = 32 if S % 64 else 64
     ro, rM = orc.attn_fwd(q, k, v, sm, causal=causal, BLOCK_M=bm, BLOCK_N=min(bm, D))
     assert np.all(np.abs(o - orc.from_bf16(ro)[0, 0]) <= 2.0 ** -8 * np.abs(wo) + O_ATOL) and np.max(np.abs(M - rM[0, 0])) <= M_ATOL
+
+
+@pytest.mark.parametrize("S,D,kernel", [(256, 128, "attn_tile_d128"), (512, 128, "attn_tile_d128"), (224, 128, "attn_ragged_d128"),
+                                        (256, 64, "attn_tile_d64"), (128, 256, "attn_tile_d256"), (128, 16, "attn_any_d16")])
+def test_causal_mask_is_the_sources_at_block_m_32(S, D, kernel):
+    """The source masks with an ADDITIVE -1.0e6 inside the diagonal block (06-fused-attention.py:58-59), so a masked
+    score more than 1e6 above the unmasked ones leaks.  The kernels evaluate the mask as the source does at
+    BLOCK_M = 32, whatever BLOCK_M the launch names: row 40 against key 41 (same 32x32 tile, 2^21 * log2e above the
+    rest) leaks exactly as in the oracle; row 70 against key 100 (a later tile) does not, where the source at
+    BLOCK_M = 128 would leak too.  Both stated in the kernels' headers."""
+    from triton_tenstorrent_amd import runtime as rt
+    g = torch.Generator().manual_seed(S + D)
+    q = torch.zeros(1, 1, S, D)
+    k = torch.zeros(1, 1, S, D)
+    q[0, 0, 40, 0], k[0, 0, 41, 0] = 2048.0, 1024.0
+    q[0, 0, 70, 1], k[0, 0, 100, 1] = 2048.0, 1024.0
+    v = torch.randn(1, 1, S, D, generator=g)
+    q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
+    wo, wM = orc.attn_fwd(bits(q), bits(k), bits(v), 1.0, causal=True, BLOCK_M=32, BLOCK_N=min(32, D))
+    wo = orc.from_bf16(wo)
+    assert np.array_equal(wo[0, 0, 40], decode(v)[0, 0, 41])                       # the oracle leaks inside the tile
+    for bm in (32, 64, 128):
+        if S % bm:
+            continue
+        o, M = K.attention(q.cuda(), k.cuda(), v.cuda(), True, 1.0, return_lse=True, BLOCK_M=bm, BLOCK_N=min(32, D))
+        assert rt.last_kernel_name() == kernel
+        assert np.max(np.abs(decode(o) - wo)) <= O_ATOL and np.max(np.abs(M.cpu().numpy() - wM)) <= M_ATOL * max(1.0, 2.0 ** 21 * 2 ** -20)
+        assert torch.equal(o[0, 0, 40].cpu(), v[0, 0, 41])                         # row 40 copies the masked key's value
+        mean70 = v[0, 0, :71].double().mean(0)
+        assert (o[0, 0, 70].cpu().double() - mean70).abs().max() <= O_ATOL          # row 70 does not see key 100
+    if S % 128 == 0:
+        # the stated difference: at BLOCK_M = 128 the source itself would leak row 70 to key 100
+        o128, _ = orc.attn_fwd(bits(q), bits(k), bits(v), 1.0, causal=True, BLOCK_M=128, BLOCK_N=min(32, D))
+        assert np.array_equal(orc.from_bf16(o128)[0, 0, 70], decode(v)[0, 0, 100])

@@ -71,9 +71,8 @@ def test_matmul_and_attention_in_a_graph():
 
 def test_large_reduction_in_a_graph():
     """A reduction of 128 KiB and more runs on several workgroups through a per-stream buffer that the first
-    call on a stream allocates.  Recorded on a stream that has no buffer yet it must not allocate (one workgroup
-    runs); recorded on a stream that has one, the multi-workgroup kernel goes into the graph and its arrival
-    counter is back at zero after every replay."""
+    eager call on a stream allocates.  Recorded into a graph it takes the one-workgroup form, whether the stream
+    has such a buffer or not, so the graph holds no address of the library's."""
     n = 1 << 20
     x = torch.randint(-2**31, 2**31 - 1, (n, ), device="cuda", dtype=torch.int64).to(torch.int32)
     z = torch.zeros(1, device="cuda", dtype=torch.int32)
@@ -111,3 +110,35 @@ def test_large_reduction_in_a_graph():
         work()                                           # and eagerly, between the replays
         torch.cuda.synchronize()
         assert int(z.item()) & 0xffffffff == want_sum and int(za.item()) == want_arg
+
+
+def test_graph_with_a_large_reduction_replayed_on_another_stream_beside_eager_calls():
+    """A graph recorded on stream A (which owns a buffer of partial results from earlier eager calls) is replayed on
+    stream B while eager several-workgroup reductions of other data run on A: the graph shares nothing with them,
+    so both give their own right answers every time.  Bounded: 100 rounds, stops at the first mismatch."""
+    n = 1 << 20
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randint(-2**31, 2**31 - 1, (n, ), device="cuda", dtype=torch.int64, generator=g).to(torch.int32)
+    y = torch.randint(-2**31, 2**31 - 1, (n, ), device="cuda", dtype=torch.int64, generator=g).to(torch.int32)
+    zx = torch.zeros(1, device="cuda", dtype=torch.int32)
+    zy = torch.zeros(1, device="cuda", dtype=torch.int32)
+    want_x = int(x.sum(dtype=torch.int64).item()) & 0xffffffff
+    want_y = int(y.sum(dtype=torch.int64).item()) & 0xffffffff
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(a):
+        K.reduce1d_kernel[(1, )](x, zx, BLOCK=n, OP="sum")     # a now owns a buffer
+    torch.cuda.synchronize()
+    gr = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gr, stream=a):
+        K.reduce1d_kernel[(1, )](x, zx, BLOCK=n, OP="sum")
+    for rep in range(100):
+        zx.fill_(-7)
+        zy.fill_(-7)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(b):
+            gr.replay()
+        with torch.cuda.stream(a):
+            for _ in range(4):
+                K.reduce1d_kernel[(1, )](y, zy, BLOCK=n, OP="sum")
+        torch.cuda.synchronize()
+        assert int(zx.item()) & 0xffffffff == want_x and int(zy.item()) & 0xffffffff == want_y, rep

@@ -12,7 +12,11 @@
 //
 // Numerics follow the kernel source: qk_scale = sm_scale*1.44269504, exp2-based
 // softmax, l_ij summed in fp32 before P is rounded to bf16, additive -1.0e6 on
-// masked entries of the diagonal block, M = m_i + log2(l_i).
+// masked entries of the diagonal block, M = m_i + log2(l_i).  The causal mask is
+// evaluated as the source does at BLOCK_M = 32, whatever BLOCK_M the launch names:
+// -1.0e6 inside the 32x32 tile on the diagonal, keys past it not visited.  At a
+// larger BLOCK_M the source adds -1.0e6 to those keys as well, which differs only
+// where a masked score exceeds the unmasked ones by more than 1e6.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -393,7 +397,9 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = n0 + kt * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-          st[kt][r] = st[kt][r] * qk_scale + (my_q >= key ? 0.0f : -1.0e6f);
+          // additive -1.0e6 inside this wavefront's 32x32 tile on the diagonal, as the source does at BLOCK_M = 32;
+          // the block's keys past that tile are not part of the product at all
+          st[kt][r] = st[kt][r] * qk_scale + (my_q >= key ? 0.0f : (key > qw + 31 ? -__builtin_inff() : -1.0e6f));
           rmax = fmaxf(rmax, st[kt][r]);
         }
       rmax = xor32_max(rmax);
@@ -500,7 +506,7 @@ extern "C" {
   }
 ATTN_TILE(32)
 ATTN_TILE(64)
-ATTN_TILE(128)
+// head dim 128 on whole 256-query blocks: attention_pipe.h
 
 #define ATTN_RAGGED(D)                                                                     \
   __global__ __launch_bounds__(512) void attn_ragged_d##D(AttnArgs a) {                    \
@@ -523,3 +529,5 @@ ATTN_TILE4(attn_tile_d256, 256, false)
 ATTN_TILE4(attn_ragged_d256, 256, true)
 
 } // extern "C"
+
+#include "attention_pipe.h"

@@ -70,7 +70,9 @@ extern "C" int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const
       !env_int("TTAMD_ATTN_FORCE_ANY", 0)) {
     void *fargs[] = {&a};
     const int queries = HEAD_DIM == 256 ? 128 : 256;   // per workgroup: 4 or 8 wavefronts of 32
-    const uint32_t wgs = (uint32_t)(cdiv64(N_CTX, queries) * (int64_t)Z * H);
+    uint32_t wgs = (uint32_t)(cdiv64(N_CTX, queries) * (int64_t)Z * H);
+    // head dim 128 on whole blocks: one workgroup takes the query blocks i and n-1-i of a head
+    if (HEAD_DIM == 128 && N_CTX % queries == 0) wgs = (uint32_t)(cdiv64(N_CTX / queries, 2) * (int64_t)Z * H);
     char name[32];
     snprintf(name, sizeof(name), "attn_%s_d%d", N_CTX % queries == 0 ? "tile" : "ragged", HEAD_DIM);
     return launch("attention", name, dim3(wgs), dim3(2 * queries), 0, stream, fargs, 1);
