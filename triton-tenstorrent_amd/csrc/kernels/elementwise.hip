@@ -9,18 +9,25 @@
 // elements, lanes at or past n are masked.  The host folds grid and BLOCK into
 // one bound n_eff = min(n, grid*BLOCK); the kernels touch exactly [0, n_eff).
 //
-// HBM-bound: 16-byte non-temporal loads and stores per lane, UNROLL independent
-// vectors in flight per lane.  Each workgroup streams one contiguous run of
-// 256*UNROLL vectors and exits (measured on MI355X: 6.4-6.5 TB/s for the
-// 2-read/1-write add, against 4.5-5.3 TB/s for grid-stride loops over a
-// CU-count-sized grid at any unroll, and 5.6 TB/s for one contiguous chunk per
-// persistent workgroup).
+// HBM-bound: 16-byte non-temporal loads and stores, ONE vector per lane and operand, ONE
+// wavefront per workgroup: a workgroup streams 1 KiB of each operand and exits, and the
+// hardware dispatcher, which hands out workgroups in order, keeps the whole chip walking
+// the arrays front to back.  Measured on MI355X, int32 add at N = 2^28 (GB/s): this shape
+// 6720; 128 lanes x 1 vector 6670; 1024 x 1 6540; 256 x 1 6460; 256 x 4 (four vectors in
+// flight per lane) 6360; 256 x 8 5980; 256 x 2 6010; 192 or 320 lanes (not a power of two)
+// 6100-6240; plain cached loads and stores 6110; grid-stride loops over a CU-count-sized
+// grid 4500-6100.  Writes are what bounds it: a write-only kernel reaches 5940 at 256 x 4
+// and 6750 at one vector per lane, a read-only one 7100-7170 at either.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "elementwise_geom.h"
+
 namespace {
 
-constexpr int kThreads = 256;
+using ewgeom::kThreads;
+using ewgeom::kVec;
+using ewgeom::kVecHeavy;
 
 template <typename T> struct Vec4 { typedef T type __attribute__((ext_vector_type(4))); };
 
@@ -371,11 +378,11 @@ extern "C" {
 // 16-byte aligned operands
 __global__ __launch_bounds__(kThreads) void ew_add_f32(const float *x, const float *y, float *out,
                                                        uint32_t n) {
-  binary_body<float, AddOp, 4>(x, y, out, n);
+  binary_body<float, AddOp, kVec>(x, y, out, n);
 }
 __global__ __launch_bounds__(kThreads) void ew_add_i32(const int *x, const int *y, int *out,
                                                        uint32_t n) {
-  binary_body<int, AddWrapOp, 4>(x, y, out, n);
+  binary_body<int, AddWrapOp, kVec>(x, y, out, n);
 }
 // any alignment (4-byte)
 __global__ __launch_bounds__(kThreads) void ew_add_f32_unaligned(const float *x, const float *y,
@@ -387,30 +394,30 @@ __global__ __launch_bounds__(kThreads) void ew_add_i32_unaligned(const int *x, c
   binary_scalar_body<int, AddWrapOp>(x, y, out, n);
 }
 
-#define EW_UNARY(name, Op)                                                                              \
+#define EW_UNARY(name, Op, VEC)                                                                             \
   __global__ __launch_bounds__(kThreads) void ew_##name##_f32(const float *x, float *out, uint32_t n) { \
-    unary_body<Op, 4>(x, out, n);                                                                        \
+    unary_body<Op, VEC>(x, out, n);                                                                         \
   }                                                                                                      \
   __global__ __launch_bounds__(kThreads) void ew_##name##_f32_unaligned(const float *x, float *out,     \
                                                                         uint32_t n) {                    \
     unary_scalar_body<Op>(x, out, n);                                                                    \
   }
-EW_UNARY(sin, SinOp)
-EW_UNARY(cos, CosOp)
-EW_UNARY(abs, AbsOp)
-EW_UNARY(ceil, CeilOp)
-EW_UNARY(floor, FloorOp)
-EW_UNARY(exp, ExpOp)
-EW_UNARY(exp2, Exp2Op)
-EW_UNARY(log, LogOp)
-EW_UNARY(log2, Log2Op)
-EW_UNARY(rsqrt, RsqrtOp)
-EW_UNARY(sqrt, SqrtOp)
+EW_UNARY(sin, SinOp, kVecHeavy)
+EW_UNARY(cos, CosOp, kVecHeavy)
+EW_UNARY(abs, AbsOp, kVec)
+EW_UNARY(ceil, CeilOp, kVec)
+EW_UNARY(floor, FloorOp, kVec)
+EW_UNARY(exp, ExpOp, kVec)
+EW_UNARY(exp2, Exp2Op, kVec)
+EW_UNARY(log, LogOp, kVec)
+EW_UNARY(log2, Log2Op, kVec)
+EW_UNARY(rsqrt, RsqrtOp, kVec)
+EW_UNARY(sqrt, SqrtOp, kVec)
 
 #define EW_BINARY(name, Op)                                                                               \
   __global__ __launch_bounds__(kThreads) void ew_##name##_f32(const float *x, const float *y, float *out, \
                                                               uint32_t n) {                                \
-    binary_body<float, Op, 4>(x, y, out, n);                                                               \
+    binary_body<float, Op, kVec>(x, y, out, n);                                                               \
   }                                                                                                        \
   __global__ __launch_bounds__(kThreads) void ew_##name##_f32_unaligned(const float *x, const float *y,   \
                                                                         float *out, uint32_t n) {          \
@@ -420,7 +427,7 @@ EW_UNARY(sqrt, SqrtOp)
 #define EW_BINARY_CONST(name, Op)                                                                              \
   __global__ __launch_bounds__(kThreads) void ew_##name##c_f32(const float *x, float c, int flip, float *out,  \
                                                                uint32_t n) {                                   \
-    binary_const_body<Op, 4>(x, c, flip, out, n);                                                              \
+    binary_const_body<Op, kVec>(x, c, flip, out, n);                                                              \
   }                                                                                                            \
   __global__ __launch_bounds__(kThreads) void ew_##name##c_f32_unaligned(const float *x, float c, int flip,    \
                                                                          float *out, uint32_t n) {             \
@@ -441,7 +448,7 @@ EW_BINARY(min, MinOp)
 
 #define EW_CAST(name, Op, IN, OUT)                                                                          \
   __global__ __launch_bounds__(kThreads) void name(const IN *x, OUT *out, uint32_t n) {                     \
-    cast_vec_body<Op, 4>(x, out, n);                                                                        \
+    cast_vec_body<Op, kVec>(x, out, n);                                                                        \
   }                                                                                                         \
   __global__ __launch_bounds__(kThreads) void name##_unaligned(const IN *x, OUT *out, uint32_t n) {         \
     cast_body<Op>(x, out, n);                                                                               \
@@ -463,9 +470,9 @@ __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restric
     const V *yv = reinterpret_cast<const V *>(y);
     const V *zv = reinterpret_cast<const V *>(z);
     V *ov = reinterpret_cast<V *>(out);
-    const uint32_t base = blockIdx.x * (kThreads * 4);
+    const uint32_t base = blockIdx.x * (kThreads * kVec);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < kVec; ++u) {
       const uint32_t i = base + threadIdx.x + u * kThreads;
       if (i < nvec) {
         V a = __builtin_nontemporal_load(xv + i), b = __builtin_nontemporal_load(yv + i),
@@ -477,7 +484,7 @@ __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restric
         __builtin_nontemporal_store(r, ov + i);
       }
     }
-    if (nvec >= base && nvec < base + kThreads * 4) { // the last workgroup also takes the n % 4 tail
+    if (nvec >= base && nvec < base + kThreads * kVec) { // the last workgroup also takes the n % 4 tail
       const uint32_t t = (nvec << 2) + threadIdx.x;
       if (t < n) out[t] = MulAdd::apply(x[t], y[t], z[t]);
     }
@@ -489,7 +496,7 @@ __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restric
 }
 
 __global__ __launch_bounds__(kThreads) void ew_copy_b128(const uint8_t *x, uint8_t *out, uint64_t nbytes) {
-  copy_vec_body<4>(x, out, nbytes);
+  copy_vec_body<kVec>(x, out, nbytes);
 }
 #define EW_COPY_UNALIGNED(name, T)                                                     \
   __global__ __launch_bounds__(kThreads) void name(const T *x, T *out, uint32_t n) {   \

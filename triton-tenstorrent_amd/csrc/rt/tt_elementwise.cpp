@@ -8,6 +8,7 @@
 #include <string>
 
 #include "tt_internal.h"
+#include "../kernels/elementwise_geom.h"
 
 namespace ttamd {
 
@@ -25,8 +26,8 @@ int env_int(const char *name, int dflt) {
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
+using ewgeom::kThreads;
+constexpr int kUnroll = ewgeom::kVec;
 
 // Elements the logical grid covers: programs 0..grid-1 own `per_program`
 // consecutive elements each, clipped by the n_elements mask.
@@ -45,15 +46,15 @@ int check_1d(const char *who, int32_t n, int64_t per_program, const uint32_t gri
 
 // One workgroup per run of kThreads*kUnroll vectors (plus one for a ragged end / scalar
 // tail); the unaligned kernels use a grid-stride loop over a grid sized to the CU count.
-uint32_t streaming_grid(uint32_t n_eff, bool aligned) {
+uint32_t streaming_grid(uint32_t n_eff, bool aligned, int vec_per_lane = kUnroll) {
   if (aligned) {
-    const uint32_t nvec = n_eff >> 2, per_wg = kThreads * kUnroll;
+    const uint32_t nvec = n_eff >> 2, per_wg = kThreads * vec_per_lane;
     uint32_t wgs = nvec / per_wg;
     if (wgs * per_wg < nvec || (n_eff & 3u) || wgs == 0) ++wgs; // ragged end or scalar tail
     return wgs;
   }
   const rt_props *p = props();
-  int64_t cap = (int64_t)p->multiprocessor_count * env_int("TTAMD_EW_WG_PER_CU", 8);
+  int64_t cap = (int64_t)p->multiprocessor_count * env_int("TTAMD_EW_WG_PER_CU", 32);
   return (uint32_t)std::max<int64_t>(1, std::min(cap, cdiv64((int64_t)n_eff, kThreads)));
 }
 
@@ -121,7 +122,7 @@ int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SI
   bool al = aligned16(x) && aligned16(out);
   void *args[] = {&x, &out, &n_eff};
   return launch("elementwise", al ? "ew_sin_f32" : "ew_sin_f32_unaligned",
-                dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 3);
+                dim3(streaming_grid(n_eff, al, ewgeom::kVecHeavy)), dim3(kThreads), 0, stream, args, 3);
 }
 
 int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
@@ -139,7 +140,9 @@ int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_elements, in
   char name[48];
   snprintf(name, sizeof(name), "ew_%s_f32%s", names[op], al ? "" : "_unaligned");
   void *args[] = {&x, &out, &n_eff};
-  return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 3);
+  const bool heavy = op == TT_OP_SIN || op == TT_OP_COS;
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al, heavy ? ewgeom::kVecHeavy : kUnroll)), dim3(kThreads), 0,
+                stream, args, 3);
 }
 
 int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_t n_elements,
