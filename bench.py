@@ -94,7 +94,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--spinup-ms", type=float, default=30.0,
                     help="untimed run of each kernel before its warm-up steps, so that the clock has left its idle state")
-    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,ops,fused,fp8,tiled,attn,add0")
+    ap.add_argument("--only", type=str, default="", help="comma list of: gemm,add,sin,ops,ew_ceiling,fused,fp8,tiled,attn,add0")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -220,6 +220,36 @@ def main() -> int:
         ops["copy"] = round(2 * 4 * n_el / (avg_ms * 1e-3) / 1e9, 1)
         extra["elementwise_ops_2p28_GBs"] = ops
         del xs, ys, outs
+    if "ew_ceiling" in only or not only:
+        # what the streaming geometry reaches when it only reads, only writes, or copies: the bounds the 2-read/1-write
+        # add and the 1-read/1-write sin sit under (the kernels are diagnostics inside the elementwise code object)
+        import ctypes as C
+        lib = rt.init(0)
+        mod = C.c_void_p()
+        rt.check(lib.rt_builtin_module(b"elementwise", C.byref(mod)))
+        xs = torch.randint(-2**20, 2**20, (n_el, ), dtype=torch.int32, device="cuda")
+        outs = torch.empty_like(xs)
+        nvec = n_el // 4
+        ceil = {}
+        for kname, per_wg in (("ew_ceiling_read_b128", 1024), ("ew_ceiling_write_b128", 256)):
+            nbytes = 4 * n_el
+            kh = C.c_void_p()
+            rt.check(lib.rt_get_kernel(mod, kname.encode(), C.byref(kh)))
+            vals = [C.c_void_p(xs.data_ptr()), C.c_void_p(outs.data_ptr()), C.c_uint32(nvec)]
+            kargs = (C.c_void_p * 3)(*[C.cast(C.pointer(v), C.c_void_p) for v in vals])
+            g3, b3 = rt.grid3(nvec // per_wg), rt.grid3(256)
+            avg_ms, per, _ = _events_time(lambda: rt.check(lib.rt_launch(kh, g3, b3, 0, C.c_void_p(stream), kargs, 3)),
+                                          max(3, steps // 2), 3, stream)
+            ceil[kname] = round(nbytes / (avg_ms * 1e-3) / 1e9, 1)
+        egrid = (K.cdiv(n_el, 1024), )
+        avg_ms, per, _ = _events_time(lambda: K.copy_kernel[egrid](xs, outs, n_el, BLOCK_SIZE=1024), max(3, steps // 2), 3, stream)
+        ceil["ew_copy_b128"] = round(2 * 4 * n_el / (avg_ms * 1e-3) / 1e9, 1)
+        r, w = ceil["ew_ceiling_read_b128"], ceil["ew_ceiling_write_b128"]
+        # bytes move at the read rate or at the write rate: the harmonic mix for a kernel's read:write ratio
+        ceil["bound_2r1w_GBs"] = round(3.0 / (2.0 / r + 1.0 / w), 1)
+        ceil["bound_1r1w_GBs"] = round(2.0 / (1.0 / r + 1.0 / w), 1)
+        extra["ew_ceiling_2p28_GBs"] = ceil
+        del xs, outs
     if want("add0"):
         n0 = 98432
         x0, y0 = torch.rand(n0, device="cuda"), torch.rand(n0, device="cuda")

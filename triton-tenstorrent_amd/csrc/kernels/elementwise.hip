@@ -495,6 +495,28 @@ __global__ __launch_bounds__(kThreads) void ew_muladd_f32(const float *__restric
   }
 }
 
+// Ceilings of streaming, for the benchmark only (launched through rt_launch, no entry point of their own): 16-byte
+// non-temporal accesses that only read (the fold is stored by a workgroup whose words happen to match a value no
+// input produces, so the loads cannot be dropped) or only write, each in the geometry that measured best for it:
+// 256 lanes x 4 vectors for reads (7100-7170 GB/s; one-wavefront workgroups of one vector move 1 KiB each and run
+// into the dispatch rate at 4700), 256 lanes x 1 vector for writes (6750; 5940 at 4 vectors per lane).
+// nvec is a whole number of 1024-vector runs.
+__global__ __launch_bounds__(256) void ew_ceiling_read_b128(const Vec4<uint32_t>::type *__restrict__ x,
+                                                            Vec4<uint32_t>::type *__restrict__ out, uint32_t nvec) {
+  const uint32_t i = blockIdx.x * 1024 + threadIdx.x;
+  if (i + 768 >= nvec) return;
+  Vec4<uint32_t>::type v = __builtin_nontemporal_load(x + i);
+#pragma unroll
+  for (int u = 1; u < 4; ++u) v ^= __builtin_nontemporal_load(x + i + u * 256);
+  if ((v.x ^ v.y ^ v.z ^ v.w) == 0x9e3779b9u && (v.x + v.y) == 0x7f4a7c15u) out[blockIdx.x] = v;
+}
+__global__ __launch_bounds__(256) void ew_ceiling_write_b128(const Vec4<uint32_t>::type *__restrict__ x,
+                                                             Vec4<uint32_t>::type *__restrict__ out, uint32_t nvec) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  __builtin_nontemporal_store((Vec4<uint32_t>::type){i, 1u, 2u, 3u}, out + i);
+}
+
 __global__ __launch_bounds__(kThreads) void ew_copy_b128(const uint8_t *x, uint8_t *out, uint64_t nbytes) {
   copy_vec_body<kVec>(x, out, nbytes);
 }
