@@ -645,3 +645,51 @@ def test_triton_jit_launches_the_fused_matmul_muladd_and_attention(tmp_path, mon
         from triton.backends import backends
         backends.pop("tenstorrent", None)
         triton.runtime.driver._active = None
+
+
+def test_installed_but_not_asked_for_the_driver_stays_passive(monkeypatch):
+    """An installed package reaches Triton through its entry point whether or not anyone wants it, and Triton refuses
+    to start with two active drivers (triton/runtime/driver.py:6-10).  Without register() / activate() or
+    TRITON_TENSTORRENT_AMD=1 the driver therefore reports itself inactive, as the reference's does where its
+    runtime is missing (backend/driver.py:449-467)."""
+    from triton_tenstorrent_amd.backend import driver as drv
+    monkeypatch.delenv("TRITON_TENSTORRENT_AMD", raising=False)
+    monkeypatch.setattr(drv, "_OPTED_IN", False)
+    assert drv.TTDriver.is_active() is False
+    monkeypatch.setattr(drv.rt, "LIB_PATH", drv.rt.LIB_PATH.parent / "missing.so")
+    monkeypatch.setenv("TRITON_TENSTORRENT_AMD", "1")
+    assert drv.TTDriver.is_active() is False      # asked for, but nothing to run on
+
+
+@pytest.mark.gpu
+def test_entry_point_coexists_with_the_stock_driver(tmp_path, monkeypatch):
+    """Both backends in Triton's table, as after `pip install`: driver selection must not raise, must pick the stock
+    HIP driver while nobody asked for this one, and register() must still route add_kernel to ew_add_f32."""
+    import importlib
+    trd = importlib.import_module("triton.runtime.driver")    # the module (the package attribute of that name is its DriverConfig)
+    from triton.backends import Backend, backends
+    from triton_tenstorrent_amd import runtime as rt
+    from triton_tenstorrent_amd.backend import driver as drv
+    from triton_tenstorrent_amd.examples import triton_kernels as tk
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("TRITON_TENSTORRENT_AMD", raising=False)
+    monkeypatch.setattr(drv, "_OPTED_IN", False)
+    backends["tenstorrent"] = Backend(compiler=ttc.TTBackend, driver=drv.TTDriver)
+    try:
+        assert "amd" in backends and backends["amd"].driver.is_active()
+        picked = trd._create_driver()                         # raises "2 active drivers" if both answer true
+        assert type(picked).__name__ != "TTDriver"
+        monkeypatch.setenv("TRITON_TENSTORRENT_AMD", "1")
+        with pytest.raises(RuntimeError, match="active drivers"):
+            trd._create_driver()                              # the opt-in is exclusive by Triton's own rule
+        monkeypatch.delenv("TRITON_TENSTORRENT_AMD")
+        ttc.register()
+        n = 5000
+        x, y = torch.rand(n, device="cuda"), torch.rand(n, device="cuda")
+        out = torch.empty_like(x)
+        tk.add_kernel[(triton.cdiv(n, 1024), )](x, y, out, n, BLOCK_SIZE=1024)
+        assert rt.last_kernel_name() == "ew_add_f32" and torch.equal(out, x + y)
+    finally:
+        backends.pop("tenstorrent", None)
+        triton.runtime.driver.reset_active()
+        drv.opt_in(False)

@@ -198,5 +198,7 @@ def register() -> None:
         raise RuntimeError("Triton is not importable; use triton_tenstorrent_amd.kernels (the C-ABI path) instead")
     import triton
     from triton.backends import Backend, backends
+    from . import driver as _drv
+    _drv.opt_in()
     backends["tenstorrent"] = Backend(compiler=TTBackend, driver=TTDriver)
     triton.runtime.driver.set_active(TTDriver())

@@ -615,11 +615,28 @@ class TTDeviceInterface:
         return TTDeviceInterface.DeviceEvent()
 
 
+_OPTED_IN = False
+
+
+def opt_in(on: bool = True) -> None:
+    """Let :meth:`TTDriver.is_active` answer true in this process (``register()`` and ``activate()`` call it)."""
+    global _OPTED_IN
+    _OPTED_IN = bool(on)
+
+
 class TTDriver(_DriverBase):
     """backend/driver.py:445-535 on an MI355X."""
 
     @staticmethod
     def is_active():
+        """True only where this backend was asked for: after ``register()`` / ``activate()`` in this process, or
+        with ``TRITON_TENSTORRENT_AMD=1`` in the environment.  Triton refuses to start with two active drivers
+        (triton/runtime/driver.py:6-10), and on a ROCm box the stock HIP driver is active already, so a package
+        that is merely installed (its entry point makes Triton import this module) must stay passive, as the
+        reference's driver does wherever its own runtime is absent (backend/driver.py:449-467)."""
+        import os
+        if not (_OPTED_IN or os.environ.get("TRITON_TENSTORRENT_AMD", "") == "1"):
+            return False
         try:
             import torch
             return bool(torch.cuda.is_available()) and rt.LIB_PATH.exists()
@@ -684,6 +701,7 @@ class TTDriver(_DriverBase):
 def activate() -> TTDriver:
     """Make this driver Triton's active one (Triton allows a single active
     driver; on a ROCm box the stock HIP driver would otherwise win)."""
+    opt_in()
     drv = TTDriver()
     if _HAVE_TRITON:
         import triton
