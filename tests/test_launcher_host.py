@@ -332,3 +332,29 @@ def test_copy_kernel_binds(fake):
     with pytest.raises(rt.InvalidLaunch):
         K.copy_kernel[(5, )](FakeTensor((5000, ), torch.float32), FakeTensor((5000, ), torch.int32), 5000, BLOCK_SIZE=1024)
 
+
+
+def test_elementwise_binders_refuse_a_launch_that_runs_past_an_operand(fake):
+    """The launch touches min(n_elements, grid * BLOCK) elements of every operand; a tensor that holds fewer would be
+    read or written out of bounds on the device, so the binder raises before anything is launched."""
+    big, small = FakeTensor((4096, ), torch.float32), FakeTensor((1000, ), torch.float32)
+    before = len(fake.calls)
+    with pytest.raises(rt.InvalidLaunch, match="covers 4096"):
+        K.add_kernel[(4, )](big, small, big, 4096, BLOCK_SIZE=1024)
+    with pytest.raises(rt.InvalidLaunch):
+        K.sin_kernel[(4, )](big, small, 4096, BLOCK_SIZE=1024)
+    with pytest.raises(rt.InvalidLaunch):
+        K.unary_kernel[(2, )](small, small, 2048, BLOCK_SIZE=1024, OP="exp")
+    with pytest.raises(rt.InvalidLaunch):
+        K.binary_kernel[(4, )](big, big, small, 4096, BLOCK_SIZE=1024, OP="mul")
+    with pytest.raises(rt.InvalidLaunch):
+        K.muladd_kernel[(4, )](big, big, small, big, 4096, BLOCK_SIZE=1024)
+    with pytest.raises(rt.InvalidLaunch):
+        K.copy_kernel[(4, )](small, big, 4096, BLOCK_SIZE=1024)
+    with pytest.raises(rt.InvalidLaunch):
+        K.add_kernel_loop[(2, )](big, big, small, 4096, 2, BLOCK_SIZE=1024)      # 2 programs x 2 rows x 1024
+    assert len(fake.calls) == before
+    # the mask and the grid both clip: a short grid or a small n_elements makes the same tensors legal
+    K.add_kernel[(1, )](big, small, big, 4096, BLOCK_SIZE=512)
+    K.add_kernel[(4, )](big, small, big, 1000, BLOCK_SIZE=1024)
+    assert len(fake.calls) == before + 2

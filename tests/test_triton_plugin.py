@@ -693,3 +693,81 @@ def test_entry_point_coexists_with_the_stock_driver(tmp_path, monkeypatch):
         backends.pop("tenstorrent", None)
         triton.runtime.driver.reset_active()
         drv.opt_in(False)
+
+
+def test_a_table_name_does_not_vouch_for_the_body(tmp_path, monkeypatch):
+    """The reference generates code from the IR, so a kernel's name means nothing there.  Here a user kernel that
+    merely carries the name of a prebuilt one (a `sin_kernel` that computes a cosine, an `add_kernel` that subtracts,
+    upstream Triton's row-major `matmul_kernel`, which shares name and signature with the reference's tile-major
+    one) must be a compile error, never a silent run of the prebuilt kernel."""
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    f32 = "*fp32"
+
+    def one_op(name, expr, nin=1):
+        ns = {"triton": triton, "tl": tl}
+        ins = ", ".join(f"p{i}" for i in range(nin))
+        loads = "\n".join(f"    v{i} = tl.load(p{i} + offs, mask=mask)" for i in range(nin))
+        src = (f"@triton.jit\ndef {name}({ins}, out_ptr, n_elements, BLOCK_SIZE: tl.constexpr):\n"
+               f"    pid = tl.program_id(axis=0)\n    offs = pid * BLOCK_SIZE + tl.arange(0, BLOCK_SIZE)\n"
+               f"    mask = offs < n_elements\n{loads}\n    tl.store(out_ptr + offs, {expr}, mask=mask)\n")
+        import linecache, hashlib
+        fname = f"<wrong_body_{hashlib.md5(src.encode()).hexdigest()[:8]}>"
+        linecache.cache[fname] = (len(src), None, src.splitlines(True), fname)
+        exec(compile(src, fname, "exec"), ns)
+        return ns[name]
+
+    sig1 = {"p0": f32, "out_ptr": f32, "n_elements": "i32", "BLOCK_SIZE": "constexpr"}
+    sig2 = {"p0": f32, "p1": f32, "out_ptr": f32, "n_elements": "i32", "BLOCK_SIZE": "constexpr"}
+    with pytest.raises(Exception, match="does not match"):
+        _compile(one_op("sin_kernel", "tl.cos(v0)"), sig1, {"BLOCK_SIZE": 1024})
+    with pytest.raises(Exception, match="does not match"):
+        _compile(one_op("add_kernel", "v0 - v1", 2), sig2, {"BLOCK_SIZE": 1024})
+    with pytest.raises(Exception, match="does not match"):
+        _compile(one_op("unary_kernel", "v0 * v1", 2), sig2, {"BLOCK_SIZE": 1024})
+    # the right bodies under those names still bind
+    assert json.loads(_compile(one_op("sin_kernel", "tl.sin(v0)"), sig1, {"BLOCK_SIZE": 1024}).kernel)["kernel"] == "sin_kernel"
+    assert json.loads(_compile(one_op("add_kernel", "v0 + v1", 2), sig2, {"BLOCK_SIZE": 1024}).kernel)["kernel"] == "add_kernel"
+    rec = json.loads(_compile(one_op("unary_kernel", "tl.exp(v0)"), sig1, {"BLOCK_SIZE": 1024}).kernel)
+    assert rec["kernel"] == "unary_kernel" and rec["match"]["op"] == "exp"
+
+    # upstream Triton's tutorial matmul: row-major, addressed through the strides
+    @triton.jit
+    def matmul_kernel(a_ptr, b_ptr, c_ptr, M, N, K, stride_am, stride_ak, stride_bk, stride_bn, stride_cm, stride_cn,
+                      BLOCK_SIZE_M: tl.constexpr, BLOCK_SIZE_N: tl.constexpr, BLOCK_SIZE_K: tl.constexpr,
+                      GROUP_SIZE_M: tl.constexpr, ACTIVATION: tl.constexpr):
+        pid = tl.program_id(axis=0)
+        num_pid_n = tl.cdiv(N, BLOCK_SIZE_N)
+        pid_m = pid // num_pid_n
+        pid_n = pid % num_pid_n
+        offs_am = (pid_m * BLOCK_SIZE_M + tl.arange(0, BLOCK_SIZE_M)) % M
+        offs_bn = (pid_n * BLOCK_SIZE_N + tl.arange(0, BLOCK_SIZE_N)) % N
+        offs_k = tl.arange(0, BLOCK_SIZE_K)
+        a_ptrs = a_ptr + (offs_am[:, None] * stride_am + offs_k[None, :] * stride_ak)
+        b_ptrs = b_ptr + (offs_k[:, None] * stride_bk + offs_bn[None, :] * stride_bn)
+        acc = tl.zeros((BLOCK_SIZE_M, BLOCK_SIZE_N), dtype=tl.float32)
+        for k in range(0, tl.cdiv(K, BLOCK_SIZE_K)):
+            a = tl.load(a_ptrs, mask=offs_k[None, :] < K - k * BLOCK_SIZE_K, other=0.0)
+            b = tl.load(b_ptrs, mask=offs_k[:, None] < K - k * BLOCK_SIZE_K, other=0.0)
+            acc = tl.dot(a, b, acc)
+            a_ptrs += BLOCK_SIZE_K * stride_ak
+            b_ptrs += BLOCK_SIZE_K * stride_bk
+        c = acc.to(tl.float16)
+        offs_cm = pid_m * BLOCK_SIZE_M + tl.arange(0, BLOCK_SIZE_M)
+        offs_cn = pid_n * BLOCK_SIZE_N + tl.arange(0, BLOCK_SIZE_N)
+        c_ptrs = c_ptr + stride_cm * offs_cm[:, None] + stride_cn * offs_cn[None, :]
+        tl.store(c_ptrs, c, mask=(offs_cm[:, None] < M) & (offs_cn[None, :] < N))
+
+    sig = {"a_ptr": "*fp16", "b_ptr": "*fp16", "c_ptr": "*fp16", "M": "i32", "N": "i32", "K": "i32", "stride_am": "i32",
+           "stride_ak": "constexpr", "stride_bk": "i32", "stride_bn": "constexpr", "stride_cm": "i32",
+           "stride_cn": "constexpr", "BLOCK_SIZE_M": "constexpr", "BLOCK_SIZE_N": "constexpr",
+           "BLOCK_SIZE_K": "constexpr", "GROUP_SIZE_M": "constexpr", "ACTIVATION": "constexpr"}
+    with pytest.raises(Exception, match="does not match"):
+        _compile(matmul_kernel, sig, {"stride_ak": 1, "stride_bn": 1, "stride_cn": 1, "BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 32,
+                                      "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 1, "ACTIVATION": ""})
+
+    # a module named like the descriptor matmul whose body is something else
+    from triton_tenstorrent_amd.backend.patterns import verify_named
+    ttir_cos = _compile(one_op("cos_user", "tl.cos(v0)"), sig1, {"BLOCK_SIZE": 1024}).asm["ttir"]
+    for table_name in ("matmul_kernel_tma", "matmul_kernel_fused", "matmul_kernel_tma_fp8_scaled", "_attn_fwd", "matmul_kernel"):
+        with pytest.raises(RuntimeError, match="does not match"):
+            verify_named(table_name, ttir_cos.replace("@cos_user", "@" + table_name))

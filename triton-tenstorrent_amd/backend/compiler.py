@@ -20,7 +20,7 @@ from types import ModuleType
 from typing import Dict, Tuple
 
 from .driver import BINARY_EXT, KERNEL_TABLE, GPUTarget, TTDriver
-from .patterns import match_empty, match_per_program, match_reduce1d, match_streaming
+from .patterns import match_empty, match_per_program, match_reduce1d, match_streaming, verify_named
 
 try:
     from triton.backends.compiler import BaseBackend, Language
@@ -153,8 +153,9 @@ class TTBackend(BaseBackend):
 
     @staticmethod
     def make_binary(src, metadata, options):
-        """Final stage: bind the kernel by NAME to the prebuilt table and return the
-        record the launcher loads.  No device code is generated."""
+        """Final stage: bind the kernel to the prebuilt table, by name where the IR under that name is the
+        table's kernel and by what the IR does otherwise, and return the record the launcher loads.  No device
+        code is generated; a kernel that matches nothing is a compile error."""
         text = str(src)
         name = TTBackend.kernel_name_of(text)
         record = {"kernel": name, "ext": BINARY_EXT, "arch": options.arch}
@@ -167,6 +168,11 @@ class TTBackend(BaseBackend):
                                    f"{sorted(KERNEL_TABLE)}, and elementwise kernels of the masked-block form with "
                                    f"one supported operation; it does no code generation")
             record.update(kernel=match["kernel"], match=match)
+        else:
+            # a table name does not vouch for the body: the IR has to be that kernel (raises otherwise)
+            match = verify_named(name, text)
+            if match is not None:
+                record.update(kernel=match["kernel"], match=match)
         metadata["name"] = name
         metadata["shared"] = 0
         metadata["warp_size"] = 64

@@ -163,6 +163,16 @@ def _contiguous_1d(t):
     return t
 
 
+def _check_extent(who: str, n: int, grid, per_program: int, *tensors):
+    """The launch touches elements [0, min(n, grid * per_program)) of every operand: each tensor has to hold that
+    many, or the kernel would read or write past an allocation (a GPU memory fault, not a Python error)."""
+    touched = min(max(int(n), 0), int(grid[0]) * int(per_program))
+    for t in tensors:
+        if t.numel() < touched:
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"{who}: the launch covers {touched} elements, an operand holds "
+                                                      f"{t.numel()}")
+
+
 # --------------------------------------------------------------------------
 # kernel name -> C entry point
 # --------------------------------------------------------------------------
@@ -178,8 +188,10 @@ def _bind_add(lib, cur: _Cursor, consts: dict, grid, stream):
     if cur.has("row_count"):  # the loop variant
         row_count = int(cur.scalar("row_count"))
         cur.done()
+        _check_extent("add_kernel", n, grid, block * max(row_count, 0), x, y, out)
         return lib.tt_add_kernel_loop(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, row_count, block, dt, grid, stream)
     cur.done()
+    _check_extent("add_kernel", n, grid, block, x, y, out)
     return lib.tt_add_kernel(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, block, dt, grid, stream)
 
 
@@ -190,6 +202,7 @@ def _bind_muladd(lib, cur, consts, grid, stream):
     for t in (x, y, z, out):
         if _torch_dtype_code(t) != rt.TT_F32:
             raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "muladd_kernel computes in fp32")
+    _check_extent("muladd_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, y, z, out)
     return lib.tt_muladd_kernel(x.data_ptr(), y.data_ptr(), z.data_ptr(), out.data_ptr(), n,
                                 int(consts["BLOCK_SIZE"]), grid, stream)
 
@@ -200,6 +213,7 @@ def _bind_sin(lib, cur, consts, grid, stream):
     cur.done()
     if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "sin_kernel computes in fp32")
+    _check_extent("sin_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, out)
     return lib.tt_sin_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
 
 
@@ -217,6 +231,7 @@ def _bind_unary(lib, cur, consts, grid, stream):
     cur.done()
     if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "unary_kernel computes in fp32")
+    _check_extent("unary_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, out)
     return lib.tt_unary_kernel(_op_code(rt.UNARY_OPS, consts, "unary_kernel"), x.data_ptr(), out.data_ptr(), n,
                                int(consts["BLOCK_SIZE"]), grid, stream)
 
@@ -229,6 +244,7 @@ def _bind_binary(lib, cur, consts, grid, stream):
     for t in (x, y, out):
         if _torch_dtype_code(t) != rt.TT_F32:
             raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "binary_kernel computes in fp32")
+    _check_extent("binary_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, y, out)
     return lib.tt_binary_kernel(_op_code(rt.BINARY_OPS, consts, "binary_kernel"), x.data_ptr(), y.data_ptr(),
                                 out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
 
@@ -241,6 +257,7 @@ def _bind_binary_const(lib, cur, consts, grid, stream):
     cur.done()
     if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "binary_const_kernel computes in fp32")
+    _check_extent("binary_const_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, out)
     return lib.tt_binary_const_kernel(_op_code(rt.BINARY_OPS, consts, "binary_const_kernel"), x.data_ptr(), float(consts["C"]),
                                       int(bool(consts.get("FLIP", False))), out.data_ptr(), n, int(consts["BLOCK_SIZE"]),
                                       grid, stream)
@@ -251,6 +268,7 @@ def _bind_cast(lib, cur, consts, grid, stream):
     x, out = _contiguous_1d(cur.tensor()), _contiguous_1d(cur.tensor())
     n = int(cur.scalar("n_elements"))
     cur.done()
+    _check_extent("cast_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, out)
     return lib.tt_cast_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), _torch_dtype_code(x),
                               _torch_dtype_code(out), grid, stream)
 
@@ -263,6 +281,7 @@ def _bind_copy(lib, cur, consts, grid, stream):
     cur.done()
     if x.dtype != out.dtype:
         raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"copy_kernel moves one element type, got {x.dtype} and {out.dtype}")
+    _check_extent("copy_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, out)
     return lib.tt_copy_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), _torch_dtype_code(x), grid, stream)
 
 

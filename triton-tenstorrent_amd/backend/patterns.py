@@ -446,3 +446,79 @@ def match_per_program(ttir: str) -> dict | None:
     strip = lambda a: a.lstrip("%")
     return {"kernel": "binary_const_kernel", "op": BINARY[op], "inputs": [strip(x_arg)], "output": strip(out_arg), "n": None,
             "n_const": None, "block": 1, "c": c, "flip": flip}
+
+
+# --------------------------------------------------------------------------
+# kernels bound by NAME: does the IR under that name do what the prebuilt kernel does?
+# --------------------------------------------------------------------------
+def _op_counts(ttir: str) -> dict:
+    text = _strip_locs(ttir)
+    ops = re.findall(r"=\s*\"?([a-z_]+\.[a-z_0-9.]+)", text) + re.findall(r"^\s*([a-z_]+\.[a-z_0-9.]+)", text, re.M)
+    counts: dict = {}
+    for o in ops:
+        counts[o] = counts.get(o, 0) + 1
+    return counts
+
+
+def verify_named(name: str, ttir: str) -> dict | None:
+    """A kernel whose NAME is in the prebuilt table still has to be that kernel: the reference generates code from
+    the IR, so there a name carries no meaning, and a user's ``sin_kernel`` that computes a cosine, or upstream
+    Triton's row-major ``matmul_kernel`` (same name and signature as the reference's tile-major one), must not run
+    the prebuilt kernel silently.  Returns the IR match to bind by (elementwise, copy and reduction forms), or None
+    to bind by name (the matmul and attention kernels, checked by a structural fingerprint); raises on a mismatch."""
+    def bad(why):
+        return RuntimeError(f"kernel '{name}' carries the name of a prebuilt gfx950 kernel but its IR does not match it "
+                            f"({why}); this backend does no code generation, rename the kernel or use the reference's source")
+
+    c = _op_counts(ttir)
+    n = lambda op: c.get(op, 0)
+    if name in ("add_kernel", "sin_kernel", "muladd_kernel", "unary_kernel", "binary_kernel", "cast_kernel",
+                "binary_const_kernel", "copy_kernel", "empty_kernel", "reduce1d_kernel"):
+        if name == "add_kernel" and n("scf.for") == 1:
+            # the loop variant (01-vector-add.loop.py:30-62): two loads, one add, one store inside one loop
+            if n("tt.load") == 2 and n("tt.store") == 1 and n("arith.addf") + n("arith.addi") >= 1 and n("tt.dot") == 0 \
+                    and not any(k.startswith("math.") for k in c) and n("arith.mulf") == 0 and n("arith.subf") == 0:
+                return None
+            raise bad("a loop, but not two loads, one addition and one store")
+        m = match_streaming(ttir) or match_reduce1d(ttir) or match_per_program(ttir) or match_empty(ttir)
+        if m is None:
+            raise bad("not a masked-block elementwise, copy, reduction or empty kernel of a supported operation")
+        want = {"add_kernel": lambda m: (m["kernel"] == "binary_kernel" and m["op"] == "add") or m["kernel"] == "add_kernel",
+                "sin_kernel": lambda m: m["kernel"] == "unary_kernel" and m["op"] == "sin",
+                "muladd_kernel": lambda m: m["kernel"] == "muladd_kernel"}.get(name, lambda m: m["kernel"] == name)
+        if not want(m):
+            raise bad(f"the IR is a {m['kernel']}" + (f" computing {m['op']}" if m.get("op") else ""))
+        # the three example kernels keep their own binders (argument order is theirs); the generic names bind by the IR
+        return None if name in ("add_kernel", "sin_kernel", "muladd_kernel") else m
+    descs = len(re.findall(r"%[\w.]+\s*:\s*!tt\.tensordesc<", _strip_locs(ttir)))
+    foreign = [k for k in c if k.startswith("math.")]
+    if name in ("matmul_kernel_tma", "matmul_kernel_tma_fp8_scaled"):
+        ok = (n("tt.dot") == 1 and n("tt.descriptor_load") == 2 and n("tt.descriptor_store") == 1 and descs == 3
+              and n("tt.load") == 0 and n("tt.store") == 0 and not foreign and n("arith.addf") == 0
+              and n("arith.mulf") <= (2 if name.endswith("fp8_scaled") else 0))
+        if not ok:
+            raise bad("expected one tt.dot over two descriptor loads, one descriptor store and no epilogue")
+    elif name == "matmul_kernel_fused":
+        ok = (n("tt.dot") == 1 and n("tt.descriptor_load") in (2, 3) and n("tt.descriptor_store") == 1 and descs == 4
+              and n("tt.load") == 0 and n("tt.store") == 0 and all(k in ("math.erf", "math.exp", "math.tanh") for k in foreign))
+        if not ok:
+            raise bad("expected one tt.dot, a bias descriptor and one descriptor store")
+    elif name == "matmul_kernel":
+        body = _body(ttir)
+        # the reference's kernel reads tile-major buffers and never uses the strides of its signature
+        # (03-matrix-multiplication.py:251-253); upstream's row-major kernel of the same name multiplies by them
+        unused = body is not None and all(not re.search(re.escape(a) + r"\b", "\n".join(body[2]))
+                                          for a, t in body[1] if "stride" in a)
+        ok = (n("tt.dot") == 1 and n("tt.load") == 2 and n("tt.store") == 1 and n("tt.descriptor_load") == 0 and descs == 0
+              and n("arith.remsi") >= 2 and unused and not foreign)
+        if not ok:
+            raise bad("expected the tile-major pointer kernel: one tt.dot over two masked loads, offsets wrapped with "
+                      "% M and % N, and the stride arguments unused")
+    elif name == "_attn_fwd":
+        d = n("tt.dot")
+        ok = (d in (2, 4) and n("math.exp2") == d and n("math.log2") == 1 and n("tt.descriptor_load") == d + 1
+              and n("tt.descriptor_store") == 1 and n("tt.store") == 1 and descs == 4 and n("tt.reduce") == d
+              and set(foreign) <= {"math.exp2", "math.log2"})
+        if not ok:
+            raise bad("expected online-softmax attention: Q.K^T and P.V per stage, exp2, log2, M stored through a pointer")
+    return None

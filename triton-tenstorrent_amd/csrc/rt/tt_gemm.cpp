@@ -144,8 +144,9 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   // fp8 fast path: e4m3 in, bf16/fp16 out, scale in the epilogue, K in steps of 64 through a 4-stage ring
   const bool fp8_io = in == TT_FP8E4M3 && (out == TT_BF16 || out == TT_F16 || out == TT_FP8E4M3) && epi == TT_EPI_NONE;
   const bool fp8_shape = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256 && g.lda < (1 << 24) && g.ldb < (1 << 24);
+  // 16-bit results leave in 16-byte stores (8 elements), e4m3 results in 4-byte ones
   const bool fp8_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 16 == 0 && g.ldb % 16 == 0 &&
-                         g.ldc % 4 == 0;
+                         g.ldc % (out == TT_FP8E4M3 ? 4 : 8) == 0;
   const bool fp8_ragged = !fp8_shape && N % 16 == 0 && K % 64 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24);
   if (full_grid && fp8_io && (fp8_shape || fp8_ragged) && fp8_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
@@ -241,8 +242,10 @@ int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t 
   // covers the problem.  Whole 256x256x128 macro tiles take the plain kernel, everything else its clamping
   // instantiation (the buffers are padded to whole 32x32 tiles, which is all it needs).
   const bool full_grid = (int64_t)grid[0] == num_pid_m * num_pid_n;
-  if (full_grid && in_dtype == TT_F16 && BM == 32 && BN == 32 && BK == 32 && aligned16(a_ptr) && aligned16(b_ptr) &&
-      aligned16(c_ptr) && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+  // the fast kernel keeps a thread's byte offset inside an A slab in 32 bits: 7 tile rows of ntk tiles of 2 KiB
+  const bool offsets_fit = cdiv64(K, 32) * 14336 + 4096 < (int64_t)1 << 32;
+  if (full_grid && offsets_fit && in_dtype == TT_F16 && BM == 32 && BN == 32 && BK == 32 && aligned16(a_ptr) &&
+      aligned16(b_ptr) && aligned16(c_ptr) && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const bool whole = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = persistent_grid(tiles, true);
