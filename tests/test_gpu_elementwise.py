@@ -140,3 +140,57 @@ def test_launch_errors_are_reported_not_fatal():
         K.add_kernel[(1, )](x.cpu(), x, x, 100, BLOCK_SIZE=1024)
     # still healthy afterwards
     assert torch.equal(K.add(x, x), x + x)
+
+
+def test_repeat_launches_keep_every_check_of_the_first():
+    """The second launch of the same call shape goes through a cached closure (one C call); whatever that
+    closure does not recognise has to fall back to the full path, with the same results and the same errors."""
+    n = 98432
+    x, y = torch.rand(n).cuda(), torch.rand(n).cuda()
+    out = torch.zeros(n, device="cuda")
+    launch = K.add_kernel[(K.cdiv(n, 1024), )]
+    for _ in range(3):
+        out.zero_()
+        launch(x, y, out, n, BLOCK_SIZE=1024)
+        assert torch.equal(out, x + y)
+    assert K.add_kernel._plan is not None
+    # another dtype, another BLOCK_SIZE, a partial grid, n == 1: same answers as a first launch
+    xi = torch.arange(n, dtype=torch.int32).cuda()
+    oi = torch.zeros_like(xi)
+    launch(xi, xi, oi, n, BLOCK_SIZE=1024)
+    assert torch.equal(oi, xi + xi)
+    out.zero_()
+    K.add_kernel[(K.cdiv(n, 512), )](x, y, out, n, BLOCK_SIZE=512)
+    assert torch.equal(out, x + y)
+    out.fill_(7.5)
+    K.add_kernel[(3, )](x, y, out, n, BLOCK_SIZE=1024)
+    K.add_kernel[(3, )](x, y, out, n, BLOCK_SIZE=1024)
+    assert torch.equal(out[:3072], (x + y)[:3072]) and torch.all(out[3072:] == 7.5)
+    out.fill_(7.5)
+    launch(x, y, out, 1, BLOCK_SIZE=1024)
+    assert out[0] == x[0] + y[0] and torch.all(out[1:] == 7.5)
+    # and the same refusals
+    launch(x, y, out, n, BLOCK_SIZE=1024)
+    with pytest.raises(ValueError):
+        launch(x[:1000], y, out, n, BLOCK_SIZE=1024)            # an operand shorter than the launch covers
+    with pytest.raises(ValueError):
+        launch(x.cpu(), y, out, n, BLOCK_SIZE=1024)
+    with pytest.raises(ValueError):
+        launch(x, y, out, -5, BLOCK_SIZE=1024)
+    with pytest.raises(ValueError):
+        launch(x, y, out.double(), n, BLOCK_SIZE=1024)
+    m = torch.rand(512, 512).cuda()
+    with pytest.raises(ValueError):
+        K.add_kernel[(256, )](m.t(), m, torch.empty_like(m), 512 * 512, BLOCK_SIZE=1024)
+    # a side stream is picked up by the cached path too
+    side = torch.cuda.Stream()
+    out.zero_()
+    with torch.cuda.stream(side):
+        launch(x, y, out, n, BLOCK_SIZE=1024)
+    side.synchronize()
+    assert torch.equal(out, x + y)
+    s = torch.zeros(n, device="cuda")
+    for _ in range(2):
+        K.sin_kernel[(K.cdiv(n, 1024), )](x, s, n, BLOCK_SIZE=1024)
+    assert K.sin_kernel._plan is not None
+    assert np.max(np.abs(s.cpu().numpy() - orc.sin(x.cpu().numpy()))) <= SIN_ATOL

@@ -135,7 +135,7 @@ def test_add_binds_and_folds_n_equal_one(fake):
     K.add_kernel[lambda meta: (K.cdiv(98432, meta["BLOCK_SIZE"]), )](x, x, x, 98432, BLOCK_SIZE=1024)
     name, a = fake.calls[-1]
     assert name == "tt_add_kernel" and a[3:6] == (98432, 1024, rt.TT_F32) and list(a[6]) == [97, 1, 1]
-    assert a[7].value == 0x1234
+    assert a[7] == 0x1234          # the stream handle, as the integer ctypes converts to void*
     K.add_kernel[(1, )](x, x, x, 1, BLOCK_SIZE=1024)     # n_elements == 1 arrives as a constexpr
     assert fake.calls[-1][1][3] == 1
     xi = FakeTensor((10, ), torch.int32)

@@ -100,9 +100,10 @@ class _Cursor:
     def __init__(self, flat: list, keep: list, ranks: list | None = None, consts: dict | None = None,
                  arg_names: list | None = None):
         self.flat, self.i, self.keep = flat, 0, keep
-        self.ranks = list(ranks or [])
-        self.consts = consts or {}
-        self.arg_names = arg_names or []
+        self.ranks = ranks if ranks is not None else []     # consumed from the front by desc()
+        self.consts = consts if consts is not None else {}
+        self.arg_names = arg_names if arg_names is not None else []
+        self.direct = None      # set by a binder that offers a repeat-launch closure (_streaming_direct)
 
     def _next(self):
         v = self.flat[self.i]
@@ -173,6 +174,39 @@ def _check_extent(who: str, n: int, grid, per_program: int, *tensors):
                                                       f"{t.numel()}")
 
 
+def _streaming_direct(fn, n_tensors: int, dtype, tail: tuple, per_program: int):
+    """Repeat-launch closure for a kernel whose launch arguments are ``n_tensors`` tensors and ``n_elements``:
+    ``direct(args, grid, stream)`` makes the same checks as the binder that built it (operand type, dtype, device,
+    contiguity, extent) and the one C call, or returns False for anything it does not recognise, so that the
+    caller takes the ordinary path (which also words the errors).  ``n_elements == 1`` is refused here because
+    Triton folds that value into the specialisation: it belongs to another launcher."""
+    import torch
+    tensor_type, grid3, check = torch.Tensor, rt.Grid3, rt.check
+
+    def direct(args, grid, stream):
+        n = args[n_tensors]
+        if type(n) is not int or not 1 < n < 2147483648 or len(grid) != 1:
+            return False
+        gx = grid[0]
+        if type(gx) is not int:
+            return False
+        touched = gx * per_program
+        if touched > n:
+            touched = n
+        ptrs = []
+        for t in args[:n_tensors]:
+            if (type(t) is not tensor_type or t.dtype is not dtype or not t.is_cuda or t.numel() < touched
+                    or not t.is_contiguous()):
+                return False
+            ptrs.append(t.data_ptr())
+        rc = fn(*ptrs, n, *tail, grid3(gx, 1, 1), stream)
+        if rc:
+            check(rc)
+        return True
+
+    return direct
+
+
 # --------------------------------------------------------------------------
 # kernel name -> C entry point
 # --------------------------------------------------------------------------
@@ -183,7 +217,7 @@ def _bind_add(lib, cur: _Cursor, consts: dict, grid, stream):
     for t in (x, y, out):
         _contiguous_1d(t)
     dt = _torch_dtype_code(x)
-    if _torch_dtype_code(y) != dt or _torch_dtype_code(out) != dt:
+    if y.dtype != x.dtype or out.dtype != x.dtype:
         raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "add_kernel: operand dtypes differ")
     if cur.has("row_count"):  # the loop variant
         row_count = int(cur.scalar("row_count"))
@@ -192,6 +226,7 @@ def _bind_add(lib, cur: _Cursor, consts: dict, grid, stream):
         return lib.tt_add_kernel_loop(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, row_count, block, dt, grid, stream)
     cur.done()
     _check_extent("add_kernel", n, grid, block, x, y, out)
+    cur.direct = _streaming_direct(lib.tt_add_kernel, 3, x.dtype, (block, dt), block)
     return lib.tt_add_kernel(x.data_ptr(), y.data_ptr(), out.data_ptr(), n, block, dt, grid, stream)
 
 
@@ -203,6 +238,8 @@ def _bind_muladd(lib, cur, consts, grid, stream):
         if _torch_dtype_code(t) != rt.TT_F32:
             raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "muladd_kernel computes in fp32")
     _check_extent("muladd_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, y, z, out)
+    cur.direct = _streaming_direct(lib.tt_muladd_kernel, 4, x.dtype, (int(consts["BLOCK_SIZE"]), ),
+                                   int(consts["BLOCK_SIZE"]))
     return lib.tt_muladd_kernel(x.data_ptr(), y.data_ptr(), z.data_ptr(), out.data_ptr(), n,
                                 int(consts["BLOCK_SIZE"]), grid, stream)
 
@@ -214,6 +251,8 @@ def _bind_sin(lib, cur, consts, grid, stream):
     if _torch_dtype_code(x) != rt.TT_F32 or _torch_dtype_code(out) != rt.TT_F32:
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "sin_kernel computes in fp32")
     _check_extent("sin_kernel", n, grid, int(consts["BLOCK_SIZE"]), x, out)
+    cur.direct = _streaming_direct(lib.tt_sin_kernel, 2, x.dtype, (int(consts["BLOCK_SIZE"]), ),
+                                   int(consts["BLOCK_SIZE"]))
     return lib.tt_sin_kernel(x.data_ptr(), out.data_ptr(), n, int(consts["BLOCK_SIZE"]), grid, stream)
 
 
@@ -538,11 +577,16 @@ class TTLauncher:
         self.signature = {idx: value for idx, value in src.signature.items()}
         self.arg_names = arg_names
         self.keepalive: list = []
+        self.direct = None      # the last launch's repeat-launch closure, when its binder offers one
         # fixed per (kernel, specialisation): computed once, used on every launch
         self._sig_types = list(self.signature.values())
         self._constexpr_pos = [(i, n) for i, (n, ty) in enumerate(zip(arg_names, self._sig_types)) if ty == "constexpr"]
         self._folded = [(arg_names[idx[0]], val) for idx, val in self.constants.items()
                         if len(idx) == 1 and idx[0] < len(arg_names)]
+        # a signature without descriptors flattens to "every non-constexpr argument, in order"
+        self._plain_pos = None
+        if not any(str(ty).startswith("tensordesc") for ty in self._sig_types):
+            self._plain_pos = [i for i, ty in enumerate(self._sig_types) if ty != "constexpr"]
 
     def __call__(self, gridX, gridY, gridZ, stream, function, *args):
         kernel_metadata, launch_metadata, launch_enter_hook, launch_exit_hook = args[0], args[1], args[2], args[3]
@@ -553,7 +597,10 @@ class TTLauncher:
             raise rt.InvalidLaunch(rt.RT_ERR_INVALID,
                                    f"{function.name}: {len(user_args)} arguments for a {len(sig_types)}-entry signature")
         ranks: list = []
-        flat = flatten_launch_args(sig_types, user_args, ranks)
+        if self._plain_pos is not None:
+            flat = [user_args[i] for i in self._plain_pos]
+        else:
+            flat = flatten_launch_args(sig_types, user_args, ranks)
         # constexprs by name: explicit constexpr parameters plus ints Triton specialised away (value 1)
         consts = {name: user_args[i] for i, name in self._constexpr_pos}
         for name, val in self._folded:
@@ -561,11 +608,13 @@ class TTLauncher:
         keep: list = []
         cur = _Cursor(flat, keep, ranks, consts, self.arg_names)
         lib = rt.init(0)
-        grid = rt.grid3(gridX, gridY, gridZ)
+        grid = rt.Grid3(gridX, gridY, gridZ)
         if launch_enter_hook is not None:
             launch_enter_hook(launch_metadata)
-        rc = function.bind(lib, cur, consts, grid, C.c_void_p(int(stream or 0)))
-        rt.check(rc)
+        rc = function.bind(lib, cur, consts, grid, stream or 0)
+        if rc:
+            rt.check(rc)
+        self.direct = cur.direct
         # launches are asynchronous: keep operands referenced until the next launch replaces them
         self.keepalive = keep
         if launch_exit_hook is not None:
