@@ -771,3 +771,34 @@ def test_a_table_name_does_not_vouch_for_the_body(tmp_path, monkeypatch):
     for table_name in ("matmul_kernel_tma", "matmul_kernel_fused", "matmul_kernel_tma_fp8_scaled", "_attn_fwd", "matmul_kernel"):
         with pytest.raises(RuntimeError, match="does not match"):
             verify_named(table_name, ttir_cos.replace("@cos_user", "@" + table_name))
+
+
+def test_every_example_kernel_passes_the_check_of_its_own_name(tmp_path, monkeypatch):
+    """The fingerprints that guard the prebuilt names must accept the kernels they are taken from, compiled by the
+    real front end at the tilings the examples launch."""
+    monkeypatch.setenv("TRITON_CACHE_DIR", str(tmp_path))
+    from triton_tenstorrent_amd.examples import triton_kernels as tk
+    mm = {"BLOCK_SIZE_M": "constexpr", "BLOCK_SIZE_N": "constexpr", "BLOCK_SIZE_K": "constexpr",
+          "GROUP_SIZE_M": "constexpr", "FP8_OUTPUT": "constexpr", "WARP_SPECIALIZE": "constexpr"}
+    mmc = {"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 8, "FP8_OUTPUT": False,
+           "WARP_SPECIALIZE": False}
+    descs = {"a_desc": "tensordesc<bf16[128,64]>", "b_desc": "tensordesc<bf16[64,128]>", "c_desc": "tensordesc<bf16[128,128]>"}
+    dims = {"M": "i32", "N": "i32", "K": "i32"}
+    k = _compile(tk.matmul_kernel_tma, {**descs, **dims, **mm}, mmc)
+    assert json.loads(k.kernel)["kernel"] == "matmul_kernel_tma"
+    k = _compile(tk.matmul_kernel_fused, {**descs, "bias_desc": "tensordesc<bf16[128,128]>", **dims, **mm}, mmc)
+    assert json.loads(k.kernel)["kernel"] == "matmul_kernel_fused"
+    qd = "tensordesc<bf16[64,64]>"
+    attn = {"sm_scale": "fp32", "M": "*fp32", "Z": "i32", "H": "i32", "desc_q": qd, "desc_k": qd, "desc_v": qd,
+            "desc_o": qd, "N_CTX": "i32", "HEAD_DIM": "constexpr", "BLOCK_M": "constexpr", "BLOCK_N": "constexpr",
+            "FP8_OUTPUT": "constexpr", "STAGE": "constexpr", "warp_specialize": "constexpr", "IS_HOPPER": "constexpr"}
+    for stage in (1, 3):
+        k = _compile(tk._attn_fwd, attn, {"HEAD_DIM": 64, "BLOCK_M": 64, "BLOCK_N": 64, "FP8_OUTPUT": False,
+                                          "STAGE": stage, "warp_specialize": False, "IS_HOPPER": False})
+        assert json.loads(k.kernel)["kernel"] == "_attn_fwd"
+    k = _compile(tk.muladd_kernel, {"x_ptr": "*fp32", "y_ptr": "*fp32", "z_ptr": "*fp32", "output_ptr": "*fp32",
+                                    "n_elements": "i32", "BLOCK_SIZE": "constexpr"}, {"BLOCK_SIZE": 1024})
+    assert json.loads(k.kernel)["kernel"] == "muladd_kernel"
+    k = _compile(tk.sin_kernel, {"x_ptr": "*fp32", "output_ptr": "*fp32", "n_elements": "i32", "BLOCK_SIZE": "constexpr"},
+                 {"BLOCK_SIZE": 1024})
+    assert json.loads(k.kernel)["kernel"] == "sin_kernel"

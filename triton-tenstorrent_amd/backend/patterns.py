@@ -490,7 +490,11 @@ def verify_named(name: str, ttir: str) -> dict | None:
             raise bad(f"the IR is a {m['kernel']}" + (f" computing {m['op']}" if m.get("op") else ""))
         # the three example kernels keep their own binders (argument order is theirs); the generic names bind by the IR
         return None if name in ("add_kernel", "sin_kernel", "muladd_kernel") else m
-    descs = len(re.findall(r"%[\w.]+\s*:\s*!tt\.tensordesc<", _strip_locs(ttir)))
+    # descriptor PARAMETERS: counted in the function header only (an op's result or operand type reads the same)
+    plain = _strip_locs(ttir)
+    head = plain[plain.find("tt.func"):]
+    head = head[:head.find("\n")] if "\n" in head else head
+    descs = len(re.findall(r"%[\w.]+\s*:\s*!tt\.tensordesc<", head))
     foreign = [k for k in c if k.startswith("math.")]
     if name in ("matmul_kernel_tma", "matmul_kernel_tma_fp8_scaled"):
         ok = (n("tt.dot") == 1 and n("tt.descriptor_load") == 2 and n("tt.descriptor_store") == 1 and descs == 3
