@@ -71,15 +71,29 @@ def _events_time(fn, steps: int, warmup: int, stream: int, tag: str | None = Non
 # dispatch, FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0: what the same counters read for the int32 add, a
 # plain copy-like kernel of known size).  Not measured live: the counters need the profiler around the process.
 # profiles/bench_all_kernels_rocprofv3.md holds the raw readings and the commands.
+TRAFFIC_FROM_COMMIT = "d86741b"   # the tree the readings below were taken from
+TRAFFIC_KERNELS_SHA = "ae4a8c729b6eb713"   # _kernel_sources_sha() of that tree: a kernel edit after the readings shows in the JSON
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_tile_bf16_epi0": int((2 * 799244 + 165485) * 1024),
-    "gemm_tile_bf16_epi2": int((2 * 386055 + 119776) * 1024),
-    "gemm_tile_fp8_bf16": int((2 * 403806 + 160068) * 1024),
-    "gemm_tiled_f16_epi0": int((2 * 860650 + 141087) * 1024),
-    "attn_tile_d128": int((2 * 197059 + 133120) * 1024),
-    "ew_add_i32": int((2 * 1048594 + 1048576) * 1024),
-    "ew_sin_f32": int((2 * 524420 + 1048595) * 1024),
+    "gemm_tile_bf16_epi0": int((2 * 800628 + 154044) * 1024),
+    "gemm_tile_bf16_epi2": int((2 * 386207 + 119310) * 1024),
+    "gemm_tile_fp8_bf16": int((2 * 400536 + 155067) * 1024),
+    "gemm_tiled_f16_epi0": int((2 * 793289 + 134912) * 1024),
+    "attn_tile_d128": int((2 * 313474 + 133262) * 1024),     # the causal launches
+    "ew_add_i32": int((2 * 1048589 + 1048576) * 1024),
+    "ew_sin_f32": int((2 * 524364 + 1048591) * 1024),
 }
+
+
+def _kernel_sources_sha() -> str:
+    """Digest of the kernel sources (names and contents of csrc/kernels), to tell whether the traffic readings above
+    still describe the kernels that run."""
+    import hashlib
+    h = hashlib.sha256()
+    for f in sorted((ROOT / "triton-tenstorrent_amd" / "csrc" / "kernels").iterdir()):
+        if f.is_file():
+            h.update(f.name.encode())
+            h.update(f.read_bytes())
+    return h.hexdigest()[:16]
 
 
 def _roof(bound: str, achieved: float, peak: float, unit: str, kernel: str = ""):
@@ -123,6 +137,8 @@ def main() -> int:
     extra: dict = {"device": props["name"], "arch": props["arch"], "cus": props["multiprocessor_count"],
                    "clock_mhz": props["clock_khz"] // 1000,
                    "peaks": {"hbm_GBs": PEAK_HBM_GBS, "bf16_TFLOPs": PEAK_BF16_TFLOPS, "fp8_TFLOPs": PEAK_FP8_TFLOPS}}
+    extra["traffic_from_commit"] = TRAFFIC_FROM_COMMIT
+    extra["traffic_kernels_unchanged"] = _kernel_sources_sha() == TRAFFIC_KERNELS_SHA
     rooflines: dict = {}
     parity_failed = False
     torch.manual_seed(0)
