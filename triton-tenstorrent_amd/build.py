@@ -19,6 +19,7 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 BUILD = PKG / "build"
 LIB = PKG / "lib" / "libttamd_rt.so"
+CPUABI_LIB = PKG / "lib" / "libttamd_cpuabi.so"
 ARCH = "gfx950"
 
 CODE_OBJECTS = ["elementwise", "gemm", "attention", "reduce"]
@@ -65,9 +66,20 @@ def build_runtime() -> Path:
     return LIB
 
 
+def build_cpu_abi() -> Path:
+    """libttamd_cpuabi.so: host-only support (the barrier) for kernels with the reference's cpu/ calling
+    convention; plain g++, no ROCm."""
+    CPUABI_LIB.parent.mkdir(exist_ok=True)
+    cxx = shutil.which("g++") or "g++"
+    _run([cxx, "-shared", "-fPIC", "-O2", "-std=c++17", "-fvisibility=hidden", "-Wall", "-Wextra", "-pthread",
+          f"-I{ROOT / 'include'}", str(CSRC / "cpuabi" / "cpu_abi.cpp"), "-o", str(CPUABI_LIB)])
+    return CPUABI_LIB
+
+
 def build_all(jobs: int = 4) -> Path:
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(build_code_object, CODE_OBJECTS))
+    build_cpu_abi()
     return build_runtime()
 
 
