@@ -329,6 +329,17 @@ def main() -> int:
         ref = torch.nn.functional.gelu(a[rows].double() @ b.double() + bias.double()).float()
         ok = bool(torch.all((c[rows].float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4))
         extra["gemm_gelu_4096x14336x4096"]["parity_rows_ok"] = ok
+        # the same shape without the epilogue: what the bias and the GELU cost, apart from what the shape costs
+        # (896 macro tiles on 256 CUs are 3.5 rounds, the last one run as half tiles)
+        c2 = torch.empty_like(c)
+        c2d = TensorDescriptor.from_tensor(c2, [32, 32])
+        avg0, _, _ = _events_time(
+            lambda: K.matmul_kernel_tma[grid](ad, bd, c2d, Mf, Nf, Kf, FP8_OUTPUT=False, WARP_SPECIALIZE=False),
+            steps, warmup, stream)
+        tf0 = 2.0 * Mf * Nf * Kf / (avg0 * 1e-3) / 1e12
+        extra["gemm_gelu_4096x14336x4096"]["plain_same_shape_TFLOPs"] = round(tf0, 2)
+        extra["gemm_gelu_4096x14336x4096"]["gelu_over_plain"] = round(tf / tf0, 4)
+        del c2, c2d
         parity_failed |= not ok
         del a, b, c, bias, ref
     if want("fp8"):
