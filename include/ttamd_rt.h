@@ -305,7 +305,10 @@ TTAMD_API int tt_matmul_kernel_tma_fp8_scaled(const tt_desc2d *a, const tt_desc2
  * pointer-based kernel.  a, b and c are TILE-MAJOR buffers with tiles of
  * BLOCK_M x BLOCK_K, BLOCK_K x BLOCK_N and BLOCK_M x BLOCK_N elements, row-major
  * inside a tile, tiles in row-major order (:326-337, 349-357, 377-385); ragged
- * edges need the buffers padded to whole tiles.  The strides are checked to be
+ * edges need the buffers padded to whole tiles; what the padding holds does not
+ * matter (elements past K are masked to zero as in the kernel, :340-342, 359-361;
+ * rows past M and columns past N only feed results that are never stored, and
+ * the padding of c is never written).  The strides are checked to be
  * positive, as the kernel asserts, and otherwise unused, as in the kernel.
  * in_dtype is TT_F16 or TT_BF16; c is always fp16 (:374).  leaky_relu != 0
  * applies ACTIVATION == "leaky_relu" to the fp32 accumulator (:370-373, 396-397). */
