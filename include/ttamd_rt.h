@@ -142,7 +142,8 @@ typedef struct tt_desc2d {
   int32_t shape[2];
   int64_t strides[2];
   int32_t block_shape[2];
-  int32_t padding_nan; /* 1 if padding == "nan" (driver.py:326); only 0 is supported */
+  int32_t padding_nan; /* 1 if padding == "nan" (driver.py:326): elements outside the matrix read as NaN (matmul
+                          operands; meaningless on outputs; refused by tt_attn_fwd) */
   int32_t dtype;       /* tt_dtype */
 } tt_desc2d;
 

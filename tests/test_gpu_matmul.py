@@ -514,3 +514,43 @@ def test_fp8_full_size_8192_properties():
     assert bool(torch.all((c[:, cols].float() - ref).abs() <= RTOL * ref.abs() + 1e-4 * ref.square().mean().sqrt()))
     eye = torch.eye(n, device="cuda").to(torch.float8_e4m3fn)
     assert torch.equal(K.matmul_fp8_scaled(qa, eye, 1.0, 1.0), qa.to(torch.bfloat16))   # e4m3 values are exact in bf16
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_nan_padded_descriptors(dtype):
+    """`padding="nan"` (reference backend/driver.py:322-329): elements of A and B outside the matrix read as NaN.
+    Rows past M and columns past N only reach results that are not stored, so the option shows exactly when K is not
+    a whole number of BLOCK_SIZE_K steps, and then in every stored element (NaN * x in each sum)."""
+    torch.manual_seed(5)
+
+    def run(M, N, Kd, pad_a, pad_b, bk=64):
+        a = (torch.randn(M, Kd, device="cuda") / 8).to(dtype)
+        b = (torch.randn(Kd, N, device="cuda") / 8).to(dtype)
+        c = torch.full((M + 1, N), 7.0, device="cuda", dtype=dtype)
+        ad = TensorDescriptor.from_tensor(a, [128, bk], padding=pad_a)
+        bd = TensorDescriptor.from_tensor(b, [bk, 128], padding=pad_b)
+        cd = TensorDescriptor.from_tensor(c[:M], [128, 128])
+        grid = (K.cdiv(M, 128) * K.cdiv(N, 128), )
+        K.matmul_kernel_tma[grid](ad, bd, cd, M, N, Kd, BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=bk,
+                                  GROUP_SIZE_M=8, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+        assert torch.all(c[M] == 7.0)                                 # nothing past the last row
+        return a, b, c[:M], rt.last_kernel_name()
+
+    # K a whole number of steps: the option changes nothing, ragged M and N included, and the fast kernels still run
+    for shape in ((512, 512, 256), (300, 264, 128)):
+        a, b, c_nan, name = run(*shape, "nan", "nan")
+        ref = (a.double() @ b.double()).float()
+        assert not torch.isnan(c_nan).any()
+        assert torch.all((c_nan.float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4)
+        assert name.startswith(("gemm_tile_", "gemm_ragged_"))
+    # K = 96 with 64-deep steps: the second step is half padding.  NaN on either operand poisons every element
+    for pads in (("nan", "zero"), ("zero", "nan"), ("nan", "nan")):
+        _, _, c, name = run(256, 256, 96, *pads)
+        assert torch.isnan(c).all() and name.startswith("gemm_any_")
+    # the same shape with zero padding on both is an ordinary product
+    a, b, c, _ = run(256, 256, 96, "zero", "zero")
+    ref = (a.double() @ b.double()).float()
+    assert torch.all((c.float() - ref).abs() <= 1e-2 * ref.abs() + 1e-4)
+    # 32-deep steps divide 96: no padding along K, no NaN
+    _, _, c, _ = run(256, 256, 96, "nan", "nan", bk=32)
+    assert not torch.isnan(c).any()

@@ -71,7 +71,9 @@ __device__ __forceinline__ void gemm_any_body(const GemmArgs &g) {
     const int64_t am = m0 + r32, bn = n0 + r32;
     const bool am_ok = am < g.M, bn_ok = bn < g.N;
     f32x16 acc = {0};
-    for (int k0 = 0; k0 < g.K; k0 += 16) {
+    // a descriptor with NaN padding pads the last BLOCK_SIZE_K step, so the walk then runs to the end of that step
+    const int k_end = (!TILED && (g.pad_a | g.pad_b)) ? (g.K + g.BK - 1) / g.BK * g.BK : g.K;
+    for (int k0 = 0; k0 < k_end; k0 += 16) {
       union { typename F::vec v; uint16_t s[8]; } a, b;
       const int kb = k0 + kg * 8;
 #pragma unroll
@@ -82,8 +84,8 @@ __device__ __forceinline__ void gemm_any_body(const GemmArgs &g) {
           a.s[j] = (am_ok && k_ok) ? F::enc(g.a, tiled_off(am, k, g.BM, g.BK, ntk)) : (uint16_t)0;
           b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, tiled_off(k, bn, g.BK, g.BN, ntn)) : (uint16_t)0;
         } else {
-          a.s[j] = (am_ok && k_ok) ? F::enc(g.a, am * g.lda + k) : (uint16_t)0;
-          b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, (int64_t)k * g.ldb + bn) : (uint16_t)0;
+          a.s[j] = (am_ok && k_ok) ? F::enc(g.a, am * g.lda + k) : (k < k_end ? g.pad_a : (uint16_t)0);
+          b.s[j] = (bn_ok && k_ok) ? F::enc(g.b, (int64_t)k * g.ldb + bn) : (k < k_end ? g.pad_b : (uint16_t)0);
         }
       }
       acc = F::mfma(a.v, b.v, acc);

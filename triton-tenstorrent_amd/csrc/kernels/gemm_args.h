@@ -16,6 +16,8 @@ struct GemmArgs {
   int32_t num_pid_m, num_pid_n;
   int32_t epi;
   float scale;              // multiplies the accumulator before the cast
+  uint16_t pad_a, pad_b;    // any-shape kernels: what an element of a / b outside the matrix reads as (16-bit operand bits):
+                            // 0, or a NaN for descriptors with padding == "nan" (backend/driver.py:322-329)
   int32_t tiled;            // operands are tile-major buffers with tiles BM x BK, BK x BN, BM x BN (ld* unused)
   unsigned long long *probe; // diagnostic: workgroup 0 stores {core-clock cycles, 100 MHz ticks} of its run, or null
 };

@@ -26,9 +26,6 @@ int check_desc(const char *who, const char *what, const tt_desc2d *d, int64_t ro
   if (!d->base) return fail(RT_ERR_INVALID, "%s: %s descriptor has a null base", who, what);
   if (d->dtype != TT_F32 && d->dtype != TT_BF16 && d->dtype != TT_F16 && d->dtype != TT_FP8E4M3)
     return fail(RT_ERR_UNSUPPORTED, "%s: %s dtype %d", who, what, d->dtype);
-  if (d->padding_nan)
-    return fail(RT_ERR_UNSUPPORTED, "%s: %s descriptor asks for NaN padding; only zero padding exists",
-                who, what);
   if (d->strides[1] != 1)
     return fail(RT_ERR_INVALID, "%s: %s descriptor's last stride is %lld, must be 1", who, what,
                 (long long)d->strides[1]);
@@ -97,8 +94,18 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   default: return fail(RT_ERR_INVALID, "%s: unknown epilogue %d", who, epi);
   }
 
-  const char *name = nullptr;
+  // padding == "nan" (backend/driver.py:322-329): elements of a and b outside the matrix read as NaN instead
+  // of zero.  Rows past M and columns past N only feed results that are never stored, so the option shows
+  // only when K is not a whole number of BLOCK_SIZE_K steps: then every product picks up NaN * x.  Those
+  // launches take the any-shape kernel, which reads out-of-range elements as pad_a / pad_b; for all others
+  // the result is the zero-padded one.  On the output (and on a full bias, whose out-of-range elements are
+  // added to results that are not stored) the option has no meaning and is ignored.
   const int in = a->dtype, out = c->dtype;
+  const uint16_t nan16 = in == TT_F16 ? 0x7e00 : 0x7fc0;   // e4m3 operands are widened to bf16 in that kernel
+  g.pad_a = a->padding_nan ? nan16 : 0;
+  g.pad_b = b->padding_nan ? nan16 : 0;
+  const bool nan_shows = (a->padding_nan || b->padding_nan) && K % BK != 0;
+  const char *name = nullptr;
   if (in == TT_BF16 && out == TT_BF16) name = "gemm_any_bf16_bf16";
   else if (in == TT_F16 && out == TT_F16) name = "gemm_any_f16_f16";
   else if (in == TT_FP8E4M3 && out == TT_BF16) name = "gemm_any_fp8_bf16";
@@ -117,7 +124,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   // The same kernel with clamped fetches, zero-padded K steps and clipped stores takes every other shape
   // whose rows can be fetched in 16-byte pieces and whose K is a whole number of 32-deep steps.
   const bool ragged_shape = !fast_shape && N % 8 == 0 && K % 32 == 0 && g.lda < (1 << 23) && g.ldb < (1 << 23);
-  if (full_grid && half_io && (fast_shape || ragged_shape) && fast_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+  if (full_grid && half_io && (fast_shape || ragged_shape) && fast_align && !nan_shows && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     char fast_name[64];
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
              epi);
@@ -148,7 +155,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   const bool fp8_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 16 == 0 && g.ldb % 16 == 0 &&
                          g.ldc % (out == TT_FP8E4M3 ? 4 : 8) == 0;
   const bool fp8_ragged = !fp8_shape && N % 16 == 0 && K % 64 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24);
-  if (full_grid && fp8_io && (fp8_shape || fp8_ragged) && fp8_align && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+  if (full_grid && fp8_io && (fp8_shape || fp8_ragged) && fp8_align && !nan_shows && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = persistent_grid(tiles, true);
     void *fargs[] = {&g};
