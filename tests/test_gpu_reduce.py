@@ -135,3 +135,33 @@ def test_large_blocks_across_workgroups_streams_and_repeats():
     for got, w in outs:
         assert got.cpu().numpy()[0] == w
 
+
+
+def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
+    """From the second call of one shape on, the launch is a cached closure; another dtype, operation or block size,
+    a short operand or a host tensor must come out as on a first call."""
+    n = 4096
+    x = torch.randn(n, device="cuda")
+    z = torch.empty(1, device="cuda")
+    launch = K.reduce1d_kernel[(1, )]
+    for _ in range(3):
+        z.zero_()
+        launch(x, z, BLOCK=n, OP="max")
+        assert z.item() == x.max().item()
+    assert K.reduce1d_kernel._plan is not None
+    zi = torch.empty(1, device="cuda", dtype=torch.int32)
+    launch(x, zi, BLOCK=n, OP="argmax")
+    assert zi.item() == int(torch.argmax(x))
+    launch(x, z, BLOCK=512, OP="max")
+    assert z.item() == x[:512].max().item()
+    xi = torch.arange(n, device="cuda", dtype=torch.int32)
+    launch(xi, zi, BLOCK=n, OP="sum")
+    launch(xi, zi, BLOCK=n, OP="sum")
+    assert zi.item() == n * (n - 1) // 2
+    launch(x, z, BLOCK=n, OP="max")
+    with pytest.raises(ValueError):
+        launch(x[:100], z, BLOCK=n, OP="max")
+    with pytest.raises(ValueError):
+        launch(x.cpu(), z, BLOCK=n, OP="max")
+    launch(x, z, BLOCK=n, OP="max")
+    assert z.item() == x.max().item()

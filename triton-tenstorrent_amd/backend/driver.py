@@ -207,6 +207,27 @@ def _streaming_direct(fn, n_tensors: int, dtype, tail: tuple, per_program: int):
     return direct
 
 
+def _reduce_direct(fn, op_code: int, x_dtype, z_dtype, fixed: tuple):
+    """Repeat-launch closure of ``reduce1d_kernel`` (see ``_streaming_direct``): the same checks as its binder for
+    a call of the same shape, then the one C call.  ``fixed`` = (BLOCK, input, accumulate and output dtype codes,
+    NaN flag), all set by the constexprs and dtypes that the closure re-checks."""
+    import torch
+    tensor_type, grid3, check, block = torch.Tensor, rt.Grid3, rt.check, fixed[0]
+
+    def direct(args, grid, stream):
+        x, z = args
+        if (type(x) is not tensor_type or type(z) is not tensor_type or x.dtype is not x_dtype or z.dtype is not z_dtype
+                or not x.is_cuda or not z.is_cuda or x.numel() < block or z.numel() < 1 or not x.is_contiguous()
+                or not 1 <= len(grid) <= 3):
+            return False
+        rc = fn(op_code, x.data_ptr(), z.data_ptr(), *fixed, grid3(*grid, *(1, 1, 1)[len(grid):]), stream)
+        if rc:
+            check(rc)
+        return True
+
+    return direct
+
+
 # --------------------------------------------------------------------------
 # kernel name -> C entry point
 # --------------------------------------------------------------------------
@@ -360,8 +381,9 @@ def _bind_reduce1d(lib, cur, consts, grid, stream):
     if x.numel() < block or z.numel() < 1:
         raise rt.InvalidLaunch(rt.RT_ERR_INVALID, f"reduce1d_kernel: X holds {x.numel()} elements, BLOCK is {block}")
     in_dt = _torch_dtype_code(x)
-    return lib.tt_reduce1d_kernel(rt.REDUCE_OPS[op], x.data_ptr(), z.data_ptr(), block, in_dt, reduce_acc_dtype(op, in_dt),
-                                  _torch_dtype_code(z), int(bool(consts.get("PROPAGATE_NAN", False))), grid, stream)
+    fixed = (block, in_dt, reduce_acc_dtype(op, in_dt), _torch_dtype_code(z), int(bool(consts.get("PROPAGATE_NAN", False))))
+    cur.direct = _reduce_direct(lib.tt_reduce1d_kernel, rt.REDUCE_OPS[op], x.dtype, z.dtype, fixed)
+    return lib.tt_reduce1d_kernel(rt.REDUCE_OPS[op], x.data_ptr(), z.data_ptr(), *fixed, grid, stream)
 
 
 def _mnk(cur: _Cursor, a: rt.tt_desc2d, b: rt.tt_desc2d):
