@@ -66,6 +66,7 @@ def fake(monkeypatch):
               K.matmul_kernel_tma_fp8_scaled, K.muladd_kernel, K.matmul_kernel, K.unary_kernel, K.binary_kernel,
               K.cast_kernel, K.reduce1d_kernel, K.binary_const_kernel, K.copy_kernel):
         k._cache.clear()
+        k._plan = None
     return lib
 
 
@@ -79,6 +80,8 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_calls_before_init_return_errors_instead_of_aborting():
+    if rt._inited_device is not None:
+        pytest.skip("an earlier test of this process has initialised the runtime")
     lib = rt.load()
     g = rt.grid3(1)
     assert lib.tt_add_kernel(None, None, None, 4, 1024, rt.TT_F32, g, None) == rt.RT_ERR_NOT_INIT

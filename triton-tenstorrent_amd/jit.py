@@ -77,6 +77,7 @@ class Config:
 
 
 _driver: TTDriver | None = None
+_STOCK_GET_STREAM = TTDriver.get_current_stream      # a driver whose stream lookup was replaced is asked, not bypassed
 _raw_stream = None      # (current device, its current stream) without building torch.cuda.Stream objects
 
 
@@ -149,7 +150,7 @@ class PrebuiltKernel:
 
     def run(self, *args, grid, **kwargs):
         plan = self._plan
-        if (plan is not None and len(args) == plan[0] and kwargs == plan[1] and type(grid) is tuple
+        if (plan is not None and TTDriver.get_current_stream is _STOCK_GET_STREAM and len(args) == plan[0] and kwargs == plan[1] and type(grid) is tuple
                 and PrebuiltKernel.launch_enter_hook is None and PrebuiltKernel.launch_exit_hook is None):
             device, stream = _raw_stream()
             if device == plan[2] and plan[3](args, grid, stream):
@@ -167,7 +168,7 @@ class PrebuiltKernel:
         constexprs = self.constexprs
         drv = active_driver()
         types = tuple([specialize(v, n in constexprs) for n, v in bound.items()])
-        if _raw_stream is not None and type(drv).get_current_stream is TTDriver.get_current_stream:
+        if _raw_stream is not None and type(drv).get_current_stream is _STOCK_GET_STREAM:
             device, stream = _raw_stream()
         else:
             device = drv.get_current_device()
