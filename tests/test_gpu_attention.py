@@ -245,3 +245,32 @@ def test_causal_mask_is_the_sources_at_block_m_32(S, D, kernel):
         # the stated difference: at BLOCK_M = 128 the source itself would leak row 70 to key 100
         o128, _ = orc.attn_fwd(bits(q), bits(k), bits(v), 1.0, causal=True, BLOCK_M=128, BLOCK_N=min(32, D))
         assert np.array_equal(orc.from_bf16(o128)[0, 0, 70], decode(v)[0, 0, 100])
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Z,H,S", [(2, 32, 2304), (1, 40, 3328), (3, 3, 768)])
+def test_items_chained_inside_a_workgroup(causal, Z, H, S):
+    """The head dim 128 kernel walks (head, pair of query blocks) items on a persistent grid and lets each item's last
+    copies fetch the first key blocks of the next one, which may belong to another head.  Shapes with more items
+    than CUs (288 and 280 against 256), an odd number of query blocks (9, 13: the middle block is an item on its own,
+    so items of one and of two blocks alternate) and a head count that is not a multiple of 8; every row of sampled
+    heads and of the heads where a workgroup changes head, against float64."""
+    from triton_tenstorrent_amd import runtime as rt
+    D = 128
+    g = torch.Generator(device="cuda").manual_seed(Z * 1000 + S)
+    q, k, v = (torch.randn(Z, H, S, D, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+    # every head gets its own offset in V, so that output rows computed from another head's keys or values show
+    v = (v.float() + torch.arange(Z * H, device="cuda").view(Z, H, 1, 1).float() * 0.25).to(torch.bfloat16)
+    sm = D ** -0.5
+    o, M = K.attention(q, k, v, causal, sm, return_lse=True)
+    assert rt.last_kernel_name() == "attn_tile_d128"
+    heads = sorted({0, 1, Z * H // 2, Z * H - 2, Z * H - 1, 7, 8} & set(range(Z * H)))
+    rows = torch.arange(S, device="cuda")
+    for hh in heads:
+        z, h = divmod(hh, H)
+        s = (q[z, h].double() @ k[z, h].double().T) * sm
+        if causal:
+            s = s.masked_fill(rows[:, None] < rows[None, :], float("-inf"))
+        ref = torch.softmax(s, -1) @ v[z, h].double()
+        assert (o[z, h].double() - ref).abs().max() <= O_ATOL * max(1.0, float(v[z, h].float().abs().max()))
+        assert (M[z, h].double() - torch.logsumexp(s, -1) / np.log(2.0)).abs().max() <= M_ATOL

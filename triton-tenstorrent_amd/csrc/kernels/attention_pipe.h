@@ -22,6 +22,12 @@
 //   + barrier between the phases, cross-phase fragment prefetch     889 / 1046
 //   + reference maximum raised only when outgrown by 2^8 (below)    936 / 1117
 //   + query blocks i and n-1-i in one workgroup                    1015 / 1112
+// and, measured against that kernel in one process on another box (996 / 1121 there):
+//   + K tiles of all stages below 64 KiB of LDS, V tiles above: every fragment address is register + immediate (the
+//     stage offsets no longer fit the instruction's 16-bit field otherwise: 18 VALU additions per block)
+//   + falling issue priority over a phase (below)
+//   + a workgroup's items back to back: each one's trailing copies fetch the first key blocks of the next, Q is
+//     loaded behind the first copies, one workgroup per CU walks its share of the items      1027 / 1149
 //
 // Two stated differences from a literal evaluation of the source, both inside the tolerance of the parity tests:
 //  * The exponent reference m_i of a row is the running maximum of the source, except that a new block maximum
@@ -49,12 +55,27 @@ constexpr int BN = 64;        // keys per block
 constexpr int NST = 4;        // LDS stages
 constexpr int GK = 2, GV = 2; // fragments per read group
 constexpr float LAZY_T = 8.0f;
+// A wavefront's issue priority falls from 3 to 0 over each phase, a step every PRIO_STEP MFMAs: of the two
+// wavefronts of a SIMD the one that is behind then wins arbitration.  Left alone the older wavefront always wins: it
+// ran its phases in 1190 + 1020 cycles and waited 800 at the barrier for the other one's 1380 + 1560.
+constexpr int PRIO_STEP = 4, PRIO_TOP = 3;
+__device__ __forceinline__ void set_prio(int p) {   // s_setprio takes an immediate
+  switch (p) {
+  case 0: __builtin_amdgcn_s_setprio(0); break;
+  case 1: __builtin_amdgcn_s_setprio(1); break;
+  case 2: __builtin_amdgcn_s_setprio(2); break;
+  default: __builtin_amdgcn_s_setprio(3); break;
+  }
+}
 
-template <int D>
-__device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int head, const int qblk) {
+// PREFETCHED: blocks 0, 1, 2 of this item are already in stages 0, 1, 2 (the item before it fetched them with its
+// trailing copies).  next_head: the head of the item that follows in this workgroup (this item's own head when none
+// does): this item's trailing copies fetch that head's first key blocks.
+template <int D, bool PREFETCHED>
+__device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int head, const int qblk, const int next_head) {
   constexpr int BM = 256;
   constexpr int DK = D / 16, DT = D / 32, ROW = D * 2, CH = D / 8;
-  constexpr int TILE = BN * ROW, STG = 2 * TILE;
+  constexpr int TILE = BN * ROW, STG = TILE, VBASE = NST * TILE;   // stage s: K at s*TILE, V at VBASE + s*TILE
   static_assert(D == 128, "the LDS swizzles below are those of 256-byte rows");
   static_assert((NST & (NST - 1)) == 0, "the stage ring wraps with a mask");
   const int tid = threadIdx.x, lane = tid & 63;
@@ -80,6 +101,8 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   const uint32_t v_voff = (uint32_t)(((int64_t)crow * a.ldv + v_chunk * 8) * 2);
   const uint8_t *kg = (const uint8_t *)(a.k + base * a.ldk);
   const uint8_t *vg = (const uint8_t *)(a.v + base * a.ldv);
+  const uint8_t *kg_next = (const uint8_t *)(a.k + (int64_t)next_head * a.n_ctx * a.ldk);
+  const uint8_t *vg_next = (const uint8_t *)(a.v + (int64_t)next_head * a.n_ctx * a.ldv);
   const int lds_wave = wave * 1024;
   auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst) {
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst + lds_wave);
@@ -92,9 +115,10 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   // the last one is fetched from the last one again (a harmless refetch into a stage nobody reads any more), so
   // that every wavefront issues four copies per block period and the vmcnt waits are the same everywhere.
   auto dma_piece = [&](int blk, int stage_o, int r) {
-    const int64_t row0 = (int64_t)min(blk, nblk - 1) * BN + (r & 1) * 32;
-    if (r < 2) dma_one(kg + row0 * a.ldk * 2, k_voff, lds + stage_o + (r & 1) * 8192);
-    else dma_one(vg + row0 * a.ldv * 2, v_voff, lds + stage_o + TILE + (r & 1) * 8192);
+    const bool own = blk < nblk;
+    const int64_t row0 = (int64_t)(own ? blk : blk - nblk) * BN + (r & 1) * 32;
+    if (r < 2) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, k_voff, lds + stage_o + (r & 1) * 8192);
+    else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, v_voff, lds + VBASE + stage_o + (r & 1) * 8192);
   };
   auto dma_block = [&](int blk, int stage_o) {
 #pragma unroll
@@ -109,18 +133,10 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   const int v_cc = (G4 & 1) * 2 + ((i16 >> 1) & 1);
   int v_off[DT];                 // V^T (A operand of O^T) through transposing reads: key row hi*4+qd (+ k4*16 + h2*8)
 #pragma unroll
-  for (int t = 0; t < DT; ++t) v_off[t] = TILE + (hi * 4 + qd) * ROW + (((t * 4 + v_cc) ^ (qd << 2)) << 4) + ((i16 & 1) << 3);
+  for (int t = 0; t < DT; ++t) v_off[t] = VBASE + (hi * 4 + qd) * ROW + (((t * 4 + v_cc) ^ (qd << 2)) << 4) + ((i16 & 1) << 3);
 
   union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; uint32_t w[4]; };
   Frag qf[DK];
-  {
-    const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
-#pragma unroll
-    for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
-    // the loads land here: the compiler's own vmcnt bookkeeping does not see the copies issued from assembly
-#pragma unroll
-    for (int s = 0; s < DK; ++s) asm volatile("" : "+v"(qf[s].v));
-  }
   f32x16 acc[DT];
 #pragma unroll
   for (int t = 0; t < DT; ++t) acc[t] = (f32x16){0};
@@ -139,11 +155,23 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   };
 
   // ---- prologue: blocks 0, 1, 2 in flight; S^T(0); the first K fragments of block 1 ----
-  dma_block(0, 0);
-  dma_block(1, STG);
-  dma_block(2, 2 * STG);
+  if constexpr (!PREFETCHED) {
+    dma_block(0, 0);
+    dma_block(1, STG);
+    dma_block(2, 2 * STG);
+  }
+  // Q after the copies, so that the two round trips to memory overlap; the wait the compiler puts in front of the
+  // first use of Q is for everything older as well, the copies included
+  {
+    const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
+#pragma unroll
+    for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+    // the loads land here: the compiler's own vmcnt bookkeeping does not see the copies issued from assembly
+#pragma unroll
+    for (int s = 0; s < DK; ++s) asm volatile("" : "+v"(qf[s].v));
+  }
   f32x16 s0[2], s1[2];   // scores of the current block and of the next, alternating roles
-  asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");   // blocks 0 and 1 have landed
+  if constexpr (!PREFETCHED) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");   // every wavefront's copies have landed
   s0[0] = s0[1] = (f32x16){0};
 #pragma unroll
   for (int i = 0; i < 2 * DK; ++i) s0[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rdK(lds, i), qf[i >> 1].v, s0[i & 1], 0, 0, 0);
@@ -223,6 +251,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
       for (int i = 0; i < GK; ++i) kf[i] = kpre[i];
 #pragma unroll
       for (int i = 0; i < 2 * DK; ++i) {
+        if (i % PRIO_STEP == 0) set_prio(PRIO_TOP - (i / PRIO_STEP) * PRIO_TOP / (2 * DK / PRIO_STEP - 1));
         if (i % GK == 0 && i + GK < 2 * DK) {
 #pragma unroll
           for (int g = 0; g < GK; ++g) kf[(i + GK + g) % (2 * GK)] = rdK(nxt, i + GK + g);
@@ -261,6 +290,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 #pragma unroll
     for (int i = 0; i < 4 * DT; ++i) {
       const int k4 = i >> 2, t = i & 3;
+      if (i % PRIO_STEP == 0) set_prio(PRIO_TOP - (i / PRIO_STEP) * PRIO_TOP / (4 * DT / PRIO_STEP - 1));
       if (i % GV == 0 && i + GV < 4 * DT) {
 #pragma unroll
         for (int g = 0; g < GV; ++g) vf[(i + GV + g) % (2 * GV)] = rdV(cur, i + GV + g);
@@ -337,20 +367,44 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 
 extern "C" {
 
-// grid: heads * ceil(qblocks / 2) workgroups of 512.  A workgroup takes the query blocks n-1-p and p of one head, the
-// heavy one first: under the causal mask every workgroup then streams the same number of key blocks, and there
-// are half as many workgroups to launch.
+// Persistent: gridDim.x workgroups (one per CU when there is that much work) walk the (head, pair of query blocks)
+// items in the order the dispatcher would have dealt one-item workgroups: item n of workgroup g is g + n * gridDim.x,
+// re-dealt so that an XCD's workgroups hold neighbouring items of the same heads.  A workgroup's items run back to
+// back: each one's trailing copies fetch the first key blocks of the next.
 __global__ __launch_bounds__(512) void attn_tile_d128(AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 128 * 2];
   const int qblocks = a.rows / 256;
   const int per_head = (qblocks + 1) / 2, total = per_head * a.heads;
-  int id = blockIdx.x;
-  if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;   // a head's workgroups on one XCD
-  const int head = id / per_head, p = id % per_head;
-  pipeattn::body<128>(a, lds, head, qblocks - 1 - p);
-  if (p != qblocks - 1 - p) {
-    asm volatile("s_barrier" ::: "memory");   // nobody reads the stages of the first block any more
-    pipeattn::body<128>(a, lds, head, p);
+  auto decode = [&](int n, int &head, int &p) {
+    int id = n;
+    if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+    head = id / per_head;
+    p = id % per_head;
+  };
+  // the items of this workgroup in order: (n, which), which = 0: query block qblocks-1-p, 1: query block p
+  auto advance = [&](int &n, int &head, int &p, int &which) -> bool {
+    if (which == 0 && p != qblocks - 1 - p) {
+      which = 1;
+      return true;
+    }
+    n += (int)gridDim.x;
+    if (n >= total) return false;
+    decode(n, head, p);
+    which = 0;
+    return true;
+  };
+  int n = blockIdx.x, head, p, which = 0;
+  if (n >= total) return;
+  decode(n, head, p);
+  int n2 = n, head2 = head, p2 = p, which2 = which;
+  bool more = advance(n2, head2, p2, which2);
+  pipeattn::body<128, false>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+  asm volatile("s_barrier" ::: "memory");   // nobody reads this item's stages any more; the next item's first blocks have landed
+  while (more) {
+    n = n2; head = head2; p = p2; which = which2;
+    more = advance(n2, head2, p2, which2);
+    pipeattn::body<128, true>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+    asm volatile("s_barrier" ::: "memory");
   }
 }
 
