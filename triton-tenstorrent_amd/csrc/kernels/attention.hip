@@ -231,6 +231,21 @@ constexpr int BN = 64;
 //
 // WAVES = 4 (head dim 256): 128 queries per workgroup, one wavefront per SIMD with the whole register file
 // (O^T alone is 128 registers and Q 64 at that head dim), and all four wavefronts share the copies.
+// Issue priority of a wavefront over a block: 3 through the two MFMA phases, 1 through the softmax, 2 at the end of
+// the block, never the default 0.  Measured A/B in one process (causal / not causal TFLOP/s): head dim 256 (one
+// wavefront per SIMD) 575 -> 667 / 658 -> 766, and a constant priority of 3 does the same there, so what counts is
+// leaving priority 0; head dim 32 495 -> 513 / 650 -> 665; head dim 128 on ragged lengths 827 -> 838 / 1017 -> 1024;
+// head dim 64 is 0.5-1 % slower with any scheme tried and keeps the default.  The GEMM kernels do not react at all.
+template <int D> __device__ __forceinline__ void attn_phase_prio(int phase) {
+  if constexpr (D != 64) {
+    switch (phase) {
+    case 1: __builtin_amdgcn_s_setprio(1); break;
+    case 3: __builtin_amdgcn_s_setprio(2); break;
+    default: __builtin_amdgcn_s_setprio(3); break;
+    }
+  }
+}
+#define ATTN_SETPRIO(phase) attn_phase_prio<D>(phase)
 template <int D, bool RAGGED = false, int WAVES = 8>
 __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *lds1) {
   constexpr int BM = WAVES * 32;
@@ -357,6 +372,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     if (b + 1 < nblk) dma_block(b + 1, nxt);
     const int n0 = b * BN;
     if (!live || (a.causal && n0 > qw + 31)) continue; // outside the sequence, or wholly above this wavefront's diagonal
+    ATTN_SETPRIO(0);
     const bool both = !RAGGED || n0 + 32 < n_end;      // the block's second 32-key tile exists (wave-uniform)
 
     // ---- S^T = K . Q^T : two 32-key tiles ----
@@ -387,6 +403,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 0);
+    ATTN_SETPRIO(1);
     // ---- online softmax (per lane = per query; keys run over registers and the hi half) ----
     const bool on_band = a.causal && (n0 + BN - 1 > qw);
     float rmax = -__builtin_inff();
@@ -440,6 +457,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
     }
     l_i = l_i * alpha + l_ij;
     m_i = m_ij;
+    ATTN_SETPRIO(2);
     // ---- P^T fragments: 16-key step k4 uses registers 8*(k4&1).. of st[k4>>1] ----
     Frag pf[4];
 #pragma unroll
@@ -473,6 +491,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds0, uint8_t *
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, AHEAD, 1);
+    ATTN_SETPRIO(3);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   if (!live) return;

@@ -55,10 +55,11 @@ constexpr int BN = 64;        // keys per block
 constexpr int NST = 4;        // LDS stages
 constexpr int GK = 2, GV = 2; // fragments per read group
 constexpr float LAZY_T = 8.0f;
-// A wavefront's issue priority falls from 3 to 0 over each phase, a step every PRIO_STEP MFMAs: of the two
+// A wavefront's issue priority falls from 3 to 1 over each phase, a step every PRIO_STEP MFMAs: of the two
 // wavefronts of a SIMD the one that is behind then wins arbitration.  Left alone the older wavefront always wins: it
 // ran its phases in 1190 + 1020 cycles and waited 800 at the barrier for the other one's 1380 + 1560.
 constexpr int PRIO_STEP = 4, PRIO_TOP = 3;
+#define PIPE_PRIO_OF(step, steps) (PRIO_TOP - (step) * 2 / ((steps) - 1))   // 3, 3, 2, 1: never the default 0
 __device__ __forceinline__ void set_prio(int p) {   // s_setprio takes an immediate
   switch (p) {
   case 0: __builtin_amdgcn_s_setprio(0); break;
@@ -251,7 +252,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
       for (int i = 0; i < GK; ++i) kf[i] = kpre[i];
 #pragma unroll
       for (int i = 0; i < 2 * DK; ++i) {
-        if (i % PRIO_STEP == 0) set_prio(PRIO_TOP - (i / PRIO_STEP) * PRIO_TOP / (2 * DK / PRIO_STEP - 1));
+        if (i % PRIO_STEP == 0) set_prio(PIPE_PRIO_OF(i / PRIO_STEP, 2 * DK / PRIO_STEP));
         if (i % GK == 0 && i + GK < 2 * DK) {
 #pragma unroll
           for (int g = 0; g < GK; ++g) kf[(i + GK + g) % (2 * GK)] = rdK(nxt, i + GK + g);
@@ -290,7 +291,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 #pragma unroll
     for (int i = 0; i < 4 * DT; ++i) {
       const int k4 = i >> 2, t = i & 3;
-      if (i % PRIO_STEP == 0) set_prio(PRIO_TOP - (i / PRIO_STEP) * PRIO_TOP / (4 * DT / PRIO_STEP - 1));
+      if (i % PRIO_STEP == 0) set_prio(PIPE_PRIO_OF(i / PRIO_STEP, 4 * DT / PRIO_STEP));
       if (i % GV == 0 && i + GV < 4 * DT) {
 #pragma unroll
         for (int g = 0; g < GV; ++g) vf[(i + GV + g) % (2 * GV)] = rdV(cur, i + GV + g);
