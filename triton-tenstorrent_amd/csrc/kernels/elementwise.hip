@@ -414,10 +414,10 @@ EW_UNARY(log2, Log2Op, kVec)
 EW_UNARY(rsqrt, RsqrtOp, kVec)
 EW_UNARY(sqrt, SqrtOp, kVec)
 
-#define EW_BINARY(name, Op)                                                                               \
+#define EW_BINARY(name, Op, VEC)                                                                          \
   __global__ __launch_bounds__(kThreads) void ew_##name##_f32(const float *x, const float *y, float *out, \
                                                               uint32_t n) {                                \
-    binary_body<float, Op, kVec>(x, y, out, n);                                                               \
+    binary_body<float, Op, VEC>(x, y, out, n);                                                                \
   }                                                                                                        \
   __global__ __launch_bounds__(kThreads) void ew_##name##_f32_unaligned(const float *x, const float *y,   \
                                                                         float *out, uint32_t n) {          \
@@ -440,11 +440,13 @@ EW_BINARY_CONST(div, DivOp)
 EW_BINARY_CONST(max, MaxOp)
 EW_BINARY_CONST(min, MinOp)
 
-EW_BINARY(sub, SubOp)
-EW_BINARY(mul, MulOp)
-EW_BINARY(div, DivOp)
-EW_BINARY(max, MaxOp)
-EW_BINARY(min, MinOp)
+EW_BINARY(sub, SubOp, kVec)
+EW_BINARY(mul, MulOp, kVec)
+EW_BINARY(div, DivOp, kVec)
+// maximum / minimum carry a NaN and signed-zero rule (about six VALU operations per element): two vectors per lane,
+// as for sin and cos
+EW_BINARY(max, MaxOp, kVecHeavy)
+EW_BINARY(min, MinOp, kVecHeavy)
 
 #define EW_CAST(name, Op, IN, OUT)                                                                          \
   __global__ __launch_bounds__(kThreads) void name(const IN *x, OUT *out, uint32_t n) {                     \

@@ -160,7 +160,9 @@ int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_
   char name[48];
   snprintf(name, sizeof(name), "ew_%s_f32%s", names[op], al ? "" : "_unaligned");
   void *args[] = {&x, &y, &out, &n_eff};
-  return launch("elementwise", name, dim3(streaming_grid(n_eff, al)), dim3(kThreads), 0, stream, args, 4);
+  const bool heavy = op == TT_OP_MAXIMUM || op == TT_OP_MINIMUM;   // built with kVecHeavy vectors per lane
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al, heavy ? ewgeom::kVecHeavy : kUnroll)), dim3(kThreads), 0,
+                stream, args, 4);
 }
 
 int tt_binary_const_kernel(int32_t op, const void *x, float c, int32_t flip, void *out, int32_t n_elements,
