@@ -535,7 +535,6 @@ ATTN_TILE(64)
   }
 ATTN_RAGGED(32)
 ATTN_RAGGED(64)
-ATTN_RAGGED(128)
 
 // head dim 256: four wavefronts, 128 queries per workgroup
 #define ATTN_TILE4(name, D, RAGGED)                                                        \

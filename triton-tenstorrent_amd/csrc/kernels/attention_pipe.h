@@ -72,7 +72,13 @@ __device__ __forceinline__ void set_prio(int p) {   // s_setprio takes an immedi
 // PREFETCHED: blocks 0, 1, 2 of this item are already in stages 0, 1, 2 (the item before it fetched them with its
 // trailing copies).  next_head: the head of the item that follows in this workgroup (this item's own head when none
 // does): this item's trailing copies fetch that head's first key blocks.
-template <int D, bool PREFETCHED>
+//
+// RAGGED: N_CTX is a whole number of 32-query wavefront tiles but not of 256-query blocks.  A wavefront whose tile lies
+// past the end computes and stores nothing but keeps up with the barriers and its share of the copies; copies of rows
+// past the end fetch the last 32 rows instead; keys past the end get a score of -inf (under the causal mask the
+// diagonal block does that anyway); and the item's stream of blocks is padded to a multiple of four periods, so that
+// the next item's first blocks land in stages 0, 1, 2 as they do for whole blocks.
+template <int D, bool PREFETCHED, bool RAGGED = false>
 __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int head, const int qblk, const int next_head) {
   constexpr int BM = 256;
   constexpr int DK = D / 16, DT = D / 32, ROW = D * 2, CH = D / 8;
@@ -91,8 +97,12 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   const int my_q = qw + c32;
   const int64_t base = (int64_t)head * a.n_ctx;
   const float qk_scale = a.sm_scale * 1.44269504f;
-  const int nblk = a.causal ? (q0 + BM) / BN : a.n_ctx / BN;      // key blocks the workgroup streams (>= 4)
+  const bool live = !RAGGED || qw < a.n_ctx;                      // wave-uniform
+  const int kend = RAGGED ? (a.causal ? min(q0 + BM, a.n_ctx) : a.n_ctx) : 0;
+  const int nblk = RAGGED ? (kend + BN - 1) / BN : (a.causal ? (q0 + BM) / BN : a.n_ctx / BN);   // key blocks of this item
+  const int nstream = RAGGED ? (nblk + 3) & ~3 : nblk;            // periods the workgroup goes through (a multiple of 4)
   const int L = a.causal ? (qw + 31) / BN : nblk - 1;             // this wavefront's last block (the masked one when causal)
+  const int last_rows = a.n_ctx - 32;                             // RAGGED: first row of the last 32 that exist
 
   // ---- copies: 512 threads x 16 B = 8 KiB per instruction round, two rounds per K or V tile ----
   const int crow = tid >> 4, cpos = tid & 15;       // row within a 32-row round, chunk position
@@ -116,8 +126,11 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   // the last one is fetched from the last one again (a harmless refetch into a stage nobody reads any more), so
   // that every wavefront issues four copies per block period and the vmcnt waits are the same everywhere.
   auto dma_piece = [&](int blk, int stage_o, int r) {
-    const bool own = blk < nblk;
-    const int64_t row0 = (int64_t)(own ? blk : blk - nblk) * BN + (r & 1) * 32;
+    const bool own = blk < nstream;
+    // (RAGGED: periods nblk .. nstream-1 are padding and refetch the last block; any 32 rows that do not exist are
+    // fetched from the last 32 that do)
+    int64_t row0 = (int64_t)(own ? (RAGGED ? min(blk, nblk - 1) : blk) : blk - nstream) * BN + (r & 1) * 32;
+    if (RAGGED) row0 = min(row0, (int64_t)last_rows);
     if (r < 2) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, k_voff, lds + stage_o + (r & 1) * 8192);
     else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, v_voff, lds + VBASE + stage_o + (r & 1) * 8192);
   };
@@ -164,7 +177,8 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   // Q after the copies, so that the two round trips to memory overlap; the wait the compiler puts in front of the
   // first use of Q is for everything older as well, the copies included
   {
-    const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
+    // (RAGGED: a wavefront past the end loads the last row that exists and never uses it)
+    const uint16_t *qrow = a.q + (base + (RAGGED ? min(my_q, a.n_ctx - 1) : my_q)) * a.ldq;
 #pragma unroll
     for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
     // the loads land here: the compiler's own vmcnt bookkeeping does not see the copies issued from assembly
@@ -241,7 +255,9 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = j * BN + kt * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-          const float add = my_q >= key ? 0.0f : (key > qw + 31 ? -__builtin_inff() : -1.0e6f);
+          // (RAGGED, no causal mask: the block that ends past N_CTX; its keys past the end are not part of the product)
+          const float add = (RAGGED && !a.causal) ? (key >= a.n_ctx ? -__builtin_inff() : 0.0f)
+                                                  : (my_q >= key ? 0.0f : (key > qw + 31 ? -__builtin_inff() : -1.0e6f));
           sc[kt][r] = sc[kt][r] * qk_scale + add;
         }
     }
@@ -314,40 +330,46 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 
   const std::false_type F{};
   const std::true_type T{};
-  int j = 0;
-  for (; j + 4 <= L; j += 4) {       // stage offsets known at compile time, score registers alternating
-    period(j, 0, STG, 2 * STG, 3 * STG, s0, s1, F, F);
-    period(j + 1, STG, 2 * STG, 3 * STG, 0, s1, s0, F, F);
-    period(j + 2, 2 * STG, 3 * STG, 0, STG, s0, s1, F, F);
-    period(j + 3, 3 * STG, 0, STG, 2 * STG, s1, s0, F, F);
-  }
-  // what is left (at most three blocks and the last one) runs with the stage offsets in registers
-  int cur_o = 0;
+  int j = 0, cur_o = 0;
   auto nx = [&](int o) { return (o + STG) & (NST * STG - 1); };
-  const int rest = L - j;
-  if (rest & 1) {
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
-    s0[0] = s1[0];
-    s0[1] = s1[1];
+  if (live) {
+    for (; j + 4 <= L; j += 4) {       // stage offsets known at compile time, score registers alternating
+      period(j, 0, STG, 2 * STG, 3 * STG, s0, s1, F, F);
+      period(j + 1, STG, 2 * STG, 3 * STG, 0, s1, s0, F, F);
+      period(j + 2, 2 * STG, 3 * STG, 0, STG, s0, s1, F, F);
+      period(j + 3, 3 * STG, 0, STG, 2 * STG, s1, s0, F, F);
+    }
+    // what is left (at most three blocks and the last one) runs with the stage offsets in registers
+    const int rest = L - j;
+    if (rest & 1) {
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
+      s0[0] = s1[0];
+      s0[1] = s1[1];
+      cur_o = nx(cur_o);
+      ++j;
+    }
+    if (rest & 2) {
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
+      cur_o = nx(cur_o);
+      ++j;
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s1, s0, F, F);
+      cur_o = nx(cur_o);
+      ++j;
+    }
+    if (a.causal || (RAGGED && (a.n_ctx & (BN - 1)))) period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, T);
+    else period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, F);
     cur_o = nx(cur_o);
     ++j;
   }
-  if (rest & 2) {
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
-    cur_o = nx(cur_o);
-    ++j;
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s1, s0, F, F);
-    cur_o = nx(cur_o);
-    ++j;
-  }
-  if (a.causal) period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, T);
-  else period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, F);
-  for (++j; j < nblk; ++j) {   // done: keep up with the others' barriers and this wavefront's share of the copies
-    cur_o = nx(cur_o);
+  // done (or, RAGGED, never started): keep up with the others' barriers and this wavefront's share of the copies;
+  // cur_o is the stage of block j
+  for (; j < nstream; ++j) {
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     dma_block(j + 3, nx(nx(nx(cur_o))));
+    cur_o = nx(cur_o);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the trailing refetches land before the stages are reused or released
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the trailing copies land before the stages are reused or released
+  if (!live) return;
   // ---- epilogue ----
   if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
   uint16_t *orow = a.o + (base + my_q) * a.ldo;
@@ -366,15 +388,13 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 
 } // namespace pipeattn
 
-extern "C" {
-
 // Persistent: gridDim.x workgroups (one per CU when there is that much work) walk the (head, pair of query blocks)
 // items in the order the dispatcher would have dealt one-item workgroups: item n of workgroup g is g + n * gridDim.x,
 // re-dealt so that an XCD's workgroups hold neighbouring items of the same heads.  A workgroup's items run back to
 // back: each one's trailing copies fetch the first key blocks of the next.
-__global__ __launch_bounds__(512) void attn_tile_d128(AttnArgs a) {
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 128 * 2];
-  const int qblocks = a.rows / 256;
+template <bool RAGGED>
+__device__ __forceinline__ void attn_pipe_d128(const AttnArgs &a, uint8_t *lds) {
+  const int qblocks = RAGGED ? (a.rows + 255) / 256 : a.rows / 256;
   const int per_head = (qblocks + 1) / 2, total = per_head * a.heads;
   auto decode = [&](int n, int &head, int &p) {
     int id = n;
@@ -399,14 +419,27 @@ __global__ __launch_bounds__(512) void attn_tile_d128(AttnArgs a) {
   decode(n, head, p);
   int n2 = n, head2 = head, p2 = p, which2 = which;
   bool more = advance(n2, head2, p2, which2);
-  pipeattn::body<128, false>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+  pipeattn::body<128, false, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
   asm volatile("s_barrier" ::: "memory");   // nobody reads this item's stages any more; the next item's first blocks have landed
   while (more) {
     n = n2; head = head2; p = p2; which = which2;
     more = advance(n2, head2, p2, which2);
-    pipeattn::body<128, true>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+    pipeattn::body<128, true, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
     asm volatile("s_barrier" ::: "memory");
   }
+}
+
+extern "C" {
+
+__global__ __launch_bounds__(512) void attn_tile_d128(AttnArgs a) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 128 * 2];
+  attn_pipe_d128<false>(a, lds);
+}
+
+// the same for sequence lengths that are whole 32-query tiles but not whole 256-query blocks
+__global__ __launch_bounds__(512) void attn_ragged_d128(AttnArgs a) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 128 * 2];
+  attn_pipe_d128<true>(a, lds);
 }
 
 } // extern "C"
