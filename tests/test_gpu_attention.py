@@ -248,9 +248,10 @@ def test_causal_mask_is_the_sources_at_block_m_32(S, D, kernel):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("Z,H,S", [(2, 32, 2304), (1, 40, 3328), (3, 3, 768), (2, 32, 2272), (1, 33, 4000), (5, 8, 1056)])
-def test_items_chained_inside_a_workgroup(causal, Z, H, S):
-    """The head dim 128 kernel walks (head, pair of query blocks) items on a persistent grid and lets each item's last
+@pytest.mark.parametrize("Z,H,S,D", [(2, 32, 2304, 128), (1, 40, 3328, 128), (3, 3, 768, 128), (2, 32, 2272, 128),
+                                     (1, 33, 4000, 128), (5, 8, 1056, 128), (2, 32, 2304, 64), (3, 11, 3328, 64), (1, 5, 512, 64)])
+def test_items_chained_inside_a_workgroup(causal, Z, H, S, D):
+    """The head dim 128 and 64 kernels walk (head, pair of query blocks) items on a persistent grid and lets each item's last
     copies fetch the first key blocks of the next one, which may belong to another head.  Shapes with more items
     than CUs (288 and 280 against 256), an odd number of query blocks (9, 13: the middle block is an item on its own,
     so items of one and of two blocks alternate), a head count that is not a multiple of 8, and lengths that are not
@@ -258,14 +259,13 @@ def test_items_chained_inside_a_workgroup(causal, Z, H, S):
     an item is padded to whole turns of the stage ring); every row of sampled
     heads and of the heads where a workgroup changes head, against float64."""
     from triton_tenstorrent_amd import runtime as rt
-    D = 128
     g = torch.Generator(device="cuda").manual_seed(Z * 1000 + S)
     q, k, v = (torch.randn(Z, H, S, D, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
     # every head gets its own offset in V, so that output rows computed from another head's keys or values show
     v = (v.float() + torch.arange(Z * H, device="cuda").view(Z, H, 1, 1).float() * 0.25).to(torch.bfloat16)
     sm = D ** -0.5
     o, M = K.attention(q, k, v, causal, sm, return_lse=True)
-    assert rt.last_kernel_name() == ("attn_tile_d128" if S % 256 == 0 else "attn_ragged_d128")
+    assert rt.last_kernel_name() == (f"attn_tile_d{D}" if S % 256 == 0 else f"attn_ragged_d{D}")
     heads = sorted({0, 1, Z * H // 2, Z * H - 2, Z * H - 1, 7, 8} & set(range(Z * H)))
     rows = torch.arange(S, device="cuda")
     for hh in heads:

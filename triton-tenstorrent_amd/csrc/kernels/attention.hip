@@ -524,7 +524,6 @@ extern "C" {
     fastattn::body<D>(a, lds0, lds1);                                                      \
   }
 ATTN_TILE(32)
-ATTN_TILE(64)
 // head dim 128 on whole 256-query blocks: attention_pipe.h
 
 #define ATTN_RAGGED(D)                                                                     \

@@ -83,7 +83,12 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   constexpr int BM = 256;
   constexpr int DK = D / 16, DT = D / 32, ROW = D * 2, CH = D / 8;
   constexpr int TILE = BN * ROW, STG = TILE, VBASE = NST * TILE;   // stage s: K at s*TILE, V at VBASE + s*TILE
-  static_assert(D == 128, "the LDS swizzles below are those of 256-byte rows");
+  constexpr int RPB = 256 / ROW;               // rows per 256 bytes of LDS: the K swizzle advances every RPB rows
+  constexpr int RPP = 8192 / ROW;              // rows that one copy instruction of the workgroup covers (512 x 16 B)
+  constexpr int PPT = BN / RPP;                // such pieces per K or V tile
+  constexpr int SLOTS = D / 8;                 // MFMAs per phase: 2*DK = 4*DT
+  constexpr int SPS = 16 / SLOTS;              // softmax work items per MFMA slot
+  static_assert(D == 128 || (D == 64 && !RAGGED), "LDS swizzles exist for 256- and 128-byte rows; ragged lengths at 256 only");
   static_assert((NST & (NST - 1)) == 0, "the stage ring wraps with a mask");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -105,9 +110,9 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   const int last_rows = a.n_ctx - 32;                             // RAGGED: first row of the last 32 that exist
 
   // ---- copies: 512 threads x 16 B = 8 KiB per instruction round, two rounds per K or V tile ----
-  const int crow = tid >> 4, cpos = tid & 15;       // row within a 32-row round, chunk position
-  const int k_chunk = cpos ^ (crow & 15);           // K: logical chunk c of row r sits at c ^ (r & 15)
-  const int v_chunk = cpos ^ ((crow & 3) << 2);     // V: at c ^ ((r & 3) << 2)
+  const int crow = tid / CH, cpos = tid % CH;       // row within a round of RPP rows, chunk position
+  const int k_chunk = cpos ^ ((crow / RPB) & (CH - 1));                       // K: logical chunk c of row r sits at c ^ ((r / RPB) & (CH-1))
+  const int v_chunk = cpos ^ ((D == 128 ? (crow & 3) : ((crow >> 1) & 1)) << 2);   // V: at c ^ ((r & 3) << 2), 128-byte rows: c ^ (((r >> 1) & 1) << 2)
   const uint32_t k_voff = (uint32_t)(((int64_t)crow * a.ldk + k_chunk * 8) * 2);
   const uint32_t v_voff = (uint32_t)(((int64_t)crow * a.ldv + v_chunk * 8) * 2);
   const uint8_t *kg = (const uint8_t *)(a.k + base * a.ldk);
@@ -129,25 +134,26 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
     const bool own = blk < nstream;
     // (RAGGED: periods nblk .. nstream-1 are padding and refetch the last block; any 32 rows that do not exist are
     // fetched from the last 32 that do)
-    int64_t row0 = (int64_t)(own ? (RAGGED ? min(blk, nblk - 1) : blk) : blk - nstream) * BN + (r & 1) * 32;
+    int64_t row0 = (int64_t)(own ? (RAGGED ? min(blk, nblk - 1) : blk) : blk - nstream) * BN + (r % PPT) * RPP;
     if (RAGGED) row0 = min(row0, (int64_t)last_rows);
-    if (r < 2) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, k_voff, lds + stage_o + (r & 1) * 8192);
-    else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, v_voff, lds + VBASE + stage_o + (r & 1) * 8192);
+    if (r < PPT) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, k_voff, lds + stage_o + (r % PPT) * 8192);
+    else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, v_voff, lds + VBASE + stage_o + (r % PPT) * 8192);
   };
   auto dma_block = [&](int blk, int stage_o) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) dma_piece(blk, stage_o, r);
+    for (int r = 0; r < 2 * PPT; ++r) dma_piece(blk, stage_o, r);
   };
 
   // ---- fragment addresses ----
   int k_off[DK];                 // K (A operand of S^T): lane = key row c32 of a 32-key tile, chunk 2s+hi of its row
 #pragma unroll
-  for (int s = 0; s < DK; ++s) k_off[s] = c32 * ROW + (((2 * s + hi) ^ (c32 & (CH - 1))) << 4);
+  for (int s = 0; s < DK; ++s) k_off[s] = c32 * ROW + (((2 * s + hi) ^ ((c32 / RPB) & (CH - 1))) << 4);
   const int G4 = lane >> 4, i16 = lane & 15, qd = i16 >> 2;
   const int v_cc = (G4 & 1) * 2 + ((i16 >> 1) & 1);
   int v_off[DT];                 // V^T (A operand of O^T) through transposing reads: key row hi*4+qd (+ k4*16 + h2*8)
 #pragma unroll
-  for (int t = 0; t < DT; ++t) v_off[t] = VBASE + (hi * 4 + qd) * ROW + (((t * 4 + v_cc) ^ (qd << 2)) << 4) + ((i16 & 1) << 3);
+  for (int t = 0; t < DT; ++t)
+    v_off[t] = VBASE + (hi * 4 + qd) * ROW + (((t * 4 + v_cc) ^ ((D == 128 ? qd : ((qd >> 1) & 1)) << 2)) << 4) + ((i16 & 1) << 3);
 
   union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; uint32_t w[4]; };
   Frag qf[DK];
@@ -161,7 +167,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   };
   auto rdV = [&](const uint8_t *stage, int i) -> bf16x8 {   // fragment i: 16-key step i>>2, d-tile i&3
     Frag f;
-    const int k4 = i >> 2, t = i & 3;
+    const int k4 = i / DT, t = i % DT;
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2)
       f.h[h2] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(stage + v_off[t] + (k4 * 16 + h2 * 8) * ROW));
@@ -278,11 +284,20 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 #pragma unroll
           for (int g = 0; g < GV; ++g) vpre[g] = rdV(cur, g);
         }
-        if (i < 4) max_part(i);
-        if (i == 4) stats();
-        if (i >= 6) exp_part(i - 6);          // 10 of the 16 pairs
+        // the softmax of block j in 16 work items, SPS of them per MFMA: four partial maxima, the statistics (and
+        // the rescale, when there is one), a gap, then 10 of the 16 pairs of exponentials
+        bool with_stats = false;
+#pragma unroll
+        for (int w = i * SPS; w < (i + 1) * SPS; ++w) {
+          if (w < 4) max_part(w);
+          if (w == 4) {
+            stats();
+            with_stats = true;
+          }
+          if (w >= 6) exp_part(w - 6);
+        }
         PIPE_FENCE();
-        if (i == 4) {
+        if (with_stats) {
           rescale();
           PIPE_FENCE();
         }
@@ -306,23 +321,26 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
     for (int i = 0; i < GV; ++i) vf[i] = vpre[i];
 #pragma unroll
     for (int i = 0; i < 4 * DT; ++i) {
-      const int k4 = i >> 2, t = i & 3;
+      const int k4 = i / DT, t = i % DT;
       if (i % PRIO_STEP == 0) set_prio(PIPE_PRIO_OF(i / PRIO_STEP, 4 * DT / PRIO_STEP));
       if (i % GV == 0 && i + GV < 4 * DT) {
 #pragma unroll
         for (int g = 0; g < GV; ++g) vf[(i + GV + g) % (2 * GV)] = rdV(cur, i + GV + g);
       }
       acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i % (2 * GV)], pfrag(k4), acc[t], 0, 0, 0);
-      if ((i & 3) == 1) dma_piece(j + 3, free_o, i >> 2);
+      if (i % (SLOTS / (2 * PPT)) == 1) dma_piece(j + 3, free_o, i / (SLOTS / (2 * PPT)));
       if (!LAST && i == 4 * DT - 4) {
 #pragma unroll
         for (int g = 0; g < GK; ++g) kpre[g] = rdK(lds + nn_o, g);
       }
-      if (i < 6) exp_part(10 + i);            // pairs 10..15 are needed from i = 8 on
-      if (i == 6) {
-        l_ij = xor32_sum(l_ij);
-        l_i = l_i * alpha + l_ij;
-        m_i = m_ij;
+#pragma unroll
+      for (int w = i * SPS; w < (i + 1) * SPS; ++w) {
+        if (w < 6) exp_part(10 + w);          // pairs 10..15 are needed from the second half of the phase on
+        if (w == 6) {
+          l_ij = xor32_sum(l_ij);
+          l_i = l_i * alpha + l_ij;
+          m_i = m_ij;
+        }
       }
       PIPE_FENCE();
     }
@@ -392,8 +410,8 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 // items in the order the dispatcher would have dealt one-item workgroups: item n of workgroup g is g + n * gridDim.x,
 // re-dealt so that an XCD's workgroups hold neighbouring items of the same heads.  A workgroup's items run back to
 // back: each one's trailing copies fetch the first key blocks of the next.
-template <bool RAGGED>
-__device__ __forceinline__ void attn_pipe_d128(const AttnArgs &a, uint8_t *lds) {
+template <int D, bool RAGGED>
+__device__ __forceinline__ void attn_pipe(const AttnArgs &a, uint8_t *lds) {
   const int qblocks = RAGGED ? (a.rows + 255) / 256 : a.rows / 256;
   const int per_head = (qblocks + 1) / 2, total = per_head * a.heads;
   auto decode = [&](int n, int &head, int &p) {
@@ -419,12 +437,12 @@ __device__ __forceinline__ void attn_pipe_d128(const AttnArgs &a, uint8_t *lds) 
   decode(n, head, p);
   int n2 = n, head2 = head, p2 = p, which2 = which;
   bool more = advance(n2, head2, p2, which2);
-  pipeattn::body<128, false, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+  pipeattn::body<D, false, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
   asm volatile("s_barrier" ::: "memory");   // nobody reads this item's stages any more; the next item's first blocks have landed
   while (more) {
     n = n2; head = head2; p = p2; which = which2;
     more = advance(n2, head2, p2, which2);
-    pipeattn::body<128, true, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+    pipeattn::body<D, true, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
     asm volatile("s_barrier" ::: "memory");
   }
 }
@@ -433,13 +451,19 @@ extern "C" {
 
 __global__ __launch_bounds__(512) void attn_tile_d128(AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 128 * 2];
-  attn_pipe_d128<false>(a, lds);
+  attn_pipe<128, false>(a, lds);
 }
 
 // the same for sequence lengths that are whole 32-query tiles but not whole 256-query blocks
 __global__ __launch_bounds__(512) void attn_ragged_d128(AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 128 * 2];
-  attn_pipe_d128<true>(a, lds);
+  attn_pipe<128, true>(a, lds);
+}
+
+// head dim 64 on whole 256-query blocks: the same pipeline with 128-byte rows (8 + 8 MFMAs per block period)
+__global__ __launch_bounds__(512) void attn_tile_d64(AttnArgs a) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 64 * 2];
+  attn_pipe<64, false>(a, lds);
 }
 
 } // extern "C"
