@@ -1,5 +1,6 @@
-// attn_tile_d128: _attn_fwd (examples/fused-attn/06-fused-attention.py:33-90, 143-215) at head dim 128 on whole
-// 256-query blocks, the configuration the fused-attention benchmark is quoted on.
+// attn_tile_d128, attn_ragged_d128, attn_tile_d64: _attn_fwd (examples/fused-attn/06-fused-attention.py:33-90,
+// 143-215) at head dim 128 (whole 256-query blocks, the configuration the fused-attention benchmark is quoted on, and
+// any length that is a whole number of 32-query tiles) and at head dim 64 (whole blocks).
 //
 // Same work layout and numerics as the kernels in attention.hip (one wavefront = 32 queries, both products
 // transposed, K/V blocks of 64 keys in LDS), with the block loop written as a software pipeline:
