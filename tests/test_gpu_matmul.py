@@ -78,11 +78,12 @@ def test_matmul_ragged_shapes_strided_views_and_sentinel():
     assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
 
 
-# Shapes that are whole 32-deep K steps and 8-column chunks but not whole 256x256x128 macro tiles take the fast
-# kernel's clamping variant: rows / chunks past the edge are fetched from inside the matrix, K is padded with
-# steps of zeros, stores are clipped.
+# Shapes in whole 8-element chunks of N and K that are not whole 256x256x128 macro tiles take the fast kernel's
+# clamping variant: rows / chunks past the edge are fetched from inside the matrix, a last 32-deep K step that ends
+# past K is cleared from K on, K is padded with steps of zeros, stores are clipped.
 RAGGED_SHAPES = [(33, 8, 32), (256, 256, 32), (260, 264, 160), (511, 520, 96), (1000, 1000, 992), (257, 1032, 4128),
-                 (4000, 4096, 1024)]
+                 (4000, 4096, 1024), (33, 8, 8), (256, 256, 40), (300, 328, 72), (1000, 1000, 1000), (257, 1032, 4104),
+                 (4000, 4096, 1048)]
 
 
 @pytest.mark.parametrize("M,N,K_", RAGGED_SHAPES)
@@ -102,13 +103,13 @@ def test_matmul_ragged_fast_path(M, N, K_, dtype):
 
 
 def test_matmul_ragged_fast_path_random_shapes_exact():
-    # a seeded sweep over shapes (M anything, N in steps of 8, K in steps of 32), small integers: bit for bit, with
+    # a seeded sweep over shapes (M anything, N and K in steps of 8), small integers: bit for bit, with
     # a sentinel frame around C and NaN frames around A and B
     rng = np.random.default_rng(2025)
-    for case in range(24):
+    for case in range(32):
         M = int(rng.integers(1, 700))
         N = 8 * int(rng.integers(1, 90))
-        K_ = 32 * int(rng.integers(1, 12))
+        K_ = 8 * int(rng.integers(1, 48))
         dtype = torch.bfloat16 if case % 2 else torch.float16
         g = torch.Generator().manual_seed(case)
         abuf = torch.full((M + 2, K_ + 8), float("nan"), dtype=dtype)
@@ -126,6 +127,25 @@ def test_matmul_ragged_fast_path_random_shapes_exact():
         want = abuf[:M, :K_].float() @ bbuf[:K_, :N].float()            # exact in fp32, and in the half types up to 2^8
         assert torch.equal(c.float().cpu(), want.to(dtype).float()), (M, N, K_)
         assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5), (M, N, K_)
+
+
+def test_matmul_ragged_fast_path_every_k_in_steps_of_eight():
+    # K = 8 .. 328: every length of the last step (8, 16, 24, 32) at every depth of the copy ring's fill (one to ten
+    # steps); small integers, bit for bit.  The operands end where their buffers end, next to NaN rows of the
+    # neighbouring allocation-sized frame: a chunk fetched past K would bring NaN (A) or the next row in
+    M, N = 261, 264
+    for K_ in range(8, 336, 8):
+        g = torch.Generator().manual_seed(K_)
+        abuf = torch.full((M + 1, K_), float("nan"), dtype=torch.bfloat16)
+        bbuf = torch.full((K_ + 1, N), float("nan"), dtype=torch.bfloat16)
+        abuf[:M] = torch.randint(-3, 4, (M, K_), generator=g).to(torch.bfloat16)
+        bbuf[:K_] = torch.randint(-3, 4, (K_, N), generator=g).to(torch.bfloat16)
+        # column K-1 large: a chunk of A cleared one element too early, or a row of B dropped, shows at once
+        abuf[:M, K_ - 1] = 64
+        c = K.matmul_tma(abuf.cuda()[:M], bbuf.cuda()[:K_])
+        assert rt.last_kernel_name() == "gemm_ragged_bf16_epi0", K_
+        want = (abuf[:M].float() @ bbuf[:K_].float()).to(torch.bfloat16)
+        assert torch.equal(c.cpu(), want), K_
 
 
 def test_matmul_ragged_fast_path_exact_and_with_wild_values_next_door():

@@ -163,7 +163,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
   // real M and N (the padding of C is never written, as under the reference's store mask).
   const int Mf = TILED ? (g.M + 31) / 32 * 32 : g.M, Nf = TILED ? (g.N + 31) / 32 * 32 : g.N;   // fetchable extent
-  const int Kf = TILED ? (g.K + 31) / 32 * 32 : g.K;
+  const int Kf = (TILED || RAGGED) ? (g.K + 31) / 32 * 32 : g.K;   // K in whole steps (row-major RAGGED: the last step may end past K)
   using X = MFMA<IN_DT>;
   using vec = typename X::vec;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -259,14 +259,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                  : "memory", "m0");
   };
 
-  // TILED && RAGGED with K not a multiple of 32: the last tile of every K row of tiles holds columns (A) and rows
-  // (B) past K.  The source masks them to zero whatever the buffers hold there
+  // RAGGED with K not a multiple of 32: the last step of every tile holds columns (A) and rows (B) past K:
+  // whatever a tile-major buffer holds there, or what the redirected copies of row-major operands brought in
+  // (dma_single).  The source masks them to zero
   // (03-matrix-multiplication.py:340-342, 359-361), so a thread clears, in the stage that received the last data
   // step, the part of its OWN sixteen bytes of each slab that lies past K, once its copies have landed and before
   // the barrier that opens the stage for reading.
-  const int k_tail = (TILED && RAGGED) ? g.K & 31 : 0;            // valid k of the last data step, 0 = all 32
+  const int k_tail = RAGGED ? g.K & 31 : 0;                       // valid k of the last data step, 0 = all 32 (row-major: a multiple of 8)
   auto clear_past_k = [&](uint8_t *stage) {
-    if constexpr (TILED && RAGGED) {
+    if constexpr (RAGGED) {
       typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
       // A: this thread's chunk holds k = 8*a_chunk .. 8*a_chunk + 7 of one row, two per 32-bit word
       const int ka = a_chunk * 8;
@@ -340,12 +341,19 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         dma_one(b_cur + (int64_t)k * b_kstep + (i - MB) * b_slab, vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
     } else if constexpr (RAGGED) {
       const bool zero = k >= nk_real;                         // a padding step: both operands are zeros
+      // row-major operands, last data step of a K that is not a whole number of steps: the 16-byte chunks of A past
+      // K belong to the next row (past the buffer, for the last row) and the rows of B past K do not exist.  They
+      // are fetched from the step's first chunk / first slab instead, which exist, and cleared once they have landed
+      // (clear_past_k).  Tile-major buffers are padded to whole tiles and need no redirection.
+      const bool tail = !TILED && k_tail != 0 && k == nk_real - 1;
       const Voffs &vo = over ? vo_nxt : vo_cur;
       if (i < MB) {
         const uint8_t *ap = zero ? zero_page : (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
-        dma_one(ap, zero ? z_voff : vo.a[i], stage + i * 4096);
+        const uint32_t av = (tail && a_chunk * 8 >= k_tail) ? vo.a[i] - (uint32_t)a_chunk * 16 : vo.a[i];
+        dma_one(ap, zero ? z_voff : av, stage + i * 4096);
       } else {
-        const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - MB) * b_slab;
+        const int slab = (tail && (i - MB) * 8 >= k_tail) ? 0 : i - MB;
+        const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + slab * b_slab;
         dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - MB) * 4096);
       }
     } else if (i < MB) {
@@ -386,7 +394,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       // All of this wave's reads of stage I have returned, and so has its share of the
       // copy into stage I+1 (the 16 younger copies may still be in flight).  After the
       // barrier that holds for every wave: I+1 may be read, I may be overwritten.
-      if constexpr (TILED && RAGGED && !decltype(inner_)::value) {
+      if constexpr (RAGGED && !decltype(inner_)::value) {
         if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
           asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
           clear_past_k(nxt);
@@ -420,7 +428,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         mm(f0, n);
         FENCE();
       }
-      if constexpr (TILED && RAGGED && !decltype(inner_)::value) {
+      if constexpr (RAGGED && !decltype(inner_)::value) {
         if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
           asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
           clear_past_k(nxt);
@@ -458,7 +466,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     for (int i = 0; i < (s == R - 1 ? MB : MB + 4); ++i) dma_single(s, ring.s[s], i, std::false_type{});
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
   // everything issued but step 0's own MB + 4 copies may still be in flight: 2 * (MB + 4) + MB
-  if (TILED && RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
+  if (RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     clear_past_k(ring.s[0]);
   }
@@ -480,7 +488,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
     int k = 0;
     // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
-    for (; k + 2 * R <= nk_real; k += R) {
+    // (row-major operands whose last step ends past K: that step's copies need the redirection above, so it stays
+    // out of these turns)
+    const int nk_inner = nk_real - ((!TILED && k_tail) ? 1 : 0);
+    for (; k + 2 * R <= nk_inner; k += R) {
       step(std::integral_constant<int, 0>{}, k, std::true_type{});
       step(std::integral_constant<int, 1>{}, k + 1, std::true_type{});
       step(std::integral_constant<int, 2>{}, k + 2, std::true_type{});

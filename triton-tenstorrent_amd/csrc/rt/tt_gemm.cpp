@@ -122,8 +122,9 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   const bool fast_align = aligned16(g.a) && aligned16(g.b) && aligned16(g.c) && g.lda % 8 == 0 &&
                           g.ldb % 8 == 0 && g.ldc % 8 == 0;
   // The same kernel with clamped fetches, zero-padded K steps and clipped stores takes every other shape
-  // whose rows can be fetched in 16-byte pieces and whose K is a whole number of 32-deep steps.
-  const bool ragged_shape = !fast_shape && N % 8 == 0 && K % 32 == 0 && g.lda < (1 << 23) && g.ldb < (1 << 23);
+  // whose rows can be fetched in 16-byte pieces (N and K multiples of 8; a last K step that ends past K has its
+  // copies redirected into the matrix and the surplus cleared in shared memory).
+  const bool ragged_shape = !fast_shape && N % 8 == 0 && K % 8 == 0 && g.lda < (1 << 23) && g.ldb < (1 << 23);
   if (full_grid && half_io && (fast_shape || ragged_shape) && fast_align && !nan_shows && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     char fast_name[64];
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
