@@ -34,11 +34,12 @@
 // contiguous: ds_read_b64_tr_b16 transposes a 4x16 block of 16-bit values
 // across each group of 16 lanes on the way out of LDS.
 //
-// RAGGED variant (M any, N a multiple of 8, K a multiple of 32): same kernel, three differences.  Rows of A
+// RAGGED variant (M any, N and K multiples of 8): same kernel, three differences.  Rows of A
 // beyond M and 16-byte column chunks of B beyond N are fetched from the last valid row / chunk instead (their
 // products land in parts of the macro tile that are never stored); K is padded to whole turns of the ring
 // with steps whose A and B slabs are copied from a page of zeros (exact: 0 * 0 accumulates nothing, whatever
-// the real operands hold); and the stores are clipped at M and N.  The MFMA stream has no branch in it.
+// the real operands hold; a last step that ends past K is cleared from K on once it has landed); and the stores
+// are clipped at M and N.  The MFMA stream has no branch in it.
 #pragma once
 #include <type_traits>
 

@@ -161,6 +161,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     }
   };
 
+  auto use_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" ::"a"(acc[i][j]));
+  };
   // One step (K += 64) on ring stage I: 16 MFMAs on `c` (read from stage I during the previous
   // step), the next stage's fragments into `p`, and the refill of stage I itself with step k+R.
   auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_) {
@@ -198,6 +204,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
         FENCE();
       }
     }
+    // Outside the peeled turns nothing reads the accumulators before the epilogue, and an MFMA is a pure function
+    // to the compiler: it sinks all 64 of a turn past the turn's barriers, down to the epilogue, keeps four steps
+    // of fragments alive for that and spills them (each reload is a memory operation whose wait drains the copies
+    // in flight: such a turn then takes four times its time).  A use of every accumulator here keeps the MFMAs
+    // in the step they belong to.
+    if constexpr (!decltype(inner_)::value) use_acc();
   };
 
   int t = blockIdx.x;
