@@ -6,33 +6,41 @@
 // in the result (up to fp32 summation order).
 //
 // One workgroup (4 wavefronts, 2x2) computes a 256x256 macro tile.  Each
-// wavefront owns 128x128 of it: 4x4 v_mfma_f32_32x32x16 accumulators (256
+// wavefront owns 128x128 of it: 8x8 v_mfma_f32_16x16x32 accumulators (256
 // registers), hence one wavefront per SIMD.  The grid is persistent, one
 // workgroup per CU, striding over the macro tiles in an XCD-aware order.
+//
+// Why the 16x16x32 shape and not 32x32x16: the part is power-limited under this kernel, and per flop the
+// smaller tile with the deeper dot product costs less energy (an accumulator is read and written once per 32
+// multiply-adds instead of once per 16).  A loop of nothing but MFMAs on random operands sustains 1990 TFLOP/s
+// with it against 1735 with 32x32x16 (2440 with all-zero operands, either shape); this kernel went from 1343
+// to 1470 on 8192^3 in one process.  Fragment bytes read from LDS per step are the same for both shapes.
 //
 // K is walked in steps of 32 through a ring of four LDS stages (A 256x32 +
 // B 32x256 = 32 KiB per stage).  Data goes global -> LDS directly
 // (global_load_lds_dwordx4, no register staging) three steps ahead of its use,
 // and the ring runs on across tile boundaries, so the first steps of the next
 // tile are already in flight while the current tile's epilogue stores C.  LDS ->
-// registers runs one 16-deep sub-step ahead of the MFMAs that consume it.  A
-// single wavefront thus keeps its matrix pipe fed without a second one to hide
-// behind: every stall that matters (HBM/L2 latency, LDS latency) is covered by
-// distance in the software pipeline.
+// registers runs one step ahead of the MFMAs that consume it (two full sets of
+// fragments).  A single wavefront thus keeps its matrix pipe fed without a second
+// one to hide behind: every stall that matters (HBM/L2 latency, LDS latency) is
+// covered by distance in the software pipeline.
 //
 // LDS layout per stage (16-byte chunks, XOR-swizzled so that the row-wise A
 // reads and the transposing B reads are both bank-conflict free):
 //   A: row m = 64 B = 4 chunks;   logical chunk c sits at c ^ ((m>>2)&3)
-//   B: row k = 512 B = 32 chunks; logical chunk c sits at c ^ ((k&3)<<2)
+//   B: row k = 512 B = 32 chunks; logical chunk c sits at c ^ (((k&3)<<2) | (((k>>3)&1)<<1));
+//      the k rows are dealt to the four 4 KiB slabs as {0-3, 8-11}, {4-7, 12-15}, {16-19, 24-27}, {20-23, 28-31}
 // A direct-to-LDS load writes lane l's 16 bytes at (wave-uniform base) + 16*l,
 // so thread t owns byte 16*t of every 4 KiB slab and the swizzle is applied to
 // the global address it fetches.
 //
 // The product is formed transposed, acc = mfma(Bfrag, Afrag): a result lane then
 // holds 4 consecutive n of one m, so epilogue stores and bias loads are 8 bytes
-// wide.  B fragments need k along the lane's registers while memory has n
-// contiguous: ds_read_b64_tr_b16 transposes a 4x16 block of 16-bit values
-// across each group of 16 lanes on the way out of LDS.
+// wide (16 after an exchange between neighbouring lane groups).  B fragments need
+// k along the lane's registers while memory has n contiguous: ds_read_b64_tr_b16
+// transposes a 4x16 block of 16-bit values across each group of 16 lanes on the
+// way out of LDS.
 //
 // RAGGED variant (M any, N and K multiples of 8): same kernel, three differences.  Rows of A
 // beyond M and 16-byte column chunks of B beyond N are fetched from the last valid row / chunk instead (their
@@ -63,16 +71,20 @@ typedef __attribute__((address_space(3))) void lds_void;
 typedef __attribute__((address_space(1))) const void global_void;
 
 template <int IN_DT> struct MFMA;
+// Written as assembly with the accumulator tied to an AGPR: given the builtin, the compiler moves some of the 64
+// four-register accumulators of a wavefront through VGPRs around every MFMA (copies and the wait states they need
+// inside the K loop).  Each accumulator is touched once per step, far from any hazard distance; the epilogue waits
+// out the last MFMAs before it reads (see there).
 template <> struct MFMA<DT_BF16> {
   typedef bf16x8 vec;
-  static __device__ __forceinline__ f32x16 run(vec a, vec b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
 };
 template <> struct MFMA<DT_F16> {
   typedef f16x8 vec;
-  static __device__ __forceinline__ f32x16 run(vec a, vec b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
 };
 
@@ -151,8 +163,8 @@ struct Ring {
 // between slabs and between K steps.  LDS layout, fragments and MFMA schedule are the same.
 //
 // MB: 32-row blocks of C per wavefront.  4 is the 256x256 macro tile described above.  With 2 a workgroup
-// computes a 128x256 HALF of a macro tile (each wavefront 64x128: 2x4 accumulators, two A slabs and six
-// copies per step, eight MFMAs per sub-step), used for the tail of the persistent loop: when the macro
+// computes a 128x256 HALF of a macro tile (each wavefront 64x128: 4x8 accumulators, two A slabs and six
+// copies per step, 32 MFMAs per step), used for the tail of the persistent loop: when the macro
 // tiles left over after the last whole round of the grid would keep at most half of the workgroups busy,
 // the kernel runs body<MB=4> over the whole rounds and then body<MB=2> over the halves of the tail tiles,
 // two workgroups per tile, instead of leaving half of the chip idle for a whole tile's time.  (RAGGED: a
@@ -181,70 +193,76 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // A slab i (64 rows): row = i*64 + (t>>2), chunk position t&3 holds logical chunk (t&3)^((row>>2)&3)
   const int a_row = tid >> 2;
   const int a_chunk = (tid & 3) ^ ((a_row >> 2) & 3);
-  // B slab i (8 k-rows): k = i*8 + (t>>5), chunk position t&31 holds logical chunk (t&31)^((k&3)<<2)
-  const int b_k = tid >> 5;
-  const int b_chunk = (tid & 31) ^ ((b_k & 3) << 2);
+  // B slab i (8 rows of 512 B): row t>>5 of the slab holds k = b_row0(i) + b_kk, b_row0(i) = 4*(i&1) + 16*(i>>1),
+  // b_kk = (t>>5 & 3) + 8*(t>>7); position t&31 holds logical chunk (t&31) ^ (((k&3)<<2) | (((k>>3)&1)<<1)).  The
+  // swizzle depends on bits 0, 1 and 3 of k, and the rows are dealt to the slabs so that these are the three bits of
+  // t>>5: one offset register then serves all four slabs.
+  const int b_r = tid >> 5;
+  const int b_kk = (b_r & 3) + 8 * (b_r >> 2);
+  const int b_chunk = (tid & 31) ^ ((b_r & 3) << 2) ^ ((b_r >> 2) << 1);
+  auto b_row0 = [](int i) { return 4 * (i & 1) + 16 * (i >> 1); };
   // row-major:  A(m,k) at m*lda + k,  B(k,n) at k*ldb + n
   // tile-major: A(m,k) at ((m/32)*ntk + k/32)*1024 + (m%32)*32 + k%32,
   //             B(k,n) at ((k/32)*ntn + n/32)*1024 + (k%32)*32 + n%32          (elements)
   const int64_t ntk = Kf / 32, ntn = Nf / 32;
   const uint32_t a_voff = TILED ? (uint32_t)((((int64_t)(a_row >> 5) * ntk << 10) + (a_row & 31) * 32 + a_chunk * 8) * 2)
                                 : (uint32_t)(((int64_t)a_row * g.lda + a_chunk * 8) * 2); // bytes, per thread
-  const uint32_t b_voff = TILED ? (uint32_t)((((b_chunk >> 2) << 10) + b_k * 32 + (b_chunk & 3) * 8) * 2)
-                                : (uint32_t)(((int64_t)b_k * g.ldb + b_chunk * 8) * 2);
+  const uint32_t b_voff = TILED ? (uint32_t)((((b_chunk >> 2) << 10) + b_kk * 32 + (b_chunk & 3) * 8) * 2)
+                                : (uint32_t)(((int64_t)b_kk * g.ldb + b_chunk * 8) * 2);
   const int64_t a_slab = TILED ? 2 * ntk * 2048 : 64 * g.lda * 2;                  // bytes, uniform
-  const int64_t b_slab = TILED ? 8 * 32 * 2 : 8 * g.ldb * 2;
+  const int64_t b_rows4 = TILED ? 4 * 32 * 2 : 4 * g.ldb * 2;                       // four k rows of B
+  auto b_slab_off = [&](int i) { return ((i & 1) + 4 * (i >> 1)) * b_rows4; };      // slab i's first row, b_row0(i)
   const int64_t a_kstep = TILED ? 2048 : BK * 2;
   const int64_t b_kstep = TILED ? ntn * 2048 : (int64_t)BK * g.ldb * 2;
   const int lds_wave = wave * 1024;
 
   // ---- LDS -> fragments ----
-  const int l32 = lane & 31, hi = lane >> 5;
-  const int a_base = (wm * (32 * MB) + l32) * 64;
-  const int a_x = (l32 >> 2) & 3;
-  int a_pos[2]; // sub-step s: logical chunk 2s + hi
-#pragma unroll
-  for (int s = 0; s < 2; ++s) a_pos[s] = a_base + (((s * 2 + hi) ^ a_x) << 4);
+  // v_mfma_f32_16x16x32: lane l supplies row (column) l%16 of its operand, k = 8*(l/16) .. +7.
+  // A fragment i (16 rows): one 16-byte read, row 16i + l%16, logical chunk l/16.
+  // B fragment j (16 columns): two transposing reads, k = 8*(l/16) + 4h + q, q = (l%16)/4, h = 0, 1: the sixteen lanes
+  // of a group read a 4 x 16 block (row q, 8 bytes at column 4*(l%4)) and lane i receives column i's four k.
   const int G4 = lane >> 4, i16 = lane & 15, q = i16 >> 2;
-  const int b_base = A_BYTES + (((G4 >> 1) * 8 + q) * 512) + ((wn * 16 + (G4 & 1) * 2 + ((i16 >> 1) & 1)) << 4) +
+  constexpr int NA = 2 * MB;                 // A fragments of a wavefront's 32*MB rows; it has 8 B fragments
+  const int a_pos = (wm * (32 * MB) + i16) * 64 + ((G4 ^ q) << 4);          // fragment i: + i * 1024
+  // k = 8*G4 + 4h + q lies in slab h + 2*(G4>>1), row q + 4*(G4&1) of it; its swizzle is (q<<2) | ((G4&1)<<1)
+  const int b_base = A_BYTES + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
-  int b_pos[4];
+  int b_pos[8];                                                             // half h: + h * 4096
 #pragma unroll
-  for (int j = 0; j < 4; ++j) b_pos[j] = b_base + ((j ^ q) << 6);
+  for (int j = 0; j < 8; ++j) b_pos[j] = b_base + ((j ^ ((q << 1) | (G4 & 1))) << 5);
 
   const uint8_t *A = (const uint8_t *)g.a;
   const uint8_t *B = (const uint8_t *)g.b;
   const long long probe_c0 = g.probe ? clock64() : 0, probe_w0 = g.probe ? wall_clock64() : 0;
 
-  // Fragment registers: two sets (even / odd sub-steps).  B fragments are kept as their
-  // two transposed halves (k 0-3 and k 4-7 of the lane's group).
+  // Fragment registers: two sets (the step being multiplied and the next one).  B fragments are kept as
+  // their two transposed halves (k 0-3 and k 4-7 of the lane's group).
   struct Frags {
-    vec a[MB];
-    union { s16x4 h[2]; vec v; } b[4];
+    vec a[NA];
+    union { s16x4 h[2]; vec v; } b[8];
   };
   Frags f0, f1;
-  f32x16 acc[MB][4]; // [m-tile][n-tile]
+  f32x4 acc[NA][8]; // [16-row block][16-column block]
+  constexpr int NR = 16 + NA;   // LDS reads per step
+  constexpr int NM = 8 * NA;    // MFMAs per step
 
-  // The 12 LDS reads of one sub-step, in the order the MFMAs will want them:
-  // b0.lo b0.hi a0 b1.lo b1.hi b2.lo b2.hi b3.lo b3.hi a1 a2 a3        (MB == 2: the first ten)
-  auto rd = [&](Frags &f, const uint8_t *stage, int s, int r) {
-    switch (r) {
-    case 2: f.a[0] = *(const vec *)(stage + a_pos[s]); break;
-    case 9: f.a[1] = *(const vec *)(stage + a_pos[s] + 2048); break;
-    case 10: if constexpr (MB == 4) f.a[2] = *(const vec *)(stage + a_pos[s] + 4096); break;
-    case 11: if constexpr (MB == 4) f.a[3] = *(const vec *)(stage + a_pos[s] + 6144); break;
-    default: {
-      const int rr = r < 2 ? r : r - 1; // 0..7 over the b reads
+  // The LDS reads of one step, in the order the MFMAs will want them:
+  // b0.lo b0.hi a0 b1.lo b1.hi ... b7.lo b7.hi a1 ... a(NA-1)
+  auto rd = [&](Frags &f, const uint8_t *stage, int r) {
+    if (r == 2) {
+      f.a[0] = *(const vec *)(stage + a_pos);
+    } else if (r < 17) {
+      const int rr = r < 2 ? r : r - 1; // 0..15 over the b reads
       const int j = rr >> 1, h = rr & 1;
-      f.b[j].h[h] =
-          __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(stage + b_pos[j] + s * 8192 + h * 2048));
-    }
+      f.b[j].h[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(stage + b_pos[j] + h * 4096));
+    } else {
+      f.a[r - 16] = *(const vec *)(stage + a_pos + (r - 16) * 1024);
     }
   };
-  // MFMA number n (0..4*MB-1) of a sub-step, m-tile major: needs a[n/4], b[n%4]
+  // MFMA number n (0..NM-1) of a step, row-block major: needs a[n/8], b[n%8]
   auto mm = [&](Frags &f, int n) {
-    const int i = n >> 2, j = n & 3;
-    acc[i][j] = X::run(f.b[j].v, f.a[i], acc[i][j]);
+    const int i = n >> 3, j = n & 7;
+    X::run(f.b[j].v, f.a[i], acc[i][j]);
   };
   // One direct-to-LDS copy: lane l's 16 bytes land at dst_slab + wave*1024 + 16*l.
   // Written as assembly on purpose: the compiler's own bookkeeping of such copies is
@@ -281,11 +299,11 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + i * 4096 + lds_wave + lane * 16);
         *p = *p & keep;
       }
-      // B: slab i holds k rows 8i .. 8i + 7, this thread's sixteen bytes lie in row 8i + b_k
+      // B: this thread's sixteen bytes of slab i lie in k row b_row0(i) + b_kk
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + A_BYTES + i * 4096 + lds_wave + lane * 16);
-        if (i * 8 + b_k >= k_tail) *p = (u32x4){0, 0, 0, 0};
+        if (b_row0(i) + b_kk >= k_tail) *p = (u32x4){0, 0, 0, 0};
       }
     }
   };
@@ -322,8 +340,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                         : (uint32_t)(((int64_t)r * g.lda + a_chunk * 8) * 2);
       }
       const int cc = min(b_chunk, last_chunk);
-      vo.b = TILED ? (uint32_t)((((cc >> 2) << 10) + b_k * 32 + (cc & 3) * 8) * 2)
-                   : (uint32_t)(((int64_t)b_k * g.ldb + cc * 8) * 2);
+      vo.b = TILED ? (uint32_t)((((cc >> 2) << 10) + b_kk * 32 + (cc & 3) * 8) * 2)
+                   : (uint32_t)(((int64_t)b_kk * g.ldb + cc * 8) * 2);
     }
   };
   // copy number i (0..MB-1: A slabs, MB..MB+3: B slabs) of step kk into `stage`; kk may run past
@@ -339,13 +357,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       if (i < MB)
         dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
       else
-        dma_one(b_cur + (int64_t)k * b_kstep + (i - MB) * b_slab, vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
+        dma_one(b_cur + (int64_t)k * b_kstep + b_slab_off(i - MB), vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
     } else if constexpr (RAGGED) {
       const bool zero = k >= nk_real;                         // a padding step: both operands are zeros
       // row-major operands, last data step of a K that is not a whole number of steps: the 16-byte chunks of A past
       // K belong to the next row (past the buffer, for the last row) and the rows of B past K do not exist.  They
-      // are fetched from the step's first chunk / first slab instead, which exist, and cleared once they have landed
-      // (clear_past_k).  Tile-major buffers are padded to whole tiles and need no redirection.
+      // are fetched from the step's first chunk / first eight rows instead, which exist (K is a multiple of 8), and
+      // cleared once they have landed (clear_past_k).  A wavefront's rows of a B slab all lie in one group of eight
+      // (b_row0(i)/8 + wave/2), so the choice is the wavefront's and the copy's base address stays scalar.
+      // Tile-major buffers are padded to whole tiles and need no redirection.
       const bool tail = !TILED && k_tail != 0 && k == nk_real - 1;
       const Voffs &vo = over ? vo_nxt : vo_cur;
       if (i < MB) {
@@ -353,100 +373,60 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         const uint32_t av = (tail && a_chunk * 8 >= k_tail) ? vo.a[i] - (uint32_t)a_chunk * 16 : vo.a[i];
         dma_one(ap, zero ? z_voff : av, stage + i * 4096);
       } else {
-        const int slab = (tail && (i - MB) * 8 >= k_tail) ? 0 : i - MB;
-        const uint8_t *bp = zero ? zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + slab * b_slab;
-        dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - MB) * 4096);
+        const int ib = i - MB;
+        const bool redirect = tail && ((b_row0(ib) >> 3) + (wave >> 1)) * 8 >= k_tail;   // to row & 7
+        const uint8_t *bp = zero ? zero_page
+                                 : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (redirect ? (ib & 1) * b_rows4 : b_slab_off(ib));
+        const uint32_t bv = redirect ? vo.b - (uint32_t)((wave >> 1) * 2 * b_rows4) : vo.b;
+        dma_one(bp, zero ? z_voff : bv, stage + A_BYTES + (i - MB) * 4096);
       }
     } else if (i < MB) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
-      dma_one(bp + (i - MB) * b_slab, b_voff, stage + A_BYTES + (i - MB) * 4096);
+      dma_one(bp + b_slab_off(i - MB), b_voff, stage + A_BYTES + (i - MB) * 4096);
     }
   };
 
-  // One step (K += 32) on ring stage I.
-  //   entry: f0 holds sub-step 0 of stage I; copies for the next R-1 steps are in flight
-  //   exit : f0 holds sub-step 0 of stage I+1
-  // The eight copies that refill a stage are spread over the step period that follows the
-  // barrier which frees it (second half of this step, first half of the next), one per two
-  // MFMAs behind the MFMAs that carry the fragment reads (7, 9, 11, 13 of each sub-step): a
-  // wavefront that issues copies back to back stalls behind the memory pipeline's input
-  // queue, and its MFMAs stall with it.  (One per four MFMAs, at 1, 5, 9, 13, keeps the pipe
-  // 77 % busy at 1.68 GHz, this placement 80 % at 1.63 GHz: the part is power-limited, so
-  // most of a gain in issue efficiency is taken back by the clock.)
-  auto step = [&](auto I_, int k, auto inner_) {
+  // One step (K += 32) on ring stage I: the NM MFMAs on `c` (read from stage I during the previous step), the next
+  // stage's fragments into `p`, and the refill of stage I itself with step k+R.
+  //   The first MFMA goes out before the barrier, so that the matrix pipe has work while the wavefronts meet.
+  //   The fragment reads ride one per MFMA behind the barrier; the MB + 4 copies that refill the stage follow
+  //   them, one per four MFMAs (64 cycles): a wavefront that issues copies back to back stalls behind the memory
+  //   pipeline's input queue, and its MFMAs stall with it.
+  auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_) {
     constexpr int I = decltype(I_)::value;
-    uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R], *prv = ring.s[(I + R - 1) % R];
-    if constexpr (MB == 4) {
-      // sub-step 0: MFMAs on f0; sub-step 1's fragments ride along (two reads per MFMA);
-      // second half of the refill of the stage freed one step ago
-  #pragma unroll
-      for (int n = 0; n < 16; ++n) {
-        if (n < 6) {
-          rd(f1, cur, 1, 2 * n);
-          rd(f1, cur, 1, 2 * n + 1);
-        }
-        if (n >= 7 && n <= 13 && (n & 1)) dma_single(k - 1 + R, prv, 4 + ((n - 7) >> 1), inner_);
-        mm(f0, n);
-        FENCE();
-      }
-      // All of this wave's reads of stage I have returned, and so has its share of the
-      // copy into stage I+1 (the 16 younger copies may still be in flight).  After the
-      // barrier that holds for every wave: I+1 may be read, I may be overwritten.
-      if constexpr (RAGGED && !decltype(inner_)::value) {
-        if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
+    uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
+    mm(c, 0);
+    FENCE();
+    if constexpr (RAGGED && !decltype(inner_)::value) {
+      if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
+        if constexpr (MB == 4)
           asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-          clear_past_k(nxt);
-        }
-      }
-      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      FENCE();
-      // sub-step 1: MFMAs on f1; the next stage's sub-step 0 fragments; first half of the
-      // refill of stage I with step k+R
-  #pragma unroll
-      for (int n = 0; n < 16; ++n) {
-        if (n < 6) {
-          rd(f0, nxt, 0, 2 * n);
-          rd(f0, nxt, 0, 2 * n + 1);
-        }
-        if (n >= 7 && n <= 13 && (n & 1)) dma_single(k + R, cur, (n - 7) >> 1, inner_);
-        mm(f1, n);
-        FENCE();
-      }
-    } else {
-      // Half tiles: the same step with eight MFMAs per sub-step, ten fragment reads (two per MFMA over the
-      // first five) and six copies: the four B slabs of step k-1+R in sub-step 0, the two A slabs of step
-      // k+R in sub-step 1.  At the barrier the two youngest steps' copies (12) may still be in flight.
-#pragma unroll
-      for (int n = 0; n < 8; ++n) {
-        if (n < 5) {
-          rd(f1, cur, 1, 2 * n);
-          rd(f1, cur, 1, 2 * n + 1);
-        }
-        if (n & 1) dma_single(k - 1 + R, prv, MB + (n >> 1), inner_);
-        mm(f0, n);
-        FENCE();
-      }
-      if constexpr (RAGGED && !decltype(inner_)::value) {
-        if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
+        else
           asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-          clear_past_k(nxt);
-        }
+        clear_past_k(nxt);
       }
+    }
+    // Every wave's reads of stage I have returned (they fed `c`), and this wave's share of the copy into stage
+    // I+1 has landed (the copies of the two younger steps may still be in flight); after the barrier that holds for
+    // all waves: I+1 may be read, I may be overwritten.
+    if constexpr (MB == 4)
+      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else
       asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      FENCE();
+    FENCE();
 #pragma unroll
-      for (int n = 0; n < 8; ++n) {
-        if (n < 5) {
-          rd(f0, nxt, 0, 2 * n);
-          rd(f0, nxt, 0, 2 * n + 1);
-        }
-        if ((n & 3) == 1) dma_single(k + R, cur, n >> 2, inner_);
-        mm(f1, n);
-        FENCE();
+    for (int n = 1; n < NM; ++n) {
+      if (n <= NR) rd(p, nxt, n - 1);
+      if constexpr (MB == 4) {
+        if (n >= 28 && n <= 56 && (n & 3) == 0) dma_single(k + R, cur, (n - 28) >> 2, inner_);
+      } else {
+        if (n % 5 == 0 && n <= 30) dma_single(k + R, cur, n / 5 - 1, inner_);
       }
+      mm(c, n);
+      FENCE();
     }
   };
 
@@ -460,32 +440,31 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   b_nxt = b_cur;
   vo_nxt = vo_cur;
   if constexpr (!RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
-  // steps 0..R-2 whole, and the first half of step R-1 (step 0's first sub-step issues the rest)
 #pragma unroll
   for (int s = 0; s < R; ++s)
 #pragma unroll
-    for (int i = 0; i < (s == R - 1 ? MB : MB + 4); ++i) dma_single(s, ring.s[s], i, std::false_type{});
+    for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
-  // everything issued but step 0's own MB + 4 copies may still be in flight: 2 * (MB + 4) + MB
   if (RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     clear_past_k(ring.s[0]);
   }
+  // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
   if constexpr (MB == 4)
-    asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // step 0 has landed
+    asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   else
-    asm volatile("s_waitcnt vmcnt(14) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-  for (int r = 0; r < 8 + MB; ++r) rd(f0, ring.s[0], 0, r);
+  for (int r = 0; r < NR; ++r) rd(f0, ring.s[0], r);
 
   for (; t < total; t += gridDim.x) {
     int tm, tn, half;
     item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, half);
     const int64_t m0 = (int64_t)tm * BM + half * 128, n0 = (int64_t)tn * BN;
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+    for (int i = 0; i < NA; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
+      for (int j = 0; j < 8; ++j) acc[i][j] = (f32x4){0, 0, 0, 0};
 
     int k = 0;
     // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
@@ -493,19 +472,19 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // out of these turns)
     const int nk_inner = nk_real - ((!TILED && k_tail) ? 1 : 0);
     for (; k + 2 * R <= nk_inner; k += R) {
-      step(std::integral_constant<int, 0>{}, k, std::true_type{});
-      step(std::integral_constant<int, 1>{}, k + 1, std::true_type{});
-      step(std::integral_constant<int, 2>{}, k + 2, std::true_type{});
-      step(std::integral_constant<int, 3>{}, k + 3, std::true_type{});
+      step(std::integral_constant<int, 0>{}, k, f0, f1, std::true_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::true_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::true_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::true_type{});
     }
     // the remaining turns copy the next tile's first steps (this tile's again when there is none: a harmless
     // refetch); RAGGED: where that tile lies is worked out only now
     if constexpr (RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
     for (; k < nk; k += R) {
-      step(std::integral_constant<int, 0>{}, k, std::false_type{});
-      step(std::integral_constant<int, 1>{}, k + 1, std::false_type{});
-      step(std::integral_constant<int, 2>{}, k + 2, std::false_type{});
-      step(std::integral_constant<int, 3>{}, k + 3, std::false_type{});
+      step(std::integral_constant<int, 0>{}, k, f0, f1, std::false_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::false_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::false_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::false_type{});
     }
     // the ring already holds the next tile's first steps; move the tile window on
     a_cur = a_nxt;
@@ -518,32 +497,32 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       tile_bases(t2 < total ? t2 : (t + (int)gridDim.x < total ? t + (int)gridDim.x : t), a_nxt, b_nxt, vo_nxt);
     }
 
-    // ---- epilogue: acc[i][j] register r of lane l is C[m][n] with
-    //      m = i*32 + l%32,  n = j*32 + (r/4)*8 + (l/32)*4 + r%4
-    const int64_t m = m0 + wm * (32 * MB) + l32;
-    // A row bias depends on n only: its 64 values for this lane are fetched once, all loads in flight
+    // ---- epilogue: acc[i][j] register e of lane l is C[m][n] with
+    //      m = i*16 + l%16,  n = j*16 + (l/16)*4 + e
+    // The MFMAs are assembly to the compiler, which therefore does not know to wait for the last of them before it
+    // reads an accumulator: sixteen idle cycles cover the four passes of a 16x16x32.
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+    const int64_t m = m0 + wm * (32 * MB) + i16;
+    // A row bias depends on n only: its 32 values for this lane are fetched once, all loads in flight
     // together, instead of one dependent load per use in the loop below.
     constexpr bool ROW_BIAS = EPI == EPI_BIAS_ROW || EPI == EPI_BIAS_ROW_GELU;
-    f32x4 brow[ROW_BIAS ? 4 : 1][ROW_BIAS ? 4 : 1];
+    f32x4 brow[ROW_BIAS ? 8 : 1];
     if constexpr (ROW_BIAS) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-          brow[j][r4] = *(const f32x4 *)((const float *)g.bias +
-                                         (RAGGED ? min(n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4, (int64_t)g.N - 4)
-                                                 : n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4));
+      for (int j = 0; j < 8; ++j)
+        brow[j] = *(const f32x4 *)((const float *)g.bias + (RAGGED ? min(n0 + wn * 128 + j * 16 + G4 * 4, (int64_t)g.N - 4)
+                                                                   : n0 + wn * 128 + j * 16 + G4 * 4));
     }
-    // the four columns n .. n+3 of row mi that this lane holds for (i, j, r4), after scale, epilogue and rounding
-    auto packed = [&](int i, int j, int r4, int64_t mi, int64_t n) {
+    // the four columns n .. n+3 of row mi that this lane holds for (i, j), after scale, epilogue and rounding
+    auto packed = [&](int i, int j, int64_t mi, int64_t n) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float x = acc[i][j][r4 * 4 + e] * g.scale;
+        const float x = acc[i][j][e] * g.scale;
         if constexpr (EPI == EPI_BIAS_ROW_GELU)
-          v[e] = gelu_erf(x + brow[j][r4][e]);
+          v[e] = gelu_erf(x + brow[j][e]);
         else if constexpr (EPI == EPI_BIAS_ROW)
-          v[e] = x + brow[j][r4][e];
+          v[e] = x + brow[j][e];
         else
           v[e] = apply_epilogue_ct<OUT_DT, EPI>(g, x, mi, n + e);
       }
@@ -554,40 +533,37 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                        (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16)};
     };
 #pragma unroll
-    for (int i = 0; i < MB; ++i) {
-      const int64_t mi = m + i * 32;
+    for (int i = 0; i < NA; ++i) {
+      const int64_t mi = m + i * 16;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int jp = 0; jp < 4; ++jp) {
         if constexpr (!(RAGGED && TILED)) {
-          // The lane pair (l, l+32) holds columns 0-3 | 4-7 for r4 = 2q and 8-11 | 12-15 for r4 = 2q+1 of one row.
-          // Swapping the upper lanes' first group with the lower lanes' second (v_permlane32_swap: upper half of
-          // its first operand <-> lower half of its second) gives the lower lane columns 0-7 and the upper lane
-          // 8-15, so each lane stores 16 contiguous bytes: half the store instructions, each covering 32 bytes of
-          // a row (8 columns never straddle a 32x32 tile of a tile-major C, nor the edge of a clipped one, whose N
-          // is a multiple of 8).  Every lane takes part in the swap; clipped lanes only skip the store, and read a
-          // full bias, if there is one, at a clamped position.
-#pragma unroll
-          for (int q = 0; q < 2; ++q) {
-            const int64_t nb = n0 + wn * 128 + j * 32 + q * 16;
-            const int64_t mb = RAGGED ? min(mi, (int64_t)g.M - 1) : mi;
-            const int64_t nl = nb + hi * 4, nh = nb + 8 + hi * 4;
-            u32x2 p0 = packed(i, j, 2 * q, mb, RAGGED ? min(nl, (int64_t)g.N - 4) : nl);
-            u32x2 p1 = packed(i, j, 2 * q + 1, mb, RAGGED ? min(nh, (int64_t)g.N - 4) : nh);
-            asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p0.x), "+v"(p1.x));
-            asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p0.y), "+v"(p1.y));
-            const int64_t n = nb + hi * 8;
-            if (RAGGED && (mi >= g.M || n >= g.N)) continue;
-            const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
-            *(u32x4 *)((uint16_t *)g.c + coff) = (u32x4){p0.x, p0.y, p1.x, p1.y};
-          }
+          // Of the 32 columns of the block pair (2jp, 2jp+1), lane group G4 = l/16 holds 4*G4 .. +3 and 16 + 4*G4 .. +3
+          // of one row.  Swapping the odd groups' first piece with the even groups' second (v_permlane16_swap: odd
+          // rows of sixteen lanes of its first operand <-> even rows of its second) leaves groups 0, 1, 2, 3 with
+          // columns 0-7, 16-23, 8-15, 24-31: each lane stores 16 contiguous bytes, four lanes a row's 64 (8 columns
+          // never straddle a 32x32 tile of a tile-major C, nor the edge of a clipped one, whose N is a multiple of
+          // 8).  Every lane takes part in the swap; clipped lanes only skip the store, and read a full bias, if
+          // there is one, at a clamped position.
+          const int64_t nb = n0 + wn * 128 + jp * 32;
+          const int64_t mb = RAGGED ? min(mi, (int64_t)g.M - 1) : mi;
+          const int64_t nl = nb + G4 * 4, nh = nb + 16 + G4 * 4;
+          u32x2 p0 = packed(i, 2 * jp, mb, RAGGED ? min(nl, (int64_t)g.N - 4) : nl);
+          u32x2 p1 = packed(i, 2 * jp + 1, mb, RAGGED ? min(nh, (int64_t)g.N - 4) : nh);
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p0.x), "+v"(p1.x));
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p0.y), "+v"(p1.y));
+          const int64_t n = nb + (G4 & 1) * 16 + (G4 >> 1) * 8;
+          if (RAGGED && (mi >= g.M || n >= g.N)) continue;
+          const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
+          *(u32x4 *)((uint16_t *)g.c + coff) = (u32x4){p0.x, p0.y, p1.x, p1.y};
         } else {
 #pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
-            if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // row-major: N is a multiple of 8, the four columns stand or fall together
-            const u32x2 pk = packed(i, j, r4, mi, n);
-            const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
-            if (TILED && RAGGED && n + 3 >= g.N) {               // N is anything here: the last group goes by element
+          for (int j = 2 * jp; j < 2 * jp + 2; ++j) {
+            const int64_t n = n0 + wn * 128 + j * 16 + G4 * 4;
+            if (mi >= g.M || n >= g.N) continue;
+            const u32x2 pk = packed(i, j, mi, n);
+            const int64_t coff = (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31);
+            if (n + 3 >= g.N) {               // N is anything here: the last group goes by element
               for (int e = 0; e < 4 && n + e < g.N; ++e)
                 ((uint16_t *)g.c)[coff + e] = (uint16_t)(e & 1 ? pk[e >> 1] >> 16 : pk[e >> 1] & 0xffffu);
               continue;
