@@ -393,8 +393,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // stage's fragments into `p`, and the refill of stage I itself with step k+R.
   //   The first MFMA goes out before the barrier, so that the matrix pipe has work while the wavefronts meet.
   //   The fragment reads ride one per MFMA behind the barrier; the MB + 4 copies that refill the stage follow
-  //   them, one per four MFMAs (64 cycles): a wavefront that issues copies back to back stalls behind the memory
-  //   pipeline's input queue, and its MFMAs stall with it.
+  //   them, one per five MFMAs (80 cycles): a wavefront that issues copies back to back stalls behind the memory
+  //   pipeline's input queue, and its MFMAs stall with it.  (Placement matters little here: two MFMAs or four
+  //   before the barrier, reads on every second MFMA, copies every third to seventh MFMA from the 7th to the 30th
+  //   on all measured within 1 % of each other, 1477-1497 TFLOP/s on 8192^3; two reads per MFMA cost 1.5 %.)
   auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_) {
     constexpr int I = decltype(I_)::value;
     uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
@@ -421,7 +423,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     for (int n = 1; n < NM; ++n) {
       if (n <= NR) rd(p, nxt, n - 1);
       if constexpr (MB == 4) {
-        if (n >= 28 && n <= 56 && (n & 3) == 0) dma_single(k + R, cur, (n - 28) >> 2, inner_);
+        if (n >= 25 && n <= 60 && n % 5 == 0) dma_single(k + R, cur, n / 5 - 5, inner_);
       } else {
         if (n % 5 == 0 && n <= 30) dma_single(k + R, cur, n / 5 - 1, inner_);
       }
