@@ -259,9 +259,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       f.a[r - 16] = *(const vec *)(stage + a_pos + (r - 16) * 1024);
     }
   };
-  // MFMA number n (0..NM-1) of a step, row-block major: needs a[n/8], b[n%8]
+  // MFMA number n (0..NM-1) of a step, row-block major: needs a[n/8] and each b once per row block
   auto mm = [&](Frags &f, int n) {
-    const int i = n >> 3, j = n & 7;
+    // (odd row blocks walk the columns backwards: every MFMA then shares one operand with the one before it)
+    const int i = n >> 3, j = (i & 1) ? 7 - (n & 7) : (n & 7);
     X::run(f.b[j].v, f.a[i], acc[i][j]);
   };
   // One direct-to-LDS copy: lane l's 16 bytes land at dst_slab + wave*1024 + 16*l.
