@@ -28,7 +28,7 @@
 //
 // LDS layout per stage (16-byte chunks, XOR-swizzled so that the row-wise A
 // reads and the transposing B reads are both bank-conflict free):
-//   A: row m = 64 B = 4 chunks;   logical chunk c sits at c ^ ((m>>2)&3)
+//   A: row m = 64 B = 4 chunks;   logical chunk c sits at c ^ a_swz((m>>2)&3)
 //   B: row k = 512 B = 32 chunks; logical chunk c sits at c ^ (((k&3)<<2) | (((k>>3)&1)<<1));
 //      the k rows are dealt to the four 4 KiB slabs as {0-3, 8-11}, {4-7, 12-15}, {16-19, 24-27}, {20-23, 28-31}
 // A direct-to-LDS load writes lane l's 16 bytes at (wave-uniform base) + 16*l,
@@ -152,6 +152,15 @@ __device__ __forceinline__ void item_tile(const PassItems &p, int item, int tile
 
 #define FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// Swizzle of A's 16-byte chunks within a 64-byte row, by the row's group of four (0..3) -> 0, 2, 3, 1.
+// A 16-byte LDS read of a wavefront is served in four passes of sixteen lanes, and not of neighbouring lanes:
+// lanes {0-3, 12-15, 20-23, 24-27} go together, then {4-7, 8-11, 16-19, 28-31}, and the same with 32 added.  With
+// the fragment layout of the 16x16x32 MFMA (lane l: row l%16, chunk l/16) a pass therefore holds two groups of four
+// rows with chunk g and two with chunk g^1, and each group of four rows spans all 256 bytes of the banks at one
+// chunk position: the four positions of a pass must differ.  c ^ (row group) does not do that (measured: every A
+// read took twice its cycles, SQ_LDS_BANK_CONFLICT = a third of SQ_LDS_IDX_ACTIVE); this permutation does.
+__device__ __forceinline__ int a_swz(int row_group) { return (((row_group ^ (row_group >> 1)) & 1) << 1) | (row_group >> 1); }
+
 struct Ring {
   uint8_t *s[R];
 };
@@ -190,9 +199,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
   // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
-  // A slab i (64 rows): row = i*64 + (t>>2), chunk position t&3 holds logical chunk (t&3)^((row>>2)&3)
+  // A slab i (64 rows): row = i*64 + (t>>2), chunk position t&3 holds logical chunk (t&3) ^ a_swz((row>>2)&3)
   const int a_row = tid >> 2;
-  const int a_chunk = (tid & 3) ^ ((a_row >> 2) & 3);
+  const int a_chunk = (tid & 3) ^ a_swz((a_row >> 2) & 3);
   // B slab i (8 rows of 512 B): row t>>5 of the slab holds k = b_row0(i) + b_kk, b_row0(i) = 4*(i&1) + 16*(i>>1),
   // b_kk = (t>>5 & 3) + 8*(t>>7); position t&31 holds logical chunk (t&31) ^ (((k&3)<<2) | (((k>>3)&1)<<1)).  The
   // swizzle depends on bits 0, 1 and 3 of k, and the rows are dealt to the slabs so that these are the three bits of
@@ -223,7 +232,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // of a group read a 4 x 16 block (row q, 8 bytes at column 4*(l%4)) and lane i receives column i's four k.
   const int G4 = lane >> 4, i16 = lane & 15, q = i16 >> 2;
   constexpr int NA = 2 * MB;                 // A fragments of a wavefront's 32*MB rows; it has 8 B fragments
-  const int a_pos = (wm * (32 * MB) + i16) * 64 + ((G4 ^ q) << 4);          // fragment i: + i * 1024
+  const int a_pos = (wm * (32 * MB) + i16) * 64 + ((G4 ^ a_swz(q)) << 4);   // fragment i: + i * 1024
   // k = 8*G4 + 4h + q lies in slab h + 2*(G4>>1), row q + 4*(G4&1) of it; its swizzle is (q<<2) | ((G4&1)<<1)
   const int b_base = A_BYTES + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
