@@ -306,6 +306,30 @@ def main() -> int:
                 red[f"{op}_f32_{nr}"] = {"us_avg": round(avg_ms * 1e3, 2), "us_min": round(min(per) * 1e3, 2)}
         extra["reduce1d"] = red
         del gr
+        # a matmul small enough that the launch path is what is timed (the kernel itself takes about 5 us): the
+        # reference-style wrapper (three descriptors made per call, a callable grid) and the bare launch
+        a512 = torch.randn(512, 512, device="cuda").to(torch.bfloat16)
+        b512 = torch.randn(512, 512, device="cuda").to(torch.bfloat16)
+        for _ in range(20):
+            K.matmul_tma(a512, b512)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(2000):
+            K.matmul_tma(a512, b512)
+        wrap_us = (time.perf_counter() - t0) / 2000 * 1e6
+        torch.cuda.synchronize()
+        c512 = torch.empty(512, 512, device="cuda", dtype=torch.bfloat16)
+        d512 = [TensorDescriptor.from_tensor(t, [32, 32]) for t in (a512, b512, c512)]
+        launch_m = K.matmul_kernel_tma[(16, )]
+        for _ in range(20):
+            launch_m(*d512, 512, 512, 512, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(2000):
+            launch_m(*d512, 512, 512, 512, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+        bare_us = (time.perf_counter() - t0) / 2000 * 1e6
+        torch.cuda.synchronize()
+        extra["matmul_bf16_512"] = {"host_us_per_launch": round(bare_us, 2), "host_us_per_wrapper_call": round(wrap_us, 2)}
 
     # ---------------- fused epilogue: GELU(A.B + bias) ----------------------
     if want("fused"):

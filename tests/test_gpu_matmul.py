@@ -574,3 +574,61 @@ def test_nan_padded_descriptors(dtype):
     # 32-deep steps divide 96: no padding along K, no NaN
     _, _, c, _ = run(256, 256, 96, "nan", "nan", bk=32)
     assert not torch.isnan(c).any()
+
+
+def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
+    """From the second launch of a call shape on, the descriptor matmuls go through a cached closure (the
+    configuration's pre_hook, then one C call).  Whatever the closure does not recognise falls back to the full path:
+    same results, same refusals."""
+    g = torch.Generator().manual_seed(5)
+    M, N, K_ = 300, 328, 224
+    a = torch.randint(-3, 4, (M, K_), generator=g).to(torch.bfloat16).cuda()
+    b = torch.randint(-3, 4, (K_, N), generator=g).to(torch.bfloat16).cuda()
+    want = (a.float() @ b.float()).to(torch.bfloat16)
+    for _ in range(3):
+        assert torch.equal(K.matmul_tma(a, b), want)
+    assert K.matmul_kernel_tma._plan is not None
+    # the pre_hook still patches the descriptors it is handed (09-persistent-matmul.py:90-100)
+    c = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+    launch = K.matmul_kernel_tma[(K.cdiv(M, 128) * K.cdiv(N, 128), )]
+    launch(ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    assert torch.equal(c, want)
+    assert ad.block_shape == [128, 64] and bd.block_shape == [64, 128] and cd.block_shape == [128, 128]
+    # another dtype, another shape, a strided view, a dimension of 1: same answers as a first launch
+    a16, b16 = a.half(), b.half()
+    assert torch.equal(K.matmul_tma(a16, b16), (a16.float() @ b16.float()).half())
+    assert torch.equal(K.matmul_tma(a[:40], b), want[:40])
+    abuf = torch.zeros(M, K_ + 8, dtype=torch.bfloat16, device="cuda")
+    abuf[:, :K_] = a
+    assert torch.equal(K.matmul_tma(abuf[:, :K_], b), want)
+    assert torch.equal(K.matmul_tma(a[:1], b), want[:1])
+    assert torch.equal(K.matmul_tma(a, b), want)
+    # and the same refusals
+    c.fill_(7.5)
+    with pytest.raises(ValueError):
+        launch(ad, bd, cd, M, N, K_ + 8, FP8_OUTPUT=False, WARP_SPECIALIZE=False)      # K that the descriptors do not have
+    with pytest.raises(ValueError):
+        launch(ad, bd, TensorDescriptor.from_tensor(c[:, :64], [32, 32]), M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    with pytest.raises((ValueError, TypeError)):
+        launch(ad, bd, c, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)           # a tensor where a descriptor belongs
+    assert torch.all(c == 7.5)
+    # a side stream is picked up by the cached path too
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        launch(ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+    side.synchronize()
+    assert torch.equal(c, want)
+    # the fused kernel with a named epilogue and the scaled fp8 kernel have the closure too
+    bias = torch.randn(N, generator=g).cuda()
+    first = K.matmul_fused(a, b, bias, epilogue="bias_row")
+    for _ in range(2):
+        assert torch.equal(K.matmul_fused(a, b, bias, epilogue="bias_row"), first)
+    assert K.matmul_kernel_fused._plan is not None
+    assert torch.equal(first, ((a.float() @ b.float()) + bias).to(torch.bfloat16))
+    qa, sa = K.quantize_fp8(a[:, :192].float())           # fp8 rows must be whole 16-byte pieces
+    qb, sb = K.quantize_fp8(b[:192, :320].float())
+    first = K.matmul_fp8_scaled(qa, qb, sa, sb)
+    for _ in range(2):
+        assert torch.equal(K.matmul_fp8_scaled(qa, qb, sa, sb), first)
+    assert K.matmul_kernel_tma_fp8_scaled._plan is not None

@@ -106,6 +106,9 @@ class _Cursor:
         self.direct = None      # set by a binder that offers a repeat-launch closure (_streaming_direct)
 
     def _next(self):
+        if self.i >= len(self.flat):
+            raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "the launch arguments ran out before the kernel's parameters did "
+                                   "(a tensor where a tensor descriptor belongs?)")
         v = self.flat[self.i]
         self.i += 1
         return v
@@ -200,6 +203,52 @@ def _streaming_direct(fn, n_tensors: int, dtype, tail: tuple, per_program: int):
                 return False
             ptrs.append(t.data_ptr())
         rc = fn(*ptrs, n, *tail, grid3(gx, 1, 1), stream)
+        if rc:
+            check(rc)
+        return True
+
+    return direct
+
+
+def _desc_matmul_direct(fn, bases: list, n_floats: int, tail: tuple):
+    """Repeat-launch closure of the descriptor matmuls (see ``_streaming_direct``): the launch arguments are
+    ``len(dtypes)`` rank-2 descriptors, then M, N, K, then ``n_floats`` floats.  The closure re-checks what selects
+    the specialisation it was built under (descriptor class, rank, base dtype and device, integer M, N, K that Triton
+    would not fold) and fills its own ``tt_desc2d`` blocks, which the library reads during the call only; shapes,
+    strides, alignment and the grid are validated by the library as on the ordinary path."""
+    import torch
+    from ..tensor_descriptor import TensorDescriptor
+    dtypes = tuple(t.dtype for t in bases)      # of the descriptors' base tensors at the launch that built this
+    tensor_type, grid3, check, n_desc = torch.Tensor, rt.Grid3, rt.check, len(dtypes)
+    blocks = [rt.tt_desc2d() for _ in dtypes]
+    for blk, t in zip(blocks, bases):
+        blk.dtype = _torch_dtype_code(t)
+    refs = [C.byref(b) for b in blocks]
+    n_args = n_desc + 3 + n_floats
+
+    def direct(args, grid, stream):
+        if len(args) != n_args or len(grid) != 1 or type(grid[0]) is not int:
+            return False
+        M, N, K = args[n_desc], args[n_desc + 1], args[n_desc + 2]
+        if (type(M) is not int or type(N) is not int or type(K) is not int or not 1 < M < 2147483648
+                or not 1 < N < 2147483648 or not 1 < K < 2147483648):
+            return False
+        for blk, d, dt in zip(blocks, args, dtypes):
+            if type(d) is not TensorDescriptor:
+                return False
+            base, shape, strides = d.base, d.shape, d.strides
+            if (type(base) is not tensor_type or base.dtype is not dt or not base.is_cuda or len(shape) != 2
+                    or len(strides) != 2):
+                return False
+            blk.base = base.data_ptr()
+            blk.shape[0], blk.shape[1] = shape
+            blk.strides[0], blk.strides[1] = strides
+            blk.padding_nan = d.padding == "nan"
+        floats = args[n_desc + 3:]
+        for f in floats:
+            if type(f) is not float:
+                return False
+        rc = fn(*refs, M, N, K, *floats, *tail, grid3(grid[0], 1, 1), stream)
         if rc:
             check(rc)
         return True
@@ -407,12 +456,18 @@ def _bind_matmul_tma(lib, cur, consts, grid, stream):
     a, b, c = cur.desc(), cur.desc(), cur.desc()
     M, N, K = _mnk(cur, a, b)
     bm, bn, bk, g = _block_consts(consts, a)
+    bases = cur.keep[-3:]      # the three descriptors' base tensors, in order
+    with_mnk = cur.has("M")    # (the minimal variant reads M, N, K from the descriptors: no closure for it)
     if cur.has("scale_a"):
         sa, sb = float(cur.scalar("scale_a")), float(cur.scalar("scale_b"))
         cur.done()
+        if with_mnk:
+            cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_tma_fp8_scaled, bases, 2, (bm, bn, bk, g))
         return lib.tt_matmul_kernel_tma_fp8_scaled(C.byref(a), C.byref(b), C.byref(c), M, N, K, sa, sb, bm, bn, bk,
                                                    g, grid, stream)
     cur.done()
+    if with_mnk:
+        cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_tma, bases, 0, (bm, bn, bk, g))
     return lib.tt_matmul_kernel_tma(C.byref(a), C.byref(b), C.byref(c), M, N, K, bm, bn, bk, g, grid, stream)
 
 
@@ -431,6 +486,10 @@ def _bind_matmul_fused(lib, cur, consts, grid, stream):
         # the reference kernel: full [M,N] bias of the output type; a [1,N]/[N] fp32 bias selects the row form
         full = (bias.shape[0], bias.shape[1]) == (c.shape[0], c.shape[1]) and bias.dtype == c.dtype
         epi = rt.TT_EPI_BIAS_FULL if full else rt.TT_EPI_BIAS_ROW
+    # (the epilogue chosen from the bias's shape and dtype holds for repeat launches only while those stay as they
+    # are: the closure is offered for the named epilogues, which do not look at the bias)
+    if _EPILOGUES.get(consts.get("EPILOGUE")) is not None and "M" in cur.arg_names:
+        cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_fused, cur.keep[-4:], 0, (bm, bn, bk, g, epi))
     return lib.tt_matmul_kernel_fused(C.byref(a), C.byref(b), C.byref(c), C.byref(bias), M, N, K, bm, bn, bk, g, epi,
                                       grid, stream)
 

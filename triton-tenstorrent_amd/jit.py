@@ -117,7 +117,8 @@ class PrebuiltKernel:
         self.defaults = dict(defaults or {})
         self.fn = SimpleNamespace(arg_names=self.arg_names, __name__=name)
         self._cache: dict = {}
-        # repeat launches: (number of positional arguments, keyword arguments, device, closure, operands kept alive)
+        # repeat launches: (number of positional arguments, keyword arguments, device, closure, the configuration's
+        # pre_hook or None, the arguments after the positional ones by name for that hook)
         self._plan = None
         self._keep = None
         n_lead = next((i for i, n in enumerate(self.arg_names) if n in self.constexprs), len(self.arg_names))
@@ -150,12 +151,22 @@ class PrebuiltKernel:
 
     def run(self, *args, grid, **kwargs):
         plan = self._plan
-        if (plan is not None and TTDriver.get_current_stream is _STOCK_GET_STREAM and len(args) == plan[0] and kwargs == plan[1] and type(grid) is tuple
+        if (plan is not None and TTDriver.get_current_stream is _STOCK_GET_STREAM and len(args) == plan[0] and kwargs == plan[1] and (type(grid) is tuple or callable(grid))
                 and PrebuiltKernel.launch_enter_hook is None and PrebuiltKernel.launch_exit_hook is None):
             device, stream = _raw_stream()
-            if device == plan[2] and plan[3](args, grid, stream):
-                self._keep = args   # launches are asynchronous: operands stay referenced until the next one
-                return self
+            if device == plan[2]:
+                g = grid
+                if plan[4] is not None or type(g) is not tuple:
+                    # the configuration's pre_hook and a callable grid see every argument by name, as on the ordinary path
+                    named = dict(zip(self.arg_names, args))
+                    named.update(plan[5])
+                    if plan[4] is not None:
+                        plan[4](named)
+                    if type(g) is not tuple:
+                        g = g(named)
+                if type(g) is tuple and plan[3](args, g, stream):
+                    self._keep = args   # launches are asynchronous: operands stay referenced until the next one
+                    return self
         user_grid = grid
         bound = self._bind(args, kwargs)
         config = self.configs[0] if self.configs else None
@@ -194,7 +205,9 @@ class PrebuiltKernel:
             launch_md = self.launch_metadata(grid, SimpleNamespace(name=self.name), bound)
         launcher(gx, gy, gz, stream, function, packed, launch_md, enter, exit_, *bound.values())
         direct = getattr(launcher, "direct", None)
-        if (direct is not None and _raw_stream is not None and len(args) == self._lead and type(user_grid) is tuple
-                and (config is None or config.pre_hook is None) and stream == _raw_stream()[1]):
-            self._plan = (len(args), dict(kwargs), device, direct)
+        if (direct is not None and _raw_stream is not None and len(args) == self._lead
+                and (type(user_grid) is tuple or callable(user_grid)) and stream == _raw_stream()[1]):
+            hook = config.pre_hook if config is not None else None
+            rest = {n: bound[n] for n in self.arg_names[len(args):]}
+            self._plan = (len(args), dict(kwargs), device, direct, hook, rest)
         return self
