@@ -104,47 +104,50 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int &tm
   tn = (id % in_group) / gsz;
 }
 
-// Work items of one pass of a kernel that finishes a short last round as half tiles: the macro-tile pass
+// Work items of one pass of a kernel that finishes a short last round as parts of tiles: the macro-tile pass
 // (MB == 4) takes the whole rounds of the grid, or every tile when the tail is not worth splitting; the
-// half-tile pass (MB == 2) takes the two 128-row halves of each tail tile.
+// half-tile pass (MB == 2) takes the two 128-row halves of each tail tile when those keep at most the whole grid
+// busy, and (QUARTERS) the quarter-tile pass (MB == 1) the four 64-row quarters when even they do.
 struct PassItems {
   int total;       // items of this pass
-  int first_tile;  // MB == 2: id of the first tail tile
+  int first_tile;  // MB < 4: id of the first tail tile
   int tail_tiles;
 };
-template <int MB, bool SPLIT_TAIL>
+template <int MB, bool SPLIT_TAIL, bool QUARTERS = false>
 __device__ __forceinline__ PassItems pass_items(int total_tiles) {
   PassItems p = {total_tiles, 0, 0};
   if constexpr (SPLIT_TAIL) {
     const int whole = total_tiles / (int)gridDim.x * (int)gridDim.x;
     p.tail_tiles = total_tiles - whole;
-    const bool split = p.tail_tiles > 0 && 2 * p.tail_tiles <= (int)gridDim.x;
+    const bool quarters = QUARTERS && p.tail_tiles > 0 && 4 * p.tail_tiles <= (int)gridDim.x;
+    const bool halves = !quarters && p.tail_tiles > 0 && 2 * p.tail_tiles <= (int)gridDim.x;
     if (MB == 4) {
-      p.total = split ? whole : total_tiles;
+      p.total = (quarters || halves) ? whole : total_tiles;
     } else {
-      p.total = split ? 2 * p.tail_tiles : 0;
+      p.total = MB == 2 ? (halves ? 2 * p.tail_tiles : 0) : (quarters ? 4 * p.tail_tiles : 0);
       p.first_tile = whole;
     }
   }
   return p;
 }
-// item -> macro tile and which half of it.  Workgroup ids go round-robin over the 8 XCDs and tile_of gives
-// tile t to XCD t % 8's run of ids, so halves are dealt in groups of 16 items over 8 tiles: both halves of
-// a tile then stay on the XCD that tile's neighbours ran on.
+// item -> macro tile and which part of it (0 .. 4/MB - 1).  Workgroup ids go round-robin over the 8 XCDs and
+// tile_of gives tile t to XCD t % 8's run of ids, so parts are dealt in groups of 8 tiles: all parts of a tile
+// then stay on the XCD that tile's neighbours ran on.
 template <int MB>
 __device__ __forceinline__ void item_tile(const PassItems &p, int item, int tiles_m, int tiles_n, int &tm, int &tn,
-                                          int &half) {
+                                          int &part) {
   if constexpr (MB == 4) {
-    half = 0;
+    part = 0;
     tile_of(item, tiles_m, tiles_n, tm, tn);
   } else {
+    constexpr int PARTS = 4 / MB, SH = MB == 2 ? 1 : 2;
     int j;
     if (p.tail_tiles % 8 == 0) {
-      j = (item >> 4) * 8 + (item & 7);
-      half = (item >> 3) & 1;
+      j = (item >> (3 + SH)) * 8 + (item & 7);
+      part = (item >> 3) & (PARTS - 1);
     } else {
-      j = item >> 1;
-      half = item & 1;
+      j = item >> SH;
+      part = item & (PARTS - 1);
     }
     tile_of(p.first_tile + j, tiles_m, tiles_n, tm, tn);
   }
@@ -178,9 +181,16 @@ struct Ring {
 // the kernel runs body<MB=4> over the whole rounds and then body<MB=2> over the halves of the tail tiles,
 // two workgroups per tile, instead of leaving half of the chip idle for a whole tile's time.  (RAGGED: a
 // half tile that lies wholly past the last row computes the other half's rows again and stores nothing.)
-template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false>
+//
+// With MB == 1 (QUARTERS) a workgroup computes a 64x256 quarter (each wavefront 32x128: 2x8 accumulators, one A slab
+// and five copies per step, 16 MFMAs per step): a problem of at most CUs/4 macro tiles, or such a tail, then fills
+// the chip four workgroups to a tile.  A quarter's step moves 20 KiB for a quarter of the flops and its fragment
+// reads (18 per wavefront and 16 MFMAs) keep the LDS busier than the matrix pipe, so it runs at about two thirds of
+// the macro tile's rate: worth it only where the alternative is idle CUs.
+template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false,
+          bool QUARTERS = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
-  static_assert(MB == 4 || (MB == 2 && SPLIT_TAIL), "half tiles exist for the tail pass only");
+  static_assert(MB == 4 || ((MB == 2 || (MB == 1 && QUARTERS)) && SPLIT_TAIL), "part tiles exist for the tail passes only");
   // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
   // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
   // real M and N (the padding of C is never written, as under the reference's store mask).
@@ -193,7 +203,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
   const int total_tiles = tiles_m * tiles_n;
-  const PassItems items = pass_items<MB, SPLIT_TAIL>(total_tiles);
+  const PassItems items = pass_items<MB, SPLIT_TAIL, QUARTERS>(total_tiles);
   const int total = items.total;
   const int nk_real = Kf / BK;                                    // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
@@ -330,12 +340,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const uint32_t z_voff = (uint32_t)tid * 16;
   // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo, bool offsets = RAGGED) {
-    int tm, tn, half;
-    item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, half);
-    int64_t row0 = (int64_t)tm * BM + half * 128;
+    int tm, tn, part;
+    item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, part);
+    int64_t row0 = (int64_t)tm * BM + part * (64 * MB);
     // RAGGED: a lower half that starts past the last row has nothing to fetch or store; it is pointed at the
     // upper half's rows (which exist) and its stores all fall to the clipping
-    if (RAGGED && MB == 2 && row0 >= Mf) row0 = (int64_t)tm * BM;
+    if (RAGGED && MB < 4 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
     if (RAGGED || offsets) {
@@ -416,26 +426,38 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
         if constexpr (MB == 4)
           asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        else
+        else if constexpr (MB == 2)
           asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+        else
+          asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
         clear_past_k(nxt);
       }
     }
     // Every wave's reads of stage I have returned (they fed `c`), and this wave's share of the copy into stage
     // I+1 has landed (the copies of the two younger steps may still be in flight); after the barrier that holds for
     // all waves: I+1 may be read, I may be overwritten.
+    // (the copies of the two younger steps, 2 * (MB + 4) of them, may still be in flight)
     if constexpr (MB == 4)
       asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    else
+    else if constexpr (MB == 2)
       asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     FENCE();
 #pragma unroll
     for (int n = 1; n < NM; ++n) {
-      if (n <= NR) rd(p, nxt, n - 1);
-      if constexpr (MB == 4) {
-        if (n >= 25 && n <= 60 && n % 5 == 0) dma_single(k + R, cur, n / 5 - 5, inner_);
+      if constexpr (MB == 1) {
+        // quarter tiles: 18 reads and 5 copies beside 15 MFMAs: two reads per MFMA, a copy with every third
+        if (2 * (n - 1) < NR) rd(p, nxt, 2 * (n - 1));
+        if (2 * (n - 1) + 1 < NR) rd(p, nxt, 2 * (n - 1) + 1);
+        if (n % 3 == 0) dma_single(k + R, cur, n / 3 - 1, inner_);
       } else {
-        if (n % 5 == 0 && n <= 30) dma_single(k + R, cur, n / 5 - 1, inner_);
+        if (n <= NR) rd(p, nxt, n - 1);
+        if constexpr (MB == 4) {
+          if (n >= 25 && n <= 60 && n % 5 == 0) dma_single(k + R, cur, n / 5 - 5, inner_);
+        } else {
+          if (n % 5 == 0 && n <= 30) dma_single(k + R, cur, n / 5 - 1, inner_);
+        }
       }
       mm(c, n);
       FENCE();
@@ -464,15 +486,17 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
   if constexpr (MB == 4)
     asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else
+  else if constexpr (MB == 2)
     asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(15) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
   for (int r = 0; r < NR; ++r) rd(f0, ring.s[0], r);
 
   for (; t < total; t += gridDim.x) {
-    int tm, tn, half;
-    item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, half);
-    const int64_t m0 = (int64_t)tm * BM + half * 128, n0 = (int64_t)tn * BN;
+    int tm, tn, part;
+    item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, part);
+    const int64_t m0 = (int64_t)tm * BM + part * (64 * MB), n0 = (int64_t)tn * BN;
 #pragma unroll
     for (int i = 0; i < NA; ++i)
 #pragma unroll
@@ -604,8 +628,9 @@ extern "C" {
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, OUT, EPI, false, false, 4, true>(g, ring);                                       \
-    fast::body<IN, OUT, EPI, false, false, 2, true>(g, ring);                                       \
+    fast::body<IN, OUT, EPI, false, false, 4, true, true>(g, ring);                                 \
+    fast::body<IN, OUT, EPI, false, false, 2, true, true>(g, ring);                                 \
+    fast::body<IN, OUT, EPI, false, false, 1, true, true>(g, ring);                                 \
   }
 #define GEMM_TILE_ALL_EPI(prefix, IN, OUT)             \
   GEMM_TILE(prefix##_epi0, IN, OUT, EPI_NONE)           \
@@ -625,8 +650,9 @@ GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, OUT, EPI, false, true, 4, true>(g, ring);                                        \
-    fast::body<IN, OUT, EPI, false, true, 2, true>(g, ring);                                        \
+    fast::body<IN, OUT, EPI, false, true, 4, true, true>(g, ring);                                  \
+    fast::body<IN, OUT, EPI, false, true, 2, true, true>(g, ring);                                  \
+    fast::body<IN, OUT, EPI, false, true, 1, true, true>(g, ring);                                  \
   }
 #define GEMM_TILE_RAGGED_ALL_EPI(prefix, IN, OUT)             \
   GEMM_TILE_RAGGED(prefix##_epi0, IN, OUT, EPI_NONE)           \

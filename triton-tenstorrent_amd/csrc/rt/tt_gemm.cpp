@@ -13,11 +13,14 @@ namespace {
 
 // Workgroups of the persistent macro-tile kernels: one per CU, or one per tile when there are fewer tiles.
 // The plain kernels (`splits`) finish a tail of at most grid/2 macro tiles as half tiles on twice the
-// workgroups, so a problem of at most CUs/2 tiles is launched with two workgroups per tile.
-uint32_t persistent_grid(int64_t tiles, bool splits) {
+// workgroups, so a problem of at most CUs/2 tiles is launched with two workgroups per tile; those that also have
+// the quarter-tile pass (`quarters`) get four workgroups per tile for a problem of at most CUs/4 tiles.
+uint32_t persistent_grid(int64_t tiles, bool splits, bool quarters = false) {
   const int64_t cus = props()->multiprocessor_count;
   if (tiles >= cus) return (uint32_t)cus;
-  if (splits && 2 * tiles <= cus && !env_int("TTAMD_GEMM_NO_SPLIT", 0)) return (uint32_t)(2 * tiles);
+  const bool no_split = env_int("TTAMD_GEMM_NO_SPLIT", 0) != 0;
+  if (quarters && 4 * tiles <= cus && !no_split) return (uint32_t)(4 * tiles);
+  if (splits && 2 * tiles <= cus && !no_split) return (uint32_t)(2 * tiles);
   return (uint32_t)tiles;
 }
 
@@ -130,7 +133,7 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
              epi);
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = persistent_grid(tiles, true);
+    const uint32_t wgs = persistent_grid(tiles, true, true);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
     // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
     static unsigned long long *probe_buf = nullptr;
