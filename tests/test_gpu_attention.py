@@ -276,3 +276,36 @@ def test_items_chained_inside_a_workgroup(causal, Z, H, S, D):
         ref = torch.softmax(s, -1) @ v[z, h].double()
         assert (o[z, h].double() - ref).abs().max() <= O_ATOL * max(1.0, float(v[z, h].float().abs().max()))
         assert (M[z, h].double() - torch.logsumexp(s, -1) / np.log(2.0)).abs().max() <= M_ATOL
+
+
+def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
+    """From the second call of a shape on, `_attn_fwd` is launched through a cached closure (N_CTX and the block
+    sizes arrive by keyword and are part of what makes two calls alike).  Batch, heads, operands and the mask may
+    change under it; whatever it does not recognise falls back to the full path."""
+    Z, H, S, D = 2, 3, 256, 128
+    q, k, v = (t.cuda() for t in _qkv(Z, H, S, D, seed=3))
+    sm = D ** -0.5
+    first_o, first_m = K.attention(q, k, v, True, sm, return_lse=True)
+    for _ in range(2):
+        o, m = K.attention(q, k, v, True, sm, return_lse=True)
+        assert torch.equal(o, first_o) and torch.equal(m, first_m)
+    assert K._attn_fwd._plan is not None
+    wo, wM = orc.attn_fwd(bits(q.cpu()), bits(k.cpu()), bits(v.cpu()), sm, causal=True, BLOCK_M=128, BLOCK_N=64)
+    assert np.max(np.abs(decode(first_o) - orc.from_bf16(wo))) <= O_ATOL
+    assert np.max(np.abs(first_m.cpu().numpy() - wM)) <= M_ATOL
+    # other operands, one head of one batch (Z = H = 1: values that Triton folds), the other mask, another length
+    q1, k1, v1 = q[:1, :1].contiguous(), k[:1, :1].contiguous(), v[:1, :1].contiguous()
+    o1 = K.attention(q1, k1, v1, True, sm)
+    assert torch.equal(o1, first_o[:1, :1])
+    of = K.attention(q, k, v, False, sm)
+    wo, _ = orc.attn_fwd(bits(q.cpu()), bits(k.cpu()), bits(v.cpu()), sm, causal=False, BLOCK_M=128, BLOCK_N=64)
+    assert np.max(np.abs(decode(of) - orc.from_bf16(wo))) <= O_ATOL
+    q2, k2, v2 = (t.cuda() for t in _qkv(1, 2, 384, D, seed=4))
+    o2 = K.attention(q2, k2, v2, True, sm)
+    wo, _ = orc.attn_fwd(bits(q2.cpu()), bits(k2.cpu()), bits(v2.cpu()), sm, causal=True, BLOCK_M=128, BLOCK_N=64)
+    assert np.max(np.abs(decode(o2) - orc.from_bf16(wo))) <= O_ATOL
+    assert torch.equal(K.attention(q, k, v, True, sm), first_o)
+    # and the same refusals
+    with pytest.raises(NotImplementedError):
+        K.attention(q.half(), k.half(), v.half(), True, sm)
+    assert torch.equal(K.attention(q, k, v, True, sm), first_o)

@@ -256,6 +256,51 @@ def _desc_matmul_direct(fn, bases: list, n_floats: int, tail: tuple):
     return direct
 
 
+def _attn_direct(fn, bases: list, tail: tuple):
+    """Repeat-launch closure of ``_attn_fwd`` (see ``_streaming_direct``): launch arguments sm_scale, M, Z, H, four
+    rank-2 descriptors, N_CTX; ``tail`` = (HEAD_DIM, BLOCK_M, BLOCK_N, STAGE).  The checks of the binder that the
+    library does not repeat (M: fp32, contiguous, Z*H*N_CTX elements) are made here; the rest is the library's."""
+    import torch
+    from ..tensor_descriptor import TensorDescriptor
+    dtypes = tuple(t.dtype for t in bases)
+    tensor_type, grid3, check, f32 = torch.Tensor, rt.Grid3, rt.check, torch.float32
+    blocks = [rt.tt_desc2d() for _ in bases]
+    for blk, t in zip(blocks, bases):
+        blk.dtype = _torch_dtype_code(t)
+    refs = [C.byref(b) for b in blocks]
+
+    def direct(args, grid, stream):
+        if len(args) != 9 or not 1 <= len(grid) <= 3:
+            return False
+        sm_scale, M, Z, H, n_ctx = args[0], args[1], args[2], args[3], args[8]
+        if (type(sm_scale) is not float or type(Z) is not int or type(H) is not int or type(n_ctx) is not int
+                or Z < 1 or H < 1 or not 0 < n_ctx < 2147483648 or Z * H >= 2147483648):
+            return False
+        if (type(M) is not tensor_type or M.dtype is not f32 or not M.is_cuda or M.numel() < Z * H * n_ctx
+                or not M.is_contiguous()):
+            return False
+        for g in grid:
+            if type(g) is not int:
+                return False
+        for blk, d, dt in zip(blocks, args[4:8], dtypes):
+            if type(d) is not TensorDescriptor:
+                return False
+            base, shape, strides = d.base, d.shape, d.strides
+            if (type(base) is not tensor_type or base.dtype is not dt or not base.is_cuda or len(shape) != 2
+                    or len(strides) != 2):
+                return False
+            blk.base = base.data_ptr()
+            blk.shape[0], blk.shape[1] = shape
+            blk.strides[0], blk.strides[1] = strides
+            blk.padding_nan = d.padding == "nan"
+        rc = fn(sm_scale, M.data_ptr(), Z, H, *refs, n_ctx, *tail, grid3(*(grid + (1, 1, 1))[:3]), stream)
+        if rc:
+            check(rc)
+        return True
+
+    return direct
+
+
 def _reduce_direct(fn, op_code: int, x_dtype, z_dtype, fixed: tuple):
     """Repeat-launch closure of ``reduce1d_kernel`` (see ``_streaming_direct``): the same checks as its binder for
     a call of the same shape, then the one C call.  ``fixed`` = (BLOCK, input, accumulate and output dtype codes,
@@ -533,9 +578,10 @@ def _bind_attn_fwd(lib, cur, consts, grid, stream):
         raise rt.InvalidLaunch(rt.RT_ERR_INVALID, "_attn_fwd: M must be a contiguous [Z,H,N_CTX] tensor")
     if consts.get("FP8_OUTPUT"):
         raise rt.Unsupported(rt.RT_ERR_UNSUPPORTED, "_attn_fwd: FP8_OUTPUT is not supported")
-    return lib.tt_attn_fwd(sm_scale, M.data_ptr(), Z, H, C.byref(q), C.byref(k), C.byref(v), C.byref(o), n_ctx,
-                           int(consts["HEAD_DIM"]), int(consts["BLOCK_M"]), int(consts["BLOCK_N"]),
-                           int(consts["STAGE"]), grid, stream)
+    tail = (int(consts["HEAD_DIM"]), int(consts["BLOCK_M"]), int(consts["BLOCK_N"]), int(consts["STAGE"]))
+    cur.direct = _attn_direct(lib.tt_attn_fwd, cur.keep[-4:], tail)
+    return lib.tt_attn_fwd(sm_scale, M.data_ptr(), Z, H, C.byref(q), C.byref(k), C.byref(v), C.byref(o), n_ctx, *tail,
+                           grid, stream)
 
 
 def _bind_matched(match: dict, lib, cur, consts, grid, stream):

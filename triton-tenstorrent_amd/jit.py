@@ -118,7 +118,8 @@ class PrebuiltKernel:
         self.fn = SimpleNamespace(arg_names=self.arg_names, __name__=name)
         self._cache: dict = {}
         # repeat launches: (number of positional arguments, keyword arguments, device, closure, the configuration's
-        # pre_hook or None, the arguments after the positional ones by name for that hook)
+        # pre_hook or None, the arguments after the positional ones by name for that hook and for a callable grid,
+        # the launch arguments among them in order or None)
         self._plan = None
         self._keep = None
         n_lead = next((i for i, n in enumerate(self.arg_names) if n in self.constexprs), len(self.arg_names))
@@ -164,7 +165,10 @@ class PrebuiltKernel:
                         plan[4](named)
                     if type(g) is not tuple:
                         g = g(named)
-                if type(g) is tuple and plan[3](args, g, stream):
+                # launch arguments that came by keyword (equal to the ones the plan was built with: see the guard) go
+                # to the closure in their positions
+                full = args if plan[6] is None else args + plan[6]
+                if type(g) is tuple and plan[3](full, g, stream):
                     self._keep = args   # launches are asynchronous: operands stay referenced until the next one
                     return self
         user_grid = grid
@@ -205,9 +209,10 @@ class PrebuiltKernel:
             launch_md = self.launch_metadata(grid, SimpleNamespace(name=self.name), bound)
         launcher(gx, gy, gz, stream, function, packed, launch_md, enter, exit_, *bound.values())
         direct = getattr(launcher, "direct", None)
-        if (direct is not None and _raw_stream is not None and len(args) == self._lead
+        if (direct is not None and _raw_stream is not None and self._lead is not None and len(args) <= self._lead
                 and (type(user_grid) is tuple or callable(user_grid)) and stream == _raw_stream()[1]):
             hook = config.pre_hook if config is not None else None
             rest = {n: bound[n] for n in self.arg_names[len(args):]}
-            self._plan = (len(args), dict(kwargs), device, direct, hook, rest)
+            by_keyword = tuple(bound[n] for n in self.arg_names[len(args):self._lead]) or None
+            self._plan = (len(args), dict(kwargs), device, direct, hook, rest, by_keyword)
         return self
