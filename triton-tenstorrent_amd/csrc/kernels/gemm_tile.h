@@ -31,6 +31,8 @@
 //   A: row m = 64 B = 4 chunks;   logical chunk c sits at c ^ a_swz((m>>2)&3)
 //   B: row k = 512 B = 32 chunks; logical chunk c sits at c ^ (((k&3)<<2) | (((k>>3)&1)<<1));
 //      the k rows are dealt to the four 4 KiB slabs as {0-3, 8-11}, {4-7, 12-15}, {16-19, 24-27}, {20-23, 28-31}
+// (The macro-tile pass of the plain row-major kernel keeps A differently: 128-byte rows holding two K steps, copied
+// as whole cache lines, see APAIR in body.)
 // A direct-to-LDS load writes lane l's 16 bytes at (wave-uniform base) + 16*l,
 // so thread t owns byte 16*t of every 4 KiB slab and the swizzle is applied to
 // the global address it fetches.
@@ -163,6 +165,9 @@ __device__ __forceinline__ void item_tile(const PassItems &p, int item, int tile
 // chunk position: the four positions of a pass must differ.  c ^ (row group) does not do that (measured: every A
 // read took twice its cycles, SQ_LDS_BANK_CONFLICT = a third of SQ_LDS_IDX_ACTIVE); this permutation does.
 __device__ __forceinline__ int a_swz(int row_group) { return (((row_group ^ (row_group >> 1)) & 1) << 1) | (row_group >> 1); }
+// The same for A rows of 128 bytes (8 chunks: two K steps side by side, the layout of the plain kernel's macro-tile
+// pass): two rows share a line of banks, so the eight even (odd) rows of a pass need eight different positions.
+__device__ __forceinline__ int a_swz_pair(int row) { return (row & 2) | ((row & 8) >> 1); }
 
 struct Ring {
   uint8_t *s[R];
@@ -243,6 +248,19 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int G4 = lane >> 4, i16 = lane & 15, q = i16 >> 2;
   constexpr int NA = 2 * MB;                 // A fragments of a wavefront's 32*MB rows; it has 8 B fragments
   const int a_pos = (wm * (32 * MB) + i16) * 64 + ((G4 ^ a_swz(q)) << 4);   // fragment i: + i * 1024
+  // APAIR (the macro-tile pass on whole row-major tiles): A is copied in 128-byte row segments, two K steps at a
+  // time, so that every request to the L2 is a whole cache line (64-byte segments are one request each too: 67 M
+  // of the 101 M read requests of an 8192^3 launch; with whole lines the kernel measured 4.3 % faster, timing-only
+  // variant).  The A regions of stages 2P and 2P+1 together hold the pair of steps (4n + 2P, 4n + 2P + 1): rows
+  // 0-127 of the macro tile in the first, rows 128-255 in the second, 128 bytes per row, step h in logical chunks
+  // 4h .. 4h+3.  A wavefront's rows all lie in region wm.
+  constexpr bool APAIR = !TILED && !RAGGED && MB == 4;
+  int a_pp[2];      // fragment i of step-half h: region base (stage 2P) + a_pp[h] + i * 2048
+#pragma unroll
+  for (int h = 0; h < 2; ++h) a_pp[h] = wm * STAGE + i16 * 128 + (((4 * h + G4) ^ a_swz_pair(i16)) << 4);
+  // copies of a pair: slab i (0..7) = rows 32i .. 32i+31; thread t: row t>>3, position t&7
+  const uint32_t a_voff_pair = (uint32_t)(((int64_t)(tid >> 3) * g.lda) * 2 + (((tid & 7) ^ a_swz_pair(tid >> 3)) << 4));
+  const int64_t a_slab32 = 32 * g.lda * 2;
   // k = 8*G4 + 4h + q lies in slab h + 2*(G4>>1), row q + 4*(G4&1) of it; its swizzle is (q<<2) | ((G4&1)<<1)
   const int b_base = A_BYTES + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
@@ -267,7 +285,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
   // The LDS reads of one step, in the order the MFMAs will want them:
   // b0.lo b0.hi a0 b1.lo b1.hi ... b7.lo b7.hi a1 ... a(NA-1)
-  auto rd = [&](Frags &f, const uint8_t *stage, int r) {
+  // (J: ring index of the stage, a constant wherever this is called)
+  auto rd = [&](Frags &f, const uint8_t *stage, int J, int r) {
+    if constexpr (APAIR) {
+      if (r == 2 || r >= 17) {
+        const int i = r == 2 ? 0 : r - 16;
+        f.a[i] = *(const vec *)(ring.s[J & 2] + a_pp[J & 1] + i * 2048);
+        return;
+      }
+    }
     if (r == 2) {
       f.a[0] = *(const vec *)(stage + a_pos);
     } else if (r < 17) {
@@ -409,6 +435,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     }
   };
 
+  // APAIR: copy number i (0..7) of the pair of steps (kk, kk+1), kk even, into pair buffer P
+  auto dma_pair = [&](int kk, int P, int i, auto inner_) {
+    constexpr bool inner = decltype(inner_)::value;
+    const bool over = !inner && kk >= nk;
+    const int k = over ? kk - nk : kk;
+    const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
+    dma_one(ap, a_voff_pair, ring.s[2 * P + (i >> 2)] + (i & 3) * 4096);
+  };
+
   // One step (K += 32) on ring stage I: the NM MFMAs on `c` (read from stage I during the previous step), the next
   // stage's fragments into `p`, and the refill of stage I itself with step k+R.
   //   The first MFMA goes out before the barrier, so that the matrix pipe has work while the wavefronts meet.
@@ -437,7 +472,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // I+1 has landed (the copies of the two younger steps may still be in flight); after the barrier that holds for
     // all waves: I+1 may be read, I may be overwritten.
     // (the copies of the two younger steps, 2 * (MB + 4) of them, may still be in flight)
-    if constexpr (MB == 4)
+    // APAIR: an odd step issues the 8 copies of the A pair whose buffer its barrier has freed (steps k+3, k+4) and
+    // then its 4 B copies, an even step only its 4 B copies; a barrier needs B of the next step and the A pair that
+    // step lies in, which on an even step leaves 4 + 8 + 4 younger copies in flight and on an odd one 4 + 4.
+    if constexpr (APAIR && (I & 1))
+      asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else if constexpr (MB == 4)
       asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else if constexpr (MB == 2)
       asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -448,12 +488,22 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     for (int n = 1; n < NM; ++n) {
       if constexpr (MB == 1) {
         // quarter tiles: 18 reads and 5 copies beside 15 MFMAs: two reads per MFMA, a copy with every third
-        if (2 * (n - 1) < NR) rd(p, nxt, 2 * (n - 1));
-        if (2 * (n - 1) + 1 < NR) rd(p, nxt, 2 * (n - 1) + 1);
+        if (2 * (n - 1) < NR) rd(p, nxt, (I + 1) % R, 2 * (n - 1));
+        if (2 * (n - 1) + 1 < NR) rd(p, nxt, (I + 1) % R, 2 * (n - 1) + 1);
         if (n % 3 == 0) dma_single(k + R, cur, n / 3 - 1, inner_);
       } else {
-        if (n <= NR) rd(p, nxt, n - 1);
-        if constexpr (MB == 4) {
+        if (n <= NR) rd(p, nxt, (I + 1) % R, n - 1);
+        if constexpr (APAIR) {
+          if constexpr (I & 1) {
+            if (n >= 26 && n <= 59 && (n - 26) % 3 == 0) {
+              const int c12 = (n - 26) / 3;
+              if (c12 < 8) dma_pair(k + 3, (I - 1) >> 1, c12, inner_);
+              else dma_single(k + R, cur, MB + c12 - 8, inner_);
+            }
+          } else {
+            if (n >= 30 && n <= 54 && (n - 30) % 8 == 0) dma_single(k + R, cur, MB + (n - 30) / 8, inner_);
+          }
+        } else if constexpr (MB == 4) {
           if (n >= 25 && n <= 60 && n % 5 == 0) dma_single(k + R, cur, n / 5 - 5, inner_);
         } else {
           if (n % 5 == 0 && n <= 30) dma_single(k + R, cur, n / 5 - 1, inner_);
@@ -474,24 +524,40 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   b_nxt = b_cur;
   vo_nxt = vo_cur;
   if constexpr (!RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
+  if constexpr (APAIR) {
+    // in the order the steps of a turn issue them: pair (0,1), B 0, B 1, B 2, pair (2,3), B 3
 #pragma unroll
-  for (int s = 0; s < R; ++s)
+    for (int i = 0; i < 8; ++i) dma_pair(0, 0, i, std::false_type{});
 #pragma unroll
-    for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
+    for (int s = 0; s < 3; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma_single(s, ring.s[s], MB + i, std::false_type{});
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_pair(2, 1, i, std::false_type{});
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_single(3, ring.s[3], MB + i, std::false_type{});
+  } else {
+#pragma unroll
+    for (int s = 0; s < R; ++s)
+#pragma unroll
+      for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
+  }
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
   if (RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     clear_past_k(ring.s[0]);
   }
   // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
-  if constexpr (MB == 4)
+  if constexpr (APAIR)
+    asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // pair (0,1) and B 0 have landed
+  else if constexpr (MB == 4)
     asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   else if constexpr (MB == 2)
     asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   else
     asm volatile("s_waitcnt vmcnt(15) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-  for (int r = 0; r < NR; ++r) rd(f0, ring.s[0], r);
+  for (int r = 0; r < NR; ++r) rd(f0, ring.s[0], 0, r);
 
   for (; t < total; t += gridDim.x) {
     int tm, tn, part;
