@@ -70,6 +70,22 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   int a_pos[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) a_pos[h] = a_base + (((2 * hi + h) ^ a_x) << 4);
+  // APAIR (the macro-tile pass on whole tiles), as in the 16-bit kernel: A is copied in 128-byte row segments, two K
+  // steps at a time, so that every request to the L2 is a whole cache line.  The A regions of stages 2P and 2P+1
+  // hold rows 0-127 and 128-255 of the macro tile for steps 4n + 2P and 4n + 2P + 1, 128 bytes per row, step s in
+  // logical chunks 4s .. 4s+3, chunk c at c ^ ((row >> 1) & 7): the sixteen lanes of a pass of a 16-byte read
+  // (rows {0-3, 12-15, 20-23, 24-27} or {4-7, 8-11, 16-19, 28-31} of a fragment, two rows to a line of banks) then
+  // meet sixteen different positions.
+  constexpr bool APAIR = !RAGGED && MB == 4;
+  int a_pp[2][2];      // [step of the pair][half of the lane's 32 bytes]: region base (stage 2P) + a_pp + i * 4096
+#pragma unroll
+  for (int st = 0; st < 2; ++st)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      a_pp[st][h] = wm * STAGE + l32 * 128 + (((4 * st + 2 * hi + h) ^ ((l32 >> 1) & 7)) << 4);
+  // copies of a pair: slab i (0..7) = rows 32i .. 32i+31; thread t: row t>>3, position t&7
+  const uint32_t a_voff_pair = (uint32_t)((int64_t)(tid >> 3) * g.lda + (((tid & 7) ^ ((tid >> 4) & 7)) << 4));
+  const int64_t a_slab32 = 32 * g.lda;
   const int G4 = lane >> 4, i16 = lane & 15, rj = i16 >> 1;
   int b_pos[4];
 #pragma unroll
@@ -88,11 +104,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
   // the 24 LDS reads of one step in the order the MFMAs want them (MB == 2: the first 20):
   // b0 (4 reads) a0 (2) b1 (4) b2 (4) b3 (4) a1 (2) a2 (2) a3 (2)
-  auto rd = [&](Frags &f, const uint8_t *stage, int r) {
+  // (J: ring index of the stage, a constant wherever this is called)
+  auto rd = [&](Frags &f, const uint8_t *stage, int J, int r) {
     auto rb = [&](int j, int q) {
       f.b[j].d[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2 *)(stage + b_pos[j] + q * 2048));
     };
-    auto ra = [&](int i, int h) { f.a[i].q[h] = *(const i32x4 *)(stage + a_pos[h] + i * 2048); };
+    auto ra = [&](int i, int h) {
+      if constexpr (APAIR) f.a[i].q[h] = *(const i32x4 *)(ring.s[J & 2] + a_pp[J & 1][h] + i * 4096);
+      else f.a[i].q[h] = *(const i32x4 *)(stage + a_pos[h] + i * 2048);
+    };
     if (r < 4) rb(0, r);
     else if (r < 6) ra(0, r - 4);
     else if (r < 18) rb(1 + (r - 6) / 4, (r - 6) % 4);
@@ -167,6 +187,14 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 #pragma unroll
       for (int j = 0; j < 4; ++j) asm volatile("" ::"a"(acc[i][j]));
   };
+  // APAIR: copy number i (0..7) of the pair of steps (kk, kk+1), kk even, into pair buffer P
+  auto dma_pair = [&](int kk, int P, int i, auto inner_) {
+    constexpr bool inner = decltype(inner_)::value;
+    const bool over = !inner && kk >= nk;
+    const int k = over ? kk - nk : kk;
+    const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
+    dma_one(ap, a_voff_pair, ring.s[2 * P + (i >> 2)] + (i & 3) * 4096);
+  };
   // One step (K += 64) on ring stage I: 16 MFMAs on `c` (read from stage I during the previous
   // step), the next stage's fragments into `p`, and the refill of stage I itself with step k+R.
   auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_) {
@@ -178,15 +206,32 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     // copy into stage I+1 has landed (the 16 younger copies may still be in flight); after the
     // barrier that holds for all waves: I+1 may be read, I may be overwritten
     if constexpr (MB == 4) {
-      asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      // APAIR: an odd step issues the 8 copies of the A pair whose buffer its barrier has freed (steps k+3, k+4) and
+      // then its 4 B copies, an even step only its 4 B copies; a barrier needs B of the next step and the A pair
+      // that step lies in, which on an even step leaves 4 + 8 + 4 younger copies in flight and on an odd one 4 + 4.
+      if constexpr (APAIR && (I & 1))
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else
+        asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       FENCE();
 #pragma unroll
       for (int n = 1; n < 16; ++n) {
         if (n <= 12) {
-          rd(p, nxt, 2 * (n - 1));
-          rd(p, nxt, 2 * (n - 1) + 1);
+          rd(p, nxt, (I + 1) % R, 2 * (n - 1));
+          rd(p, nxt, (I + 1) % R, 2 * (n - 1) + 1);
         }
-        if (n & 1) dma_single(k + R, cur, n >> 1, inner_); // one copy per two MFMAs: thin enough not to stall issue
+        if constexpr (APAIR) {
+          if constexpr (I & 1) {
+            if (n >= 3 && n <= 14) {          // twelve copies, one per MFMA (64 cycles)
+              if (n - 3 < 8) dma_pair(k + 3, (I - 1) >> 1, n - 3, inner_);
+              else dma_single(k + R, cur, MB + n - 11, inner_);
+            }
+          } else {
+            if (n >= 5 && n <= 14 && (n - 5) % 3 == 0) dma_single(k + R, cur, MB + (n - 5) / 3, inner_);
+          }
+        } else {
+          if (n & 1) dma_single(k + R, cur, n >> 1, inner_); // one copy per two MFMAs: thin enough not to stall issue
+        }
         mm(c, n);
         FENCE();
       }
@@ -198,7 +243,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 #pragma unroll
       for (int n = 1; n < 8; ++n) {
 #pragma unroll
-        for (int r = 3 * (n - 1); r < 3 * n && r < 20; ++r) rd(p, nxt, r);
+        for (int r = 3 * (n - 1); r < 3 * n && r < 20; ++r) rd(p, nxt, (I + 1) % R, r);
         if (n <= 6) dma_single(k + R, cur, n - 1, inner_);
         mm(c, n);
         FENCE();
@@ -222,17 +267,34 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   vo_nxt = vo_cur;
   if constexpr (!RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
   // fill the ring with steps 0..R-1
+  if constexpr (APAIR) {
+    // in the order the steps of a turn issue them: pair (0,1), B 0, B 1, B 2, pair (2,3), B 3
 #pragma unroll
-  for (int s = 0; s < R; ++s)
+    for (int i = 0; i < 8; ++i) dma_pair(0, 0, i, std::false_type{});
 #pragma unroll
-    for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
-  // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
-  if constexpr (MB == 4)
+    for (int s = 0; s < 3; ++s)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dma_single(s, ring.s[s], MB + i, std::false_type{});
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dma_pair(2, 1, i, std::false_type{});
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma_single(3, ring.s[3], MB + i, std::false_type{});
+  } else {
+#pragma unroll
+    for (int s = 0; s < R; ++s)
+#pragma unroll
+      for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
+  }
+  // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight (APAIR: B 1, B 2, the
+  // second pair and B 3)
+  if constexpr (APAIR)
+    asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else if constexpr (MB == 4)
     asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   else
     asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-  for (int r = 0; r < 16 + 2 * MB; ++r) rd(f0, ring.s[0], r);
+  for (int r = 0; r < 16 + 2 * MB; ++r) rd(f0, ring.s[0], 0, r);
 
   for (; t < total; t += gridDim.x) {
     int tm, tn, half;
