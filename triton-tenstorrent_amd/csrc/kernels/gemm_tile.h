@@ -248,19 +248,20 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int G4 = lane >> 4, i16 = lane & 15, q = i16 >> 2;
   constexpr int NA = 2 * MB;                 // A fragments of a wavefront's 32*MB rows; it has 8 B fragments
   const int a_pos = (wm * (32 * MB) + i16) * 64 + ((G4 ^ a_swz(q)) << 4);   // fragment i: + i * 1024
-  // APAIR (the macro-tile pass on whole row-major tiles): A is copied in 128-byte row segments, two K steps at a
+  // APAIR (the macro-tile pass on row-major operands): A is copied in 128-byte row segments, two K steps at a
   // time, so that every request to the L2 is a whole cache line (64-byte segments are one request each too: 67 M
   // of the 101 M read requests of an 8192^3 launch; with whole lines the kernel measured 4.3 % faster, timing-only
   // variant).  The A regions of stages 2P and 2P+1 together hold the pair of steps (4n + 2P, 4n + 2P + 1): rows
   // 0-127 of the macro tile in the first, rows 128-255 in the second, 128 bytes per row, step h in logical chunks
   // 4h .. 4h+3.  A wavefront's rows all lie in region wm.
-  constexpr bool APAIR = !TILED && !RAGGED && MB == 4;
+  constexpr bool APAIR = !TILED && MB == 4;
   int a_pp[2];      // fragment i of step-half h: region base (stage 2P) + a_pp[h] + i * 2048
 #pragma unroll
   for (int h = 0; h < 2; ++h) a_pp[h] = wm * STAGE + i16 * 128 + (((4 * h + G4) ^ a_swz_pair(i16)) << 4);
   // copies of a pair: slab i (0..7) = rows 32i .. 32i+31; thread t: row t>>3, position t&7
   const uint32_t a_voff_pair = (uint32_t)(((int64_t)(tid >> 3) * g.lda) * 2 + (((tid & 7) ^ a_swz_pair(tid >> 3)) << 4));
   const int64_t a_slab32 = 32 * g.lda * 2;
+  const int pair_r8 = tid >> 3, pair_c = (tid & 7) ^ a_swz_pair(tid >> 3);   // row in the slab, logical chunk
   // k = 8*G4 + 4h + q lies in slab h + 2*(G4>>1), row q + 4*(G4&1) of it; its swizzle is (q<<2) | ((G4&1)<<1)
   const int b_base = A_BYTES + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
@@ -335,15 +336,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if constexpr (RAGGED) {
       typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
       // A: this thread's chunk holds k = 8*a_chunk .. 8*a_chunk + 7 of one row, two per 32-bit word
-      const int ka = a_chunk * 8;
-      u32x4 keep;
+      // (APAIR keeps A in pairs of steps and clears them by the pair, clear_pair)
+      if constexpr (!APAIR) {
+        const int ka = a_chunk * 8;
+        u32x4 keep;
 #pragma unroll
-      for (int w = 0; w < 4; ++w)
-        keep[w] = (ka + 2 * w + 1 < k_tail) ? 0xffffffffu : (ka + 2 * w < k_tail) ? 0x0000ffffu : 0u;
+        for (int w = 0; w < 4; ++w)
+          keep[w] = (ka + 2 * w + 1 < k_tail) ? 0xffffffffu : (ka + 2 * w < k_tail) ? 0x0000ffffu : 0u;
 #pragma unroll
-      for (int i = 0; i < MB; ++i) {
-        lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + i * 4096 + lds_wave + lane * 16);
-        *p = *p & keep;
+        for (int i = 0; i < MB; ++i) {
+          lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + i * 4096 + lds_wave + lane * 16);
+          *p = *p & keep;
+        }
       }
       // B: this thread's sixteen bytes of slab i lie in k row b_row0(i) + b_kk
 #pragma unroll
@@ -361,7 +365,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // RAGGED: per-thread byte offsets of a tile's copies, rows and column chunks clamped into the matrix.
   // The A offsets then carry the whole row offset from the tile's first row (a clamp can point backwards
   // from a slab's own first row, and the instruction's register offset is unsigned).
-  struct Voffs { uint32_t a[4]; uint32_t b; };
+  struct Voffs { uint32_t a[4]; uint32_t b; int last_row; };
   Voffs vo_cur, vo_nxt;
   const uint32_t z_voff = (uint32_t)tid * 16;
   // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
@@ -378,6 +382,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       // per-thread offsets of the tile's copies from ap / bp, one per A slab (RAGGED: rows and column chunks
       // clamped into the matrix)
       const int last_row = RAGGED ? Mf - 1 - (int)row0 : BM;  // >= 0
+      vo.last_row = last_row;
       const int last_chunk = RAGGED ? (Nf - tn * BN) / 8 - 1 : 32;   // >= 0: the fetchable N is a multiple of 8
 #pragma unroll
       for (int i = 0; i < MB; ++i) {
@@ -440,8 +445,43 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
-    const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
-    dma_one(ap, a_voff_pair, ring.s[2 * P + (i >> 2)] + (i & 3) * 4096);
+    uint8_t *dst = ring.s[2 * P + (i >> 2)] + (i & 3) * 4096;
+    if constexpr (RAGGED) {
+      // rows past M are fetched from the last row; a pair that ends past K (K is a multiple of 8) fetches the
+      // chunks past K from the pair's first chunk, which exists, and clear_pair zeroes them once they have landed;
+      // a pair that starts at or past K comes from the page of zeros
+      const int valid = inner ? 64 : min(max(g.K - 32 * k, 0), 64);
+      const int last_row = (over ? vo_nxt : vo_cur).last_row;
+      if constexpr (decltype(inner_)::value == 2) {
+        // a whole pair of a tile that lies inside the matrix (all but the last row of tiles; the caller knows):
+        // nothing depends on the lane but the constant offset.  It matters: between two 16-cycle MFMAs a lone
+        // wavefront has room for three other instructions, and the half dozen VALU operations of the path below,
+        // once per copy, cost the kernel 8 % (a branch per copy instead cost more).
+        dma_one(a_cur + (int64_t)(k >> 1) * 128 + i * a_slab32, a_voff_pair, dst);
+      } else {
+        // (worked out here, from one register each: left free, the compiler keeps the eight slabs' rows in
+        // registers from the start of the kernel, spills them, and a reload in a step drains the copies in flight)
+        int r8 = pair_r8, c = pair_c;
+        asm volatile("" : "+v"(r8), "+v"(c));
+        const int row = min(i * 32 + r8, last_row);
+        if (!inner && 8 * c + 8 > valid) c = 0;
+        const uint32_t voff = (uint32_t)row * (uint32_t)(g.lda * 2) + (uint32_t)c * 16;
+        const uint8_t *ap = valid == 0 ? zero_page : (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128;
+        dma_one(ap, valid == 0 ? z_voff : voff, dst);
+      }
+    } else {
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
+      dma_one(ap, a_voff_pair, dst);
+    }
+  };
+  // RAGGED APAIR: this thread's sixteen bytes of each slab of pair buffer P, when they hold k at or past `valid`
+  auto clear_pair = [&](int P, int valid) {
+    typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+    if (8 * pair_c + 8 > valid) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *(lds_u32x4 *)(lds_void *)(ring.s[2 * P + (i >> 2)] + (i & 3) * 4096 + lds_wave + lane * 16) = (u32x4){0, 0, 0, 0};
+    }
   };
 
   // One step (K += 32) on ring stage I: the NM MFMAs on `c` (read from stage I during the previous step), the next
@@ -458,8 +498,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     mm(c, 0);
     FENCE();
     if constexpr (RAGGED && !decltype(inner_)::value) {
+      if constexpr (APAIR && (I & 1)) {
+        // the pair about to open (its first step is the next one) ends past K: clear what lies past
+        const int valid = min(max(g.K - 32 * (k + 1 == nk ? 0 : k + 1), 0), 64);
+        if (valid > 0 && valid < 64) {
+          asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+          clear_pair(((I + 1) % R) >> 1, valid);
+        }
+      }
       if (k_tail && (k + 1 == nk ? 0 : k + 1) == nk_real - 1) {   // the stage about to open holds a tile's last data step
-        if constexpr (MB == 4)
+        if constexpr (APAIR && (I & 1))
+          asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else if constexpr (MB == 4)
           asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
         else if constexpr (MB == 2)
           asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
@@ -547,6 +597,13 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     clear_past_k(ring.s[0]);
   }
+  if constexpr (RAGGED && APAIR) {
+    if (g.K < 128 && (g.K & 63)) {          // one of the first tile's two pairs ends past K
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (g.K < 64) clear_pair(0, g.K);
+      else clear_pair(1, g.K - 64);
+    }
+  }
   // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
   if constexpr (APAIR)
     asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // pair (0,1) and B 0 have landed
@@ -573,6 +630,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // (row-major operands whose last step ends past K: that step's copies need the redirection above, so it stays
     // out of these turns)
     const int nk_inner = nk_real - ((!TILED && k_tail) ? 1 : 0);
+    if (RAGGED && APAIR && __builtin_amdgcn_readfirstlane(vo_cur.last_row) >= BM - 1) {
+      // (a tile whose 256 rows all exist: the copies of A need no clamping)
+      for (; k + 2 * R <= nk_inner; k += R) {
+        step(std::integral_constant<int, 0>{}, k, f0, f1, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::integral_constant<int, 2>{});
+      }
+    }
     for (; k + 2 * R <= nk_inner; k += R) {
       step(std::integral_constant<int, 0>{}, k, f0, f1, std::true_type{});
       step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::true_type{});
