@@ -70,13 +70,13 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   int a_pos[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) a_pos[h] = a_base + (((2 * hi + h) ^ a_x) << 4);
-  // APAIR (the macro-tile pass on whole tiles), as in the 16-bit kernel: A is copied in 128-byte row segments, two K
+  // APAIR (the macro-tile pass), as in the 16-bit kernel: A is copied in 128-byte row segments, two K
   // steps at a time, so that every request to the L2 is a whole cache line.  The A regions of stages 2P and 2P+1
   // hold rows 0-127 and 128-255 of the macro tile for steps 4n + 2P and 4n + 2P + 1, 128 bytes per row, step s in
   // logical chunks 4s .. 4s+3, chunk c at c ^ ((row >> 1) & 7): the sixteen lanes of a pass of a 16-byte read
   // (rows {0-3, 12-15, 20-23, 24-27} or {4-7, 8-11, 16-19, 28-31} of a fragment, two rows to a line of banks) then
   // meet sixteen different positions.
-  constexpr bool APAIR = !RAGGED && MB == 4;
+  constexpr bool APAIR = MB == 4;
   int a_pp[2][2];      // [step of the pair][half of the lane's 32 bytes]: region base (stage 2P) + a_pp + i * 4096
 #pragma unroll
   for (int st = 0; st < 2; ++st)
@@ -86,6 +86,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   // copies of a pair: slab i (0..7) = rows 32i .. 32i+31; thread t: row t>>3, position t&7
   const uint32_t a_voff_pair = (uint32_t)((int64_t)(tid >> 3) * g.lda + (((tid & 7) ^ ((tid >> 4) & 7)) << 4));
   const int64_t a_slab32 = 32 * g.lda;
+  const int pair_r8 = tid >> 3, pair_c = (tid & 7) ^ ((tid >> 4) & 7);   // row in the slab, logical chunk
   const int G4 = lane >> 4, i16 = lane & 15, rj = i16 >> 1;
   int b_pos[4];
 #pragma unroll
@@ -131,7 +132,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
                  : "memory", "m0");
   };
   const uint8_t *a_cur, *b_cur, *a_nxt, *b_nxt;
-  struct Voffs { uint32_t a[4]; uint32_t b; };   // RAGGED: a tile's per-thread offsets, clamped into the matrix
+  struct Voffs { uint32_t a[4]; uint32_t b; int last_row; };   // RAGGED: a tile's per-thread offsets, clamped into the matrix
   Voffs vo_cur, vo_nxt;
   const uint32_t z_voff = (uint32_t)tid * 16;
   // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
@@ -146,6 +147,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     bp = B + (int64_t)tn * BN;
     if (RAGGED || offsets) {
       const int last_row = RAGGED ? g.M - 1 - (int)row0 : BM;
+      vo.last_row = last_row;
       const int last_chunk = RAGGED ? (g.N - tn * BN) / 16 - 1 : 16;        // N is a multiple of 16
 #pragma unroll
       for (int i = 0; i < MB; ++i) vo.a[i] = (uint32_t)((int64_t)min(i * 64 + a_row, last_row) * g.lda + a_chunk * 16);
@@ -192,8 +194,39 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
-    const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
-    dma_one(ap, a_voff_pair, ring.s[2 * P + (i >> 2)] + (i & 3) * 4096);
+    uint8_t *dst = ring.s[2 * P + (i >> 2)] + (i & 3) * 4096;
+    if constexpr (RAGGED) {
+      // as in the 16-bit kernel: rows past M come from the last row; K is a whole number of steps here, so a pair
+      // holds 128, 64 (its second step is padding: fetched from the pair's first chunk, cleared by clear_pair) or 0
+      // bytes (the page of zeros) of each row; the turns of a tile whose 256 rows all exist take the form without
+      // any of this (value 2), because the VALU operations below, once per copy, would cost more than the whole
+      // lines gain
+      if constexpr (decltype(inner_)::value == 2) {
+        dma_one(a_cur + (int64_t)(k >> 1) * 128 + i * a_slab32, a_voff_pair, dst);
+      } else {
+        const int valid = inner ? 128 : min(max(g.K - 64 * k, 0), 128);
+        int r8 = pair_r8, c = pair_c;
+        asm volatile("" : "+v"(r8), "+v"(c));
+        const int row = min(i * 32 + r8, (over ? vo_nxt : vo_cur).last_row);
+        if (!inner && 16 * c + 16 > valid) c = 0;
+        const uint32_t voff = (uint32_t)row * (uint32_t)g.lda + (uint32_t)c * 16;
+        const uint8_t *ap = valid == 0 ? fast::zero_page : (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128;
+        dma_one(ap, valid == 0 ? z_voff : voff, dst);
+      }
+    } else {
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
+      dma_one(ap, a_voff_pair, dst);
+    }
+  };
+  // RAGGED: this thread's sixteen bytes of each slab of pair buffer P, when they belong to the pair's second step
+  // and that step is padding
+  auto clear_pair = [&](int P) {
+    typedef __attribute__((address_space(3))) i32x4 lds_i32x4;
+    if (pair_c >= 4) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *(lds_i32x4 *)(lds_void *)(ring.s[2 * P + (i >> 2)] + (i & 3) * 4096 + lds_wave + lane * 16) = (i32x4){0, 0, 0, 0};
+    }
   };
   // One step (K += 64) on ring stage I: 16 MFMAs on `c` (read from stage I during the previous
   // step), the next stage's fragments into `p`, and the refill of stage I itself with step k+R.
@@ -209,6 +242,14 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
       // APAIR: an odd step issues the 8 copies of the A pair whose buffer its barrier has freed (steps k+3, k+4) and
       // then its 4 B copies, an even step only its 4 B copies; a barrier needs B of the next step and the A pair
       // that step lies in, which on an even step leaves 4 + 8 + 4 younger copies in flight and on an odd one 4 + 4.
+      if constexpr (RAGGED && APAIR && (I & 1) && !decltype(inner_)::value) {
+        // the pair about to open (its first step is the next one) has a padding step for its second: clear it
+        const int kn = k + 1 == nk ? 0 : k + 1;
+        if (g.K - 64 * kn == 64) {
+          asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+          clear_pair(((I + 1) % R) >> 1);
+        }
+      }
       if constexpr (APAIR && (I & 1))
         asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       else
@@ -285,6 +326,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 #pragma unroll
       for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
   }
+  if constexpr (RAGGED && APAIR) {
+    if (g.K < 256 && (g.K & 127)) {          // one of the first tile's two pairs ends in a padding step
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      clear_pair(g.K < 128 ? 0 : 1);
+    }
+  }
   // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight (APAIR: B 1, B 2, the
   // second pair and B 3)
   if constexpr (APAIR)
@@ -306,6 +353,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
       for (int j = 0; j < 4; ++j) acc[i][j] = (f32x16){0};
     int k = 0;
     // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
+    if (RAGGED && APAIR && __builtin_amdgcn_readfirstlane(vo_cur.last_row) >= BM - 1) {
+      // (a tile whose 256 rows all exist: the copies of A need no clamping)
+      for (; k + 2 * R <= nk_real; k += R) {
+        step(std::integral_constant<int, 0>{}, k, f0, f1, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::integral_constant<int, 2>{});
+      }
+    }
     for (; k + 2 * R <= nk_real; k += R) {
       step(std::integral_constant<int, 0>{}, k, f0, f1, std::true_type{});
       step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::true_type{});
