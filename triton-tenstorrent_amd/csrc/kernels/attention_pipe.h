@@ -140,9 +140,32 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
     if (r < PPT) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, k_voff, lds + stage_o + (r % PPT) * 8192);
     else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, v_voff, lds + VBASE + stage_o + (r % PPT) * 8192);
   };
+  // The same for whole blocks only, from two running pointers (K and V rows of the block that is fetched next) instead
+  // of a 64-bit product per piece: the pieces of a block are issued in order and the pointers step after the last one,
+  // into the next item's keys when this item's run out.
+  const int64_t kstep = (int64_t)BN * a.ldk * 2, vstep = (int64_t)BN * a.ldv * 2;
+  const int64_t kpiece = (int64_t)RPP * a.ldk * 2, vpiece = (int64_t)RPP * a.ldv * 2;
+  const uint8_t *kp = kg + 3 * kstep, *vp = vg + 3 * vstep;   // block 3: blocks 0..2 are the prologue's (or the item before's)
+  auto dma_run = [&](int blk, int stage_o, int r) {
+    if constexpr (RAGGED) {
+      dma_piece(blk, stage_o, r);
+    } else {
+      if (r < PPT) dma_one(kp + (r % PPT) * kpiece, k_voff, lds + stage_o + (r % PPT) * 8192);
+      else dma_one(vp + (r % PPT) * vpiece, v_voff, lds + VBASE + stage_o + (r % PPT) * 8192);
+      if (r == 2 * PPT - 1) {
+        const bool wrap = blk + 1 == nstream;
+        kp = wrap ? kg_next : kp + kstep;
+        vp = wrap ? vg_next : vp + vstep;
+      }
+    }
+  };
   auto dma_block = [&](int blk, int stage_o) {
 #pragma unroll
     for (int r = 0; r < 2 * PPT; ++r) dma_piece(blk, stage_o, r);
+  };
+  auto dma_block_run = [&](int blk, int stage_o) {
+#pragma unroll
+    for (int r = 0; r < 2 * PPT; ++r) dma_run(blk, stage_o, r);
   };
 
   // ---- fragment addresses ----
@@ -278,12 +301,12 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
         if (i % PRIO_STEP == 0) set_prio(PIPE_PRIO_OF(i / PRIO_STEP, 2 * DK / PRIO_STEP));
         if (i % GK == 0 && i + GK < 2 * DK) {
 #pragma unroll
-          for (int g = 0; g < GK; ++g) kf[(i + GK + g) % (2 * GK)] = rdK(nxt, i + GK + g);
+          for (int g = GK - 1; g >= 0; --g) kf[(i + GK + g) % (2 * GK)] = rdK(nxt, i + GK + g);
         }
         sn[i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i % (2 * GK)], qf[i >> 1].v, sn[i & 1], 0, 0, 0);
         if (i == 2 * DK - 4) {
 #pragma unroll
-          for (int g = 0; g < GV; ++g) vpre[g] = rdV(cur, g);
+          for (int g = GV - 1; g >= 0; --g) vpre[g] = rdV(cur, g);
         }
         // the softmax of block j in 16 work items, SPS of them per MFMA: four partial maxima, the statistics (and
         // the rescale, when there is one), a gap, then 10 of the 16 pairs of exponentials
@@ -326,13 +349,13 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
       if (i % PRIO_STEP == 0) set_prio(PIPE_PRIO_OF(i / PRIO_STEP, 4 * DT / PRIO_STEP));
       if (i % GV == 0 && i + GV < 4 * DT) {
 #pragma unroll
-        for (int g = 0; g < GV; ++g) vf[(i + GV + g) % (2 * GV)] = rdV(cur, i + GV + g);
+        for (int g = GV - 1; g >= 0; --g) vf[(i + GV + g) % (2 * GV)] = rdV(cur, i + GV + g);
       }
       acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[i % (2 * GV)], pfrag(k4), acc[t], 0, 0, 0);
-      if (i % (SLOTS / (2 * PPT)) == 1) dma_piece(j + 3, free_o, i / (SLOTS / (2 * PPT)));
+      if (i % (SLOTS / (2 * PPT)) == 1) dma_run(j + 3, free_o, i / (SLOTS / (2 * PPT)));
       if (!LAST && i == 4 * DT - 4) {
 #pragma unroll
-        for (int g = 0; g < GK; ++g) kpre[g] = rdK(lds + nn_o, g);
+        for (int g = GK - 1; g >= 0; --g) kpre[g] = rdK(lds + nn_o, g);
       }
 #pragma unroll
       for (int w = i * SPS; w < (i + 1) * SPS; ++w) {
@@ -384,7 +407,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   // cur_o is the stage of block j
   for (; j < nstream; ++j) {
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    dma_block(j + 3, nx(nx(nx(cur_o))));
+    dma_block_run(j + 3, nx(nx(nx(cur_o))));
     cur_o = nx(cur_o);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the trailing copies land before the stages are reused or released
