@@ -6,8 +6,8 @@
 // direct-to-LDS copies three steps ahead, persistent XCD-aware grid, transposed product so
 // that the epilogue stores 4 consecutive n per lane.  What differs:
 //   * one step is K = 64 (64 one-byte elements per A row = the same 64 bytes as 32 bf16),
-//     consumed by ONE v_mfma_scale_f32_32x32x64_f8f6f4 per accumulator (block scales fixed
-//     at 1.0 = E8M0 0x7f; the per-tensor scales are applied in the epilogue);
+//     consumed by ONE v_mfma_f32_32x32x64_f8f6f4 per accumulator (no block scales, i.e. 1.0;
+//     the per-tensor scales are applied in the epilogue);
 //   * a lane's operand is 32 bytes: k = 32*(lane/32) .. +31.  A rows are k-contiguous: two
 //     ds_read_b128.  B is [K,N] with n contiguous: ds_read_b64_tr_b8 transposes an 8x16
 //     block of bytes across 16 lanes (result lane i, byte j = source lane 2j + i/8, byte
@@ -121,8 +121,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   };
   auto mm = [&](Frags &f, int n) {
     const int i = n >> 2, j = n & 3;
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j].v, f.a[i].v, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                 0x7f7f7f7f);
+    // both scale operands the constant 0: the compiler then emits the instruction without its scale-loading half
+    // (v_mfma_f32_32x32x64_f8f6f4, block scales 1.0), half the code bytes and one operand read less per MFMA
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j].v, f.a[i].v, acc[i][j], 0, 0, 0, 0, 0, 0);
   };
   auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
