@@ -262,6 +262,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const uint32_t a_voff_pair = (uint32_t)(((int64_t)(tid >> 3) * g.lda) * 2 + (((tid & 7) ^ a_swz_pair(tid >> 3)) << 4));
   const int64_t a_slab32 = 32 * g.lda * 2;
   const int pair_r8 = tid >> 3, pair_c = (tid & 7) ^ a_swz_pair(tid >> 3);   // row in the slab, logical chunk
+  // APAIR on whole tiles: a slab's distance from the first one rides in the thread's offset register, one register
+  // per slab, so that the copies of a step share one scalar address: two scalar additions less per copy, and with
+  // one wavefront per SIMD every instruction between two MFMAs counts (two more scalar instructions per copy cost
+  // 2.6 %).  The clamping kernel has no registers to spare for it (it measured 1.5 % slower with them).
+  uint32_t a_vp[8], b_vs[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a_vp[i] = a_voff_pair + (uint32_t)(i * a_slab32);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) b_vs[i] = b_voff + (uint32_t)b_slab_off(i);
   // k = 8*G4 + 4h + q lies in slab h + 2*(G4>>1), row q + 4*(G4&1) of it; its swizzle is (q<<2) | ((G4&1)<<1)
   const int b_base = A_BYTES + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
@@ -319,10 +328,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // s_waitcnt vmcnt(n) for exactly the copies that the following reads depend on.
   auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+    // (m0 is the compiler's to write: it then sees a scalar instruction between the MFMA before and this statement
+    // and does not pad with a wait state of its own; the one M0 needs before the copy reads it stays in here)
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(m0v), "v"(voff), "s"(src_uniform)
-                 : "memory", "m0");
+                 : "{m0}"(m0v), "v"(voff), "s"(src_uniform)
+                 : "memory");
   };
 
   // RAGGED with K not a multiple of 32: the last step of every tile holds columns (A) and rows (B) past K:
@@ -407,6 +418,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if constexpr (inner) {
       if (i < MB)
         dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
+      else if constexpr (APAIR && !RAGGED)
+        dma_one(b_cur + (int64_t)k * b_kstep, b_vs[i - MB], stage + A_BYTES + (i - MB) * 4096);
       else
         dma_one(b_cur + (int64_t)k * b_kstep + b_slab_off(i - MB), vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
     } else if constexpr (RAGGED) {
@@ -436,7 +449,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
-      dma_one(bp + b_slab_off(i - MB), b_voff, stage + A_BYTES + (i - MB) * 4096);
+      if constexpr (APAIR) dma_one(bp, b_vs[i - MB], stage + A_BYTES + (i - MB) * 4096);
+      else dma_one(bp + b_slab_off(i - MB), b_voff, stage + A_BYTES + (i - MB) * 4096);
     }
   };
 
@@ -470,8 +484,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         dma_one(ap, valid == 0 ? z_voff : voff, dst);
       }
     } else {
-      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128 + i * a_slab32;
-      dma_one(ap, a_voff_pair, dst);
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)(k >> 1) * 128;
+      dma_one(ap, a_vp[i], dst);
     }
   };
   // RAGGED APAIR: this thread's sixteen bytes of each slab of pair buffer P, when they hold k at or past `valid`

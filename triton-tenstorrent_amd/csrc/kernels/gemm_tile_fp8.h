@@ -127,10 +127,11 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   };
   auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+    // (m0 written by the compiler, as in the 16-bit kernel)
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(m0v), "v"(voff), "s"(src_uniform)
-                 : "memory", "m0");
+                 : "{m0}"(m0v), "v"(voff), "s"(src_uniform)
+                 : "memory");
   };
   const uint8_t *a_cur, *b_cur, *a_nxt, *b_nxt;
   struct Voffs { uint32_t a[4]; uint32_t b; int last_row; };   // RAGGED: a tile's per-thread offsets, clamped into the matrix
