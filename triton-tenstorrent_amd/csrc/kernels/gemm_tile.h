@@ -82,11 +82,27 @@ template <> struct MFMA<DT_BF16> {
   static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
+  // The MFMA and, behind it, one direct-to-LDS copy (m0: its LDS destination, written by the compiler in front of
+  // the statement): the MFMA is the wait state that the copy needs after a write to m0.
+  static __device__ __forceinline__ void run_copy(vec a, vec b, f32x4 &c, uint32_t m0v, uint32_t voff, const uint8_t *src) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
+                 : "memory");
+  }
 };
 template <> struct MFMA<DT_F16> {
   typedef f16x8 vec;
   static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  // The MFMA and, behind it, one direct-to-LDS copy (m0: its LDS destination, written by the compiler in front of
+  // the statement): the MFMA is the wait state that the copy needs after a write to m0.
+  static __device__ __forceinline__ void run_copy(vec a, vec b, f32x4 &c, uint32_t m0v, uint32_t voff, const uint8_t *src) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
+                 : "memory");
   }
 };
 
@@ -326,7 +342,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // unrelated), which would flatten the multi-step prefetch.  Completion is tracked by
   // hand instead: copies retire in issue order, and each step's barrier waits with
   // s_waitcnt vmcnt(n) for exactly the copies that the following reads depend on.
-  auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+  auto dma_plain = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
     // (m0 is the compiler's to write: it then sees a scalar instruction between the MFMA before and this statement
     // and does not pad with a wait state of its own; the one M0 needs before the copy reads it stays in here)
@@ -334,6 +350,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                  :
                  : "{m0}"(m0v), "v"(voff), "s"(src_uniform)
                  : "memory");
+  };
+  // MFMA number n of a step and a copy in one statement (inside the K loop every copy rides behind an MFMA)
+  auto mm_copy = [&](Frags &f, int n, const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+    const int i = n >> 3, j = (i & 1) ? 7 - (n & 7) : (n & 7);
+    const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
+    X::run_copy(f.b[j].v, f.a[i], acc[i][j], m0v, voff, src_uniform);
   };
 
   // RAGGED with K not a multiple of 32: the last step of every tile holds columns (A) and rows (B) past K:
@@ -411,10 +433,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // `inner`: the caller knows that step kk belongs to this tile and carries data, so the choices between this
   // tile and the next and (RAGGED) between data and the page of zeros are not made at run time, and a copy's
   // source is one scalar address per operand and step plus the thread's offset for that slab
-  auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_) {
+  // (f, n: the MFMA that the copy is issued behind, n < 0: none)
+  auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_, Frags &f, int n) {
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
+    auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+      if (n >= 0) mm_copy(f, n, src_uniform, voff, dst_slab);
+      else dma_plain(src_uniform, voff, dst_slab);
+    };
     if constexpr (inner) {
       if (i < MB)
         dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
@@ -455,10 +482,14 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   };
 
   // APAIR: copy number i (0..7) of the pair of steps (kk, kk+1), kk even, into pair buffer P
-  auto dma_pair = [&](int kk, int P, int i, auto inner_) {
+  auto dma_pair = [&](int kk, int P, int i, auto inner_, Frags &f, int n) {
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
+    auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
+      if (n >= 0) mm_copy(f, n, src_uniform, voff, dst_slab);
+      else dma_plain(src_uniform, voff, dst_slab);
+    };
     uint8_t *dst = ring.s[2 * P + (i >> 2)] + (i & 3) * 4096;
     if constexpr (RAGGED) {
       // rows past M are fetched from the last row; a pair that ends past K (K is a multiple of 8) fetches the
@@ -550,30 +581,44 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     FENCE();
 #pragma unroll
     for (int n = 1; n < NM; ++n) {
+      bool with_copy = false;
       if constexpr (MB == 1) {
         // quarter tiles: 18 reads and 5 copies beside 15 MFMAs: two reads per MFMA, a copy with every third
         if (2 * (n - 1) < NR) rd(p, nxt, (I + 1) % R, 2 * (n - 1));
         if (2 * (n - 1) + 1 < NR) rd(p, nxt, (I + 1) % R, 2 * (n - 1) + 1);
-        if (n % 3 == 0) dma_single(k + R, cur, n / 3 - 1, inner_);
+        if (n % 3 == 0) {
+          dma_single(k + R, cur, n / 3 - 1, inner_, c, n);
+          with_copy = true;
+        }
       } else {
         if (n <= NR) rd(p, nxt, (I + 1) % R, n - 1);
         if constexpr (APAIR) {
           if constexpr (I & 1) {
             if (n >= 26 && n <= 59 && (n - 26) % 3 == 0) {
               const int c12 = (n - 26) / 3;
-              if (c12 < 8) dma_pair(k + 3, (I - 1) >> 1, c12, inner_);
-              else dma_single(k + R, cur, MB + c12 - 8, inner_);
+              if (c12 < 8) dma_pair(k + 3, (I - 1) >> 1, c12, inner_, c, n);
+              else dma_single(k + R, cur, MB + c12 - 8, inner_, c, n);
+              with_copy = true;
             }
           } else {
-            if (n >= 30 && n <= 54 && (n - 30) % 8 == 0) dma_single(k + R, cur, MB + (n - 30) / 8, inner_);
+            if (n >= 30 && n <= 54 && (n - 30) % 8 == 0) {
+              dma_single(k + R, cur, MB + (n - 30) / 8, inner_, c, n);
+              with_copy = true;
+            }
           }
         } else if constexpr (MB == 4) {
-          if (n >= 25 && n <= 60 && n % 5 == 0) dma_single(k + R, cur, n / 5 - 5, inner_);
+          if (n >= 25 && n <= 60 && n % 5 == 0) {
+            dma_single(k + R, cur, n / 5 - 5, inner_, c, n);
+            with_copy = true;
+          }
         } else {
-          if (n % 5 == 0 && n <= 30) dma_single(k + R, cur, n / 5 - 1, inner_);
+          if (n % 5 == 0 && n <= 30) {
+            dma_single(k + R, cur, n / 5 - 1, inner_, c, n);
+            with_copy = true;
+          }
         }
       }
-      mm(c, n);
+      if (!with_copy) mm(c, n);   // (a copy took MFMA n with it)
       FENCE();
     }
   };
@@ -591,20 +636,20 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   if constexpr (APAIR) {
     // in the order the steps of a turn issue them: pair (0,1), B 0, B 1, B 2, pair (2,3), B 3
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dma_pair(0, 0, i, std::false_type{});
+    for (int i = 0; i < 8; ++i) dma_pair(0, 0, i, std::false_type{}, f0, -1);
 #pragma unroll
     for (int s = 0; s < 3; ++s)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dma_single(s, ring.s[s], MB + i, std::false_type{});
+      for (int i = 0; i < 4; ++i) dma_single(s, ring.s[s], MB + i, std::false_type{}, f0, -1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dma_pair(2, 1, i, std::false_type{});
+    for (int i = 0; i < 8; ++i) dma_pair(2, 1, i, std::false_type{}, f0, -1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma_single(3, ring.s[3], MB + i, std::false_type{});
+    for (int i = 0; i < 4; ++i) dma_single(3, ring.s[3], MB + i, std::false_type{}, f0, -1);
   } else {
 #pragma unroll
     for (int s = 0; s < R; ++s)
 #pragma unroll
-      for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{});
+      for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{}, f0, -1);
   }
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
   if (RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
