@@ -46,6 +46,8 @@
 
 namespace pipeattn {
 
+union Frag { bf16x8 v; u16x8 u; fastattn::s16x4 h[2]; uint32_t w[4]; };   // one MFMA operand: 8 bf16 of a lane
+
 using fastattn::lds_s16x4;
 using fastattn::lds_void;
 using fastattn::s16x4;
@@ -72,7 +74,11 @@ __device__ __forceinline__ void set_prio(int p) {   // s_setprio takes an immedi
 
 // PREFETCHED: blocks 0, 1, 2 of this item are already in stages 0, 1, 2 (the item before it fetched them with its
 // trailing copies).  next_head: the head of the item that follows in this workgroup (this item's own head when none
-// does): this item's trailing copies fetch that head's first key blocks.
+// does): this item's trailing copies fetch that head's first key blocks.  next_qblk: that item's query block, -1 when
+// there is none.  Whole blocks: a wavefront's Q fragments (qf, the caller's) are dead once its last block's scores are
+// done, so it loads the next item's Q into them before it normalises and stores this item's results, and a chained
+// item starts with its Q on the way or there (the wavefronts that finish an item early have it long before): +1 % causal.
+// (Loading it a phase earlier, behind the last P.V MFMAs, spills in the masked period: 20 % slower.)
 //
 // RAGGED: N_CTX is a whole number of 32-query wavefront tiles but not of 256-query blocks.  A wavefront whose tile lies
 // past the end computes and stores nothing but keeps up with the barriers and its share of the copies; copies of rows
@@ -80,7 +86,8 @@ __device__ __forceinline__ void set_prio(int p) {   // s_setprio takes an immedi
 // diagonal block does that anyway); and the item's stream of blocks is padded to a multiple of four periods, so that
 // the next item's first blocks land in stages 0, 1, 2 as they do for whole blocks.
 template <int D, bool PREFETCHED, bool RAGGED = false>
-__device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int head, const int qblk, const int next_head) {
+__device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int head, const int qblk, const int next_head,
+                                     const int next_qblk, Frag (&qf)[D / 16]) {
   constexpr int BM = 256;
   constexpr int DK = D / 16, DT = D / 32, ROW = D * 2, CH = D / 8;
   constexpr int TILE = BN * ROW, STG = TILE, VBASE = NST * TILE;   // stage s: K at s*TILE, V at VBASE + s*TILE
@@ -179,8 +186,6 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   for (int t = 0; t < DT; ++t)
     v_off[t] = VBASE + (hi * 4 + qd) * ROW + (((t * 4 + v_cc) ^ ((D == 128 ? qd : ((qd >> 1) & 1)) << 2)) << 4) + ((i16 & 1) << 3);
 
-  union Frag { bf16x8 v; u16x8 u; s16x4 h[2]; uint32_t w[4]; };
-  Frag qf[DK];
   f32x16 acc[DT];
 #pragma unroll
   for (int t = 0; t < DT; ++t) acc[t] = (f32x16){0};
@@ -207,10 +212,12 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   // Q after the copies, so that the two round trips to memory overlap; the wait the compiler puts in front of the
   // first use of Q is for everything older as well, the copies included
   {
-    // (RAGGED: a wavefront past the end loads the last row that exists and never uses it)
-    const uint16_t *qrow = a.q + (base + (RAGGED ? min(my_q, a.n_ctx - 1) : my_q)) * a.ldq;
+    if constexpr (!PREFETCHED || RAGGED) {   // (otherwise the item before this one loaded them)
+      // (RAGGED: a wavefront past the end loads the last row that exists and never uses it)
+      const uint16_t *qrow = a.q + (base + (RAGGED ? min(my_q, a.n_ctx - 1) : my_q)) * a.ldq;
 #pragma unroll
-    for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+      for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+    }
     // the loads land here: the compiler's own vmcnt bookkeeping does not see the copies issued from assembly
 #pragma unroll
     for (int s = 0; s < DK; ++s) asm volatile("" : "+v"(qf[s].v));
@@ -411,6 +418,18 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
     cur_o = nx(cur_o);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the trailing copies land before the stages are reused or released
+  if constexpr (!RAGGED) {
+    if (next_qblk >= 0) {   // the next item's Q, on its way while this item's results are stored
+      const uint16_t *qrow = a.q + ((int64_t)next_head * a.n_ctx + next_qblk * BM + sub * 32 + c32) * a.ldq;
+#pragma unroll
+      for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+    } else {
+#pragma unroll
+      for (int s = 0; s < DK; ++s) qf[s].u = (u16x8){0, 0, 0, 0, 0, 0, 0, 0};   // (no next item.  Written all the same: left
+                                                                                 // alone, the old fragments count as live through
+                                                                                 // the last periods on this path, and those spill)
+    }
+  }
   if (!live) return;
   // ---- epilogue ----
   if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
@@ -461,12 +480,15 @@ __device__ __forceinline__ void attn_pipe(const AttnArgs &a, uint8_t *lds) {
   decode(n, head, p);
   int n2 = n, head2 = head, p2 = p, which2 = which;
   bool more = advance(n2, head2, p2, which2);
-  pipeattn::body<D, false, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+  pipeattn::Frag qf[D / 16];   // Q fragments of the running item; its last period refills them for the next
+  pipeattn::body<D, false, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head,
+                                   more ? (which2 ? p2 : qblocks - 1 - p2) : -1, qf);
   asm volatile("s_barrier" ::: "memory");   // nobody reads this item's stages any more; the next item's first blocks have landed
   while (more) {
     n = n2; head = head2; p = p2; which = which2;
     more = advance(n2, head2, p2, which2);
-    pipeattn::body<D, true, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head);
+    pipeattn::body<D, true, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head,
+                                    more ? (which2 ? p2 : qblocks - 1 - p2) : -1, qf);
     asm volatile("s_barrier" ::: "memory");
   }
 }
