@@ -323,7 +323,23 @@ TTAMD_API int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr
  *           BLOCK_M, BLOCK_N, FP8_OUTPUT, STAGE, warp_specialize, IS_HOPPER)
  * examples/fused-attn/06-fused-attention.py:143-215.  bf16 descriptors of shape
  * [Z*H*N_CTX, HEAD_DIM]; M receives m_i + log2(l_i); STAGE 3 = causal, 1 = full;
- * grid = (cdiv(N_CTX, BLOCK_M), Z*H, 1). */
+ * grid = (cdiv(N_CTX, BLOCK_M), Z*H, 1).
+ * Numerics are the source's (qk_scale = sm_scale * 1.44269504, exp2, l_ij summed
+ * in fp32 before P is rounded to bf16, fp32 accumulation), with two stated
+ * differences from a literal evaluation, both inside the tolerance the parity
+ * tests state (O within 2e-2, M within 1e-3 of the source's values):
+ *  - the exponent reference m_i of a row follows the running maximum lazily: a
+ *    new block maximum replaces it only when some row of its 32-query tile
+ *    exceeds it by more than 8 (log2 units).  Until then p = exp2(s - m_i) may
+ *    reach 2^8 instead of 1; l_i and the accumulator carry the same factor, so
+ *    O = acc / l_i and M = m_i + log2(l_i) are those of the true maximum up to
+ *    fp32 rounding;
+ *  - keys are taken in blocks of 64 whatever BLOCK_N says (fp32 summation order
+ *    only), and the causal mask is evaluated as the source does at BLOCK_M = 32:
+ *    -1.0e6 is added to masked scores inside the 32x32 tile on the diagonal and
+ *    keys past it are not visited.  At a larger BLOCK_M the source adds -1.0e6
+ *    to those as well; exp2 of that is exactly 0 unless a score exceeds 1e6, so
+ *    the results differ only for such scores. */
 TTAMD_API int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const tt_desc2d *desc_q,
                 const tt_desc2d *desc_k, const tt_desc2d *desc_v, const tt_desc2d *desc_o,
                 int32_t N_CTX, int32_t HEAD_DIM, int32_t BLOCK_M, int32_t BLOCK_N,

@@ -207,3 +207,126 @@ def test_the_launcher_stands_apart_from_the_gpu_runtime_and_the_oracle():
     subprocess.run([sys.executable, "-c", code], check=True, cwd=root)
     text = (root / "triton-tenstorrent_amd" / "cpu_abi.py").read_text()
     assert "import oracle" not in text and "from oracle" not in text and "libttamd_rt" not in text
+
+
+def test_a_kernel_without_the_block_loop_covers_its_grid_when_the_launcher_is_told(lib):
+    k = lib.get_kernel("single_block_kernel", ["*i32"])
+    out = torch.zeros(6, dtype=torch.int32)
+    k.launch((6, ), out, workers=2, persistent=False)          # called once per block with [b, b + 1)
+    assert out.tolist() == [1] * 6
+    # threads of a team still share memory and barriers from block to block
+    k = lib.get_kernel("team_kernel", ["*i32", "i32"])
+    threads, blocks, rounds = 3, 5, 20
+    out = torch.zeros(blocks * threads, dtype=torch.int32)
+    k.launch((blocks, ), out, rounds, shared=4 * threads, num_warps=threads, workers=2, persistent=False)
+    want = [sum((b + 1) * 1000 + r * 10 + t for r in range(rounds) for t in range(threads))
+            for b in range(blocks) for _ in range(threads)]
+    assert out.tolist() == want
+
+
+# --------------------------------------------------------------------------
+# the same kernels through the plugin surface: TTUtils.load_binary + TTLauncher
+# --------------------------------------------------------------------------
+DESC_KERNEL_C = r"""
+#include <stdint.h>
+/* a rank-2 descriptor arrives decomposed: base, shape x2 and strides x2 as i64, the padding flag, shape x2 as i32,
+   strides x2 as i64; then the launch scalars */
+void desc_kernel(const float *base, int64_t s0, int64_t s1, int64_t st0, int64_t st1, int8_t pad,
+                 int32_t t0, int32_t t1, int64_t tt0, int64_t tt1, float *out, int32_t n,
+                 int32_t *launch_sz, int32_t *launch_id, int8_t *smem, void *barrier) {
+  (void)launch_sz; (void)smem; (void)barrier;
+  if (launch_id[0] != 0) return;
+  out[0] = (float)s0; out[1] = (float)s1; out[2] = (float)st0; out[3] = (float)st1; out[4] = (float)pad;
+  out[5] = (float)t0; out[6] = (float)t1; out[7] = (float)tt0; out[8] = (float)tt1; out[9] = (float)n;
+  out[10] = base[st0 * (s0 - 1) + (s1 - 1)];          /* the last element, through the descriptor */
+}
+"""
+
+
+def _launcher_for(arg_names, signature, constants=None):
+    from types import SimpleNamespace
+    from triton_tenstorrent_amd.backend import driver as drv
+    src = SimpleNamespace(fn=SimpleNamespace(arg_names=list(arg_names)), signature=dict(zip(arg_names, signature)),
+                          constants=constants or {})
+    return drv.TTLauncher(src, SimpleNamespace())
+
+
+def test_an_elf_image_goes_through_load_binary_and_the_launcher(tmp_path):
+    """The reference hands a shared object to its runtime inside TTUtils.load_binary and launches it from
+    TTLauncher.__call__ (backend/driver.py:68-74, 98-170).  Here an ELF image given to load_binary comes back as a
+    host function, and the launcher runs it on host tensors with the cpu/ kernel ABI: no GPU, no GPU library."""
+    from triton_tenstorrent_amd.backend import driver as drv
+    src, so = tmp_path / "k.c", tmp_path / "libk.so"
+    src.write_text(KERNELS_C + DESC_KERNEL_C)
+    subprocess.run(["gcc", "-shared", "-fPIC", "-O2", "-std=c99", "-Wall", "-Werror", str(src), "-o", str(so)], check=True)
+    image = so.read_bytes()
+    utils = drv.TTDriver().utils
+    module, function, n_regs, shared, max_threads = utils.load_binary("add_kernel", image, 0, 0)
+    assert isinstance(function, cpu_abi.HostFunction) and function.host and (n_regs, shared, max_threads) == (1, 0, 4096)
+
+    n = 5000
+    torch.manual_seed(1)
+    x, y, out = torch.rand(n), torch.rand(n), torch.full((n + 4, ), -1.0)
+    launcher = _launcher_for(["x_ptr", "y_ptr", "output_ptr", "n_elements", "BLOCK_SIZE"],
+                             ["*fp32", "*fp32", "*fp32", "i32", "constexpr"])
+    seen = []
+    packed = (1, 1, 0, 1, 1, 1)              # num_warps, num_ctas, shared, cluster dims (backend/compiler.py:96-104)
+    launcher((n + 1023) // 1024, 1, 1, 0, function, packed, {"name": "add"}, lambda md: seen.append(("enter", md["name"])),
+             lambda md: seen.append(("exit", md["name"])), x, y, out, n, 1024)
+    assert torch.equal(out[:n], x + y) and torch.all(out[n:] == -1.0)
+    assert seen == [("enter", "add"), ("exit", "add")]
+
+    # threads, shared memory and the barrier come from the packed metadata
+    _, team, _, _, _ = utils.load_binary("team_kernel", image, 16, 0)
+    threads, blocks, rounds = 4, 3, 10
+    res = torch.zeros(blocks * threads, dtype=torch.int32)
+    _launcher_for(["out", "rounds"], ["*i32", "i32"])(blocks, 1, 1, 0, team, (threads, 1, 4 * threads, 1, 1, 1), None, None, None,
+                                                      res, rounds)
+    want = [sum((b + 1) * 1000 + r * 10 + t for r in range(rounds) for t in range(threads))
+            for b in range(blocks) for _ in range(threads)]
+    assert res.tolist() == want
+
+    # a descriptor is decomposed the way the reference's argument walk lists it
+    from triton_tenstorrent_amd.tensor_descriptor import TensorDescriptor
+    _, dk, _, _, _ = utils.load_binary("desc_kernel", image, 0, 0)
+    base = torch.arange(8 * 12, dtype=torch.float32).reshape(8, 12)
+    d = TensorDescriptor(base, [8, 12], [12, 1], [4, 4])
+    rec = torch.zeros(11)
+    _launcher_for(["d", "out", "n"], ["tensordesc<fp32[4,4]>", "*fp32", "i32"])(2, 1, 1, 0, dk, packed, None, None, None, d, rec, 77)
+    assert rec.tolist() == [8, 12, 12, 1, 0, 8, 12, 12, 1, 77, 95]
+
+    # device tensors are still refused, a missing kernel is an error at load_binary, and a JSON record is still the
+    # other kind of binary
+    class DeviceTensor:
+        is_cuda = True
+
+        def data_ptr(self):
+            raise AssertionError("must not be asked for an address")
+
+    with pytest.raises(ValueError, match="device memory"):
+        launcher(1, 1, 1, 0, function, packed, None, None, None, DeviceTensor(), y, out, 8, 1024)
+    with pytest.raises(LookupError):
+        utils.load_binary("no_such_kernel", image, 0, 0)
+    assert not cpu_abi.is_elf_image(b'{"kernel": "add_kernel"}')
+
+
+def test_the_elf_route_loads_neither_the_gpu_library_nor_the_oracle(tmp_path):
+    src, so = tmp_path / "k.c", tmp_path / "libk.so"
+    src.write_text(KERNELS_C)
+    subprocess.run(["gcc", "-shared", "-fPIC", "-O2", "-std=c99", str(src), "-o", str(so)], check=True)
+    code = ("import sys; sys.path.insert(0, '.'); import __graft_entry__ as g; g._package();"
+            "import torch;"
+            "from types import SimpleNamespace as NS;"
+            "from triton_tenstorrent_amd.backend import driver as drv;"
+            f"img = open({str(so)!r}, 'rb').read();"
+            "_, fn, _, _, _ = drv.TTDriver().utils.load_binary('add_kernel', img, 0, 0);"
+            "names = ['x', 'y', 'o', 'n', 'B'];"
+            "src = NS(fn=NS(arg_names=names), signature=dict(zip(names, ['*fp32', '*fp32', '*fp32', 'i32', 'constexpr'])), constants={});"
+            "x = torch.ones(2048); o = torch.zeros(2048);"
+            "drv.TTLauncher(src, NS())(2, 1, 1, 0, fn, (1, 1, 0, 1, 1, 1), None, None, None, x, x, o, 2048, 1024);"
+            "assert bool((o == 2).all());"
+            "maps = open('/proc/self/maps').read();"
+            "assert 'libttamd_rt' not in maps and 'liboracle' not in maps, 'a GPU or oracle library was mapped';"
+            "assert not [m for m in sys.modules if m.startswith('oracle')]")
+    from pathlib import Path
+    subprocess.run([sys.executable, "-c", code], check=True, cwd=Path(__file__).resolve().parents[1])

@@ -361,3 +361,165 @@ def test_elementwise_binders_refuse_a_launch_that_runs_past_an_operand(fake):
     K.add_kernel[(1, )](big, small, big, 4096, BLOCK_SIZE=512)
     K.add_kernel[(4, )](big, small, big, 1000, BLOCK_SIZE=1024)
     assert len(fake.calls) == before + 2
+
+
+# --------------------------------------------------------------------------
+# the cached repeat-launch path under threads (no GPU: stand-ins for the library and for tensors)
+# --------------------------------------------------------------------------
+import threading
+
+
+def _descriptors(ptr, shape=(256, 128), dtype=torch.bfloat16):
+    t = FakeTensor(shape, dtype, ptr)
+    return TensorDescriptor(t, list(shape), [shape[1], 1], [32, 32])
+
+
+def test_a_closure_parked_inside_the_c_call_keeps_its_own_descriptors(monkeypatch):
+    """ctypes releases the interpreter lock for the duration of a C call, so a second thread can run the same
+    closure while the first one's call is still reading its descriptor blocks.  The stand-in for the C entry point
+    parks thread A inside the call until thread B has launched with other operands, and then looks at the blocks it
+    was handed: they must still be A's."""
+    monkeypatch.setattr(drv, "_tensor_type", lambda: FakeTensor)
+    a_inside, b_done = threading.Event(), threading.Event()
+    seen = {}
+
+    def fn(da, db, dc, M, N, K_, bm, bn, bk, g, grid, stream):
+        who = threading.current_thread().name
+        if who == "A":
+            a_inside.set()
+            assert b_done.wait(10)
+        seen[who] = tuple(r._obj.base for r in (da, db, dc)) + (da._obj.shape[0], M)
+        return 0
+
+    bases = [FakeTensor((256, 128), torch.bfloat16)] * 3
+    direct = drv._desc_matmul_direct(fn, bases, 0, (128, 128, 64, 8))
+    ops = {"A": (0x1000, 0x2000, 0x3000, 256), "B": (0x5000, 0x6000, 0x7000, 512)}
+    ok = {}
+
+    def launch(who):
+        pa, pb, pc, M = ops[who]
+        ok[who] = direct((_descriptors(pa, (M, 128)), _descriptors(pb, (128, 128)), _descriptors(pc, (M, 128)), M, 128, 128),
+                         (4, ), 0)
+
+    ta = threading.Thread(target=launch, args=("A", ), name="A")
+    ta.start()
+    assert a_inside.wait(10)
+    tb = threading.Thread(target=launch, args=("B", ), name="B")
+    tb.start()
+    tb.join(10)
+    b_done.set()
+    ta.join(10)
+    assert ok == {"A": True, "B": True}
+    assert seen["A"] == (0x1000, 0x2000, 0x3000, 256, 256), seen
+    assert seen["B"] == (0x5000, 0x6000, 0x7000, 512, 512), seen
+
+
+def test_attention_closure_is_per_thread_too(monkeypatch):
+    monkeypatch.setattr(drv, "_tensor_type", lambda: FakeTensor)
+    a_inside, b_done = threading.Event(), threading.Event()
+    seen = {}
+
+    def fn(sm, m_ptr, Z, H, dq, dk, dv, do, n_ctx, hd, bm, bn, stage, grid, stream):
+        who = threading.current_thread().name
+        if who == "A":
+            a_inside.set()
+            assert b_done.wait(10)
+        seen[who] = tuple(r._obj.base for r in (dq, dk, dv, do)) + (m_ptr, )
+        return 0
+
+    direct = drv._attn_direct(fn, [FakeTensor((512, 64), torch.bfloat16)] * 4, (64, 128, 64, 3))
+    ok = {}
+
+    def launch(who, p0):
+        M = FakeTensor((2, 256), torch.float32, p0 + 0x900)
+        ds = [_descriptors(p0 + i * 0x100, (512, 64)) for i in range(4)]
+        ok[who] = direct((0.125, M, 1, 2, *ds, 256), (2, 2, 1), 0)
+
+    ta = threading.Thread(target=launch, args=("A", 0x10000), name="A")
+    ta.start()
+    assert a_inside.wait(10)
+    tb = threading.Thread(target=launch, args=("B", 0x20000), name="B")
+    tb.start()
+    tb.join(10)
+    b_done.set()
+    ta.join(10)
+    assert ok == {"A": True, "B": True}
+    assert seen["A"] == (0x10000, 0x10100, 0x10200, 0x10300, 0x10900), seen
+    assert seen["B"] == (0x20000, 0x20100, 0x20200, 0x20300, 0x20900), seen
+
+
+@pytest.fixture
+def fast(monkeypatch):
+    """The recording library with the cached repeat-launch path left ON: tensors are FakeTensors, the stream
+    lookup is the stock one (so plans are built and taken) and answers a fixed handle."""
+    lib = RecordingLib()
+    monkeypatch.setattr(rt, "init", lambda device=0: lib)
+    monkeypatch.setattr(drv, "_tensor_type", lambda: FakeTensor)
+    jit.active_driver()
+    monkeypatch.setattr(jit, "_raw_stream", lambda: (0, 0x1234))
+    for k in (K.add_kernel, K.matmul_kernel_tma, K._attn_fwd):
+        k._cache.clear()
+        k._plan = None
+    yield lib
+    for k in (K.add_kernel, K.matmul_kernel_tma, K._attn_fwd):
+        k._cache.clear()
+        k._plan = None
+
+
+def test_a_tensor_given_by_keyword_is_taken_from_the_call_not_from_the_plan(fast):
+    """Launch arguments may arrive by keyword.  A second call with ANOTHER output tensor under the same keyword
+    has to write there: the cached path compares only the values that select the kernel and reads the launch
+    arguments from the call in hand (comparing whole keyword dictionaries would compare tensors, and taking the
+    stored ones would write the previous call's buffer)."""
+    x, y = FakeTensor((4096, ), torch.float32, 0x1000), FakeTensor((4096, ), torch.float32, 0x2000)
+    out1, out2 = FakeTensor((4096, ), torch.float32, 0x3000), FakeTensor((4096, ), torch.float32, 0x4000)
+    K.add_kernel[(4, )](x, y, output_ptr=out1, n_elements=4096, BLOCK_SIZE=1024)
+    assert K.add_kernel._plan is not None
+    n0 = len(fast.calls)
+    K.add_kernel[(4, )](x, y, output_ptr=out2, n_elements=4096, BLOCK_SIZE=1024)
+    name, a = fast.calls[-1]
+    assert len(fast.calls) == n0 + 1 and name == "tt_add_kernel" and a[:4] == (0x1000, 0x2000, 0x4000, 4096)
+    assert K.add_kernel._keep[2] is out2                     # and that is the tensor kept alive
+    K.add_kernel[(2, )](x, y, output_ptr=out1, n_elements=2000, BLOCK_SIZE=1024)   # another n by keyword as well
+    assert fast.calls[-1][1][:4] == (0x1000, 0x2000, 0x3000, 2000)
+    K.add_kernel[(4, )](x, y, output_ptr=out2, n_elements=4096, BLOCK_SIZE=512)    # another constexpr: not the plan's kernel
+    assert fast.calls[-1][1][2:5] == (0x4000, 4096, 512)
+    K.add_kernel[(4, )](x, y, out1, n_elements=4096, BLOCK_SIZE=512)               # another split of the arguments
+    assert fast.calls[-1][1][2:5] == (0x3000, 4096, 512)
+
+
+def test_threads_with_different_constexprs_never_take_each_others_closure(fast):
+    """One launcher serves every thread that launches a specialisation, and the closure a binder leaves carries the
+    constexprs of ITS launch.  Two threads that launch the same kernel with different BLOCK sizes, again and again,
+    each have to see their own BLOCK in every C call."""
+    x = FakeTensor((1 << 16, ), torch.float32, 0x1000)
+    errors = []
+    start = threading.Barrier(2)
+
+    def worker(block, out_ptr):
+        out = FakeTensor((1 << 16, ), torch.float32, out_ptr)
+        start.wait()
+        for _ in range(300):
+            K.add_kernel[(8, )](x, x, out, 1 << 16, BLOCK_SIZE=block)
+
+    threads = [threading.Thread(target=worker, args=(256, 0xA000)), threading.Thread(target=worker, args=(1024, 0xB000))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(30)
+    for name, a in fast.calls:
+        if (a[2], a[4]) not in ((0xA000, 256), (0xB000, 1024)):
+            errors.append((name, a[2], a[4]))
+    assert len(fast.calls) == 600 and not errors, errors[:3]
+
+
+def test_launcher_keeps_operands_and_closure_per_thread(fake):
+    x = FakeTensor((4096, ), torch.float32)
+    K.add_kernel[(4, )](x, x, x, 4096, BLOCK_SIZE=1024)
+    launcher = next(iter(K.add_kernel._cache.values()))[0]
+    assert launcher.direct is not None and len(launcher.keepalive) == 3
+    other = {}
+    t = threading.Thread(target=lambda: other.update(direct=launcher.direct, keep=list(launcher.keepalive)))
+    t.start()
+    t.join(10)
+    assert other == {"direct": None, "keep": []}             # a thread that has not launched holds nothing

@@ -765,6 +765,31 @@ def test_a_table_name_does_not_vouch_for_the_body(tmp_path, monkeypatch):
         _compile(matmul_kernel, sig, {"stride_ak": 1, "stride_bn": 1, "stride_cn": 1, "BLOCK_SIZE_M": 32, "BLOCK_SIZE_N": 32,
                                       "BLOCK_SIZE_K": 32, "GROUP_SIZE_M": 1, "ACTIVATION": ""})
 
+    # upstream Triton's descriptor matmul (python/tutorials/09-persistent-matmul.py): same name and signature as
+    # the reference's, but B is [N, K] and the product is A.B^T; the reference removed that transpose
+    # (examples/matmul_tensor_descriptor/09-persistent-matmul.py:139), and with N == K the shapes would pass
+    @triton.jit
+    def matmul_kernel_tma(a_desc, b_desc, c_desc, M, N, K, BLOCK_SIZE_M: tl.constexpr, BLOCK_SIZE_N: tl.constexpr,
+                          BLOCK_SIZE_K: tl.constexpr, GROUP_SIZE_M: tl.constexpr, FP8_OUTPUT: tl.constexpr,
+                          WARP_SPECIALIZE: tl.constexpr):
+        pid = tl.program_id(axis=0)
+        num_pid_n = tl.cdiv(N, BLOCK_SIZE_N)
+        pid_m = pid // num_pid_n
+        pid_n = pid % num_pid_n
+        acc = tl.zeros((BLOCK_SIZE_M, BLOCK_SIZE_N), dtype=tl.float32)
+        for k in range(tl.cdiv(K, BLOCK_SIZE_K)):
+            a = a_desc.load([pid_m * BLOCK_SIZE_M, k * BLOCK_SIZE_K])
+            b = b_desc.load([pid_n * BLOCK_SIZE_N, k * BLOCK_SIZE_K])
+            acc = tl.dot(a, b.T, acc)
+        c_desc.store([pid_m * BLOCK_SIZE_M, pid_n * BLOCK_SIZE_N], acc.to(tl.bfloat16))
+
+    tma_sig = {"a_desc": "tensordesc<bf16[128,64]>", "b_desc": "tensordesc<bf16[128,64]>", "c_desc": "tensordesc<bf16[128,128]>",
+               "M": "i32", "N": "i32", "K": "i32", "BLOCK_SIZE_M": "constexpr", "BLOCK_SIZE_N": "constexpr",
+               "BLOCK_SIZE_K": "constexpr", "GROUP_SIZE_M": "constexpr", "FP8_OUTPUT": "constexpr", "WARP_SPECIALIZE": "constexpr"}
+    with pytest.raises(Exception, match="does not match"):
+        _compile(matmul_kernel_tma, tma_sig, {"BLOCK_SIZE_M": 128, "BLOCK_SIZE_N": 128, "BLOCK_SIZE_K": 64, "GROUP_SIZE_M": 8,
+                                              "FP8_OUTPUT": False, "WARP_SPECIALIZE": False})
+
     # a module named like the descriptor matmul whose body is something else
     from triton_tenstorrent_amd.backend.patterns import verify_named
     ttir_cos = _compile(one_op("cos_user", "tl.cos(v0)"), sig1, {"BLOCK_SIZE": 1024}).asm["ttir"]

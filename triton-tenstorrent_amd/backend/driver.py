@@ -11,6 +11,7 @@ from __future__ import annotations
 import ctypes as C
 import functools
 import json
+import threading
 import time
 from typing import Callable
 
@@ -177,14 +178,39 @@ def _check_extent(who: str, n: int, grid, per_program: int, *tensors):
                                                       f"{t.numel()}")
 
 
+def _tensor_type():
+    """The class a repeat-launch closure accepts as a tensor operand (exactly this class: a subclass may override
+    what the closure reads).  Looked up when a closure is built."""
+    import torch
+    return torch.Tensor
+
+
+def _desc_blocks_per_thread(dtype_codes: tuple):
+    """``get()`` -> (blocks, refs): one set of ``tt_desc2d`` blocks, and the ``byref`` handles to pass, PER CALLING
+    THREAD.  A closure refills its blocks on every call and ``ctypes`` releases the interpreter lock for the duration
+    of the C call, so blocks shared between threads would let one thread's launch read another's descriptors."""
+    tls = threading.local()
+
+    def get():
+        try:
+            return tls.state
+        except AttributeError:
+            blocks = [rt.tt_desc2d() for _ in dtype_codes]
+            for blk, code in zip(blocks, dtype_codes):
+                blk.dtype = code
+            tls.state = (blocks, tuple(C.byref(b) for b in blocks))
+            return tls.state
+
+    return get
+
+
 def _streaming_direct(fn, n_tensors: int, dtype, tail: tuple, per_program: int):
     """Repeat-launch closure for a kernel whose launch arguments are ``n_tensors`` tensors and ``n_elements``:
     ``direct(args, grid, stream)`` makes the same checks as the binder that built it (operand type, dtype, device,
     contiguity, extent) and the one C call, or returns False for anything it does not recognise, so that the
     caller takes the ordinary path (which also words the errors).  ``n_elements == 1`` is refused here because
     Triton folds that value into the specialisation: it belongs to another launcher."""
-    import torch
-    tensor_type, grid3, check = torch.Tensor, rt.Grid3, rt.check
+    tensor_type, grid3, check = _tensor_type(), rt.Grid3, rt.check
 
     def direct(args, grid, stream):
         n = args[n_tensors]
@@ -214,16 +240,12 @@ def _desc_matmul_direct(fn, bases: list, n_floats: int, tail: tuple):
     """Repeat-launch closure of the descriptor matmuls (see ``_streaming_direct``): the launch arguments are
     ``len(dtypes)`` rank-2 descriptors, then M, N, K, then ``n_floats`` floats.  The closure re-checks what selects
     the specialisation it was built under (descriptor class, rank, base dtype and device, integer M, N, K that Triton
-    would not fold) and fills its own ``tt_desc2d`` blocks, which the library reads during the call only; shapes,
-    strides, alignment and the grid are validated by the library as on the ordinary path."""
-    import torch
+    would not fold) and fills the calling thread's own ``tt_desc2d`` blocks, which the library reads during the call
+    only; shapes, strides, alignment and the grid are validated by the library as on the ordinary path."""
     from ..tensor_descriptor import TensorDescriptor
     dtypes = tuple(t.dtype for t in bases)      # of the descriptors' base tensors at the launch that built this
-    tensor_type, grid3, check, n_desc = torch.Tensor, rt.Grid3, rt.check, len(dtypes)
-    blocks = [rt.tt_desc2d() for _ in dtypes]
-    for blk, t in zip(blocks, bases):
-        blk.dtype = _torch_dtype_code(t)
-    refs = [C.byref(b) for b in blocks]
+    tensor_type, grid3, check, n_desc = _tensor_type(), rt.Grid3, rt.check, len(dtypes)
+    my_blocks = _desc_blocks_per_thread(tuple(_torch_dtype_code(t) for t in bases))
     n_args = n_desc + 3 + n_floats
 
     def direct(args, grid, stream):
@@ -233,6 +255,7 @@ def _desc_matmul_direct(fn, bases: list, n_floats: int, tail: tuple):
         if (type(M) is not int or type(N) is not int or type(K) is not int or not 1 < M < 2147483648
                 or not 1 < N < 2147483648 or not 1 < K < 2147483648):
             return False
+        blocks, refs = my_blocks()
         for blk, d, dt in zip(blocks, args, dtypes):
             if type(d) is not TensorDescriptor:
                 return False
@@ -263,11 +286,8 @@ def _attn_direct(fn, bases: list, tail: tuple):
     import torch
     from ..tensor_descriptor import TensorDescriptor
     dtypes = tuple(t.dtype for t in bases)
-    tensor_type, grid3, check, f32 = torch.Tensor, rt.Grid3, rt.check, torch.float32
-    blocks = [rt.tt_desc2d() for _ in bases]
-    for blk, t in zip(blocks, bases):
-        blk.dtype = _torch_dtype_code(t)
-    refs = [C.byref(b) for b in blocks]
+    tensor_type, grid3, check, f32 = _tensor_type(), rt.Grid3, rt.check, torch.float32
+    my_blocks = _desc_blocks_per_thread(tuple(_torch_dtype_code(t) for t in bases))
 
     def direct(args, grid, stream):
         if len(args) != 9 or not 1 <= len(grid) <= 3:
@@ -282,6 +302,7 @@ def _attn_direct(fn, bases: list, tail: tuple):
         for g in grid:
             if type(g) is not int:
                 return False
+        blocks, refs = my_blocks()
         for blk, d, dt in zip(blocks, args[4:8], dtypes):
             if type(d) is not TensorDescriptor:
                 return False
@@ -305,8 +326,7 @@ def _reduce_direct(fn, op_code: int, x_dtype, z_dtype, fixed: tuple):
     """Repeat-launch closure of ``reduce1d_kernel`` (see ``_streaming_direct``): the same checks as its binder for
     a call of the same shape, then the one C call.  ``fixed`` = (BLOCK, input, accumulate and output dtype codes,
     NaN flag), all set by the constexprs and dtypes that the closure re-checks."""
-    import torch
-    tensor_type, grid3, check, block = torch.Tensor, rt.Grid3, rt.check, fixed[0]
+    tensor_type, grid3, check, block = _tensor_type(), rt.Grid3, rt.check, fixed[0]
 
     def direct(args, grid, stream):
         x, z = args
@@ -654,6 +674,8 @@ KERNEL_TABLE: dict[str, Callable] = {
 class BoundKernel:
     """What ``load_binary`` hands back as ``function``: the kernel name and its binder."""
 
+    host = False        # (cpu_abi.HostFunction, the other kind of ``function``, says True)
+
     def __init__(self, name: str, record: dict):
         if name not in KERNEL_TABLE:
             raise rt.RuntimeError_(rt.RT_ERR_NOT_FOUND, f"no prebuilt kernel named {name!r}; have {sorted(KERNEL_TABLE)}")
@@ -676,6 +698,15 @@ class TTUtils:
         self.driver = driver
 
     def load_binary(self, name, kernel, shared_mem, device_id):
+        """``kernel`` is the JSON record of a prebuilt gfx950 kernel (what ``TTBackend`` emits), or an ELF shared
+        object that the CALLER built with the reference's cpu/ kernel ABI (what its ``make_library`` stage emits,
+        backend/compiler.py:452-466).  The second kind is loaded as the reference loads one
+        (``device.load_library(kernel, len(kernel))``, ``lib.get_kernel(name)``, backend/driver.py:68-74) and runs on
+        the host, on host tensors; it needs no GPU and is never chosen for a kernel of the first kind."""
+        from .. import cpu_abi
+        if cpu_abi.is_elf_image(kernel):
+            lib = cpu_abi.load_image(kernel)
+            return (lib, cpu_abi.HostFunction(lib, name), 1, shared_mem, 2**12)
         rt.init(int(device_id or 0))
         record = json.loads(kernel.decode() if isinstance(kernel, (bytes, bytearray)) else kernel) if kernel else {}
         fn = BoundKernel(record.get("kernel", name), record)
@@ -703,8 +734,10 @@ class TTLauncher:
         self.constants = {arg_idx(idx): value for idx, value in constants.items()}
         self.signature = {idx: value for idx, value in src.signature.items()}
         self.arg_names = arg_names
-        self.keepalive: list = []
-        self.direct = None      # the last launch's repeat-launch closure, when its binder offers one
+        # One launcher serves every thread that launches this specialisation, so what a launch leaves behind is kept
+        # per thread: its operands (launches are asynchronous) and the repeat-launch closure its binder offered,
+        # which carries the constexprs of THAT launch (two threads may launch with different BLOCK sizes).
+        self._tls = threading.local()
         # fixed per (kernel, specialisation): computed once, used on every launch
         self._sig_types = list(self.signature.values())
         self._constexpr_pos = [(i, n) for i, (n, ty) in enumerate(zip(arg_names, self._sig_types)) if ty == "constexpr"]
@@ -715,14 +748,35 @@ class TTLauncher:
         if not any(str(ty).startswith("tensordesc") for ty in self._sig_types):
             self._plain_pos = [i for i, ty in enumerate(self._sig_types) if ty != "constexpr"]
 
+    @property
+    def direct(self):
+        """The repeat-launch closure of this thread's last launch, when its binder offers one."""
+        return getattr(self._tls, "direct", None)
+
+    @property
+    def keepalive(self) -> list:
+        """The operands of this thread's last launch."""
+        return getattr(self._tls, "keepalive", [])
+
     def __call__(self, gridX, gridY, gridZ, stream, function, *args):
         kernel_metadata, launch_metadata, launch_enter_hook, launch_exit_hook = args[0], args[1], args[2], args[3]
-        del kernel_metadata  # num_warps / shared describe Triton codegen; the prebuilt kernels fix their own
         user_args = args[4:]
         sig_types = self._sig_types
         if len(user_args) != len(sig_types):
             raise rt.InvalidLaunch(rt.RT_ERR_INVALID,
                                    f"{function.name}: {len(user_args)} arguments for a {len(sig_types)}-entry signature")
+        if function.host:
+            # a caller-supplied shared object with the cpu/ kernel ABI: num_warps and the shared-memory size are
+            # the launch's own (packed metadata entries 0 and 2, backend/driver.py:103-106); host tensors only
+            from .. import cpu_abi
+            if launch_enter_hook is not None:
+                launch_enter_hook(launch_metadata)
+            cpu_abi.launch_host(function, sig_types, (gridX, gridY, gridZ), user_args, kernel_metadata[0],
+                                kernel_metadata[2], persistent=getattr(function, "persistent", True))
+            if launch_exit_hook is not None:
+                launch_exit_hook(launch_metadata)
+            return
+        # (num_warps / shared describe Triton codegen; the prebuilt gfx950 kernels fix their own)
         ranks: list = []
         if self._plain_pos is not None:
             flat = [user_args[i] for i in self._plain_pos]
@@ -741,9 +795,10 @@ class TTLauncher:
         rc = function.bind(lib, cur, consts, grid, stream or 0)
         if rc:
             rt.check(rc)
-        self.direct = cur.direct
-        # launches are asynchronous: keep operands referenced until the next launch replaces them
-        self.keepalive = keep
+        tls = self._tls
+        tls.direct = cur.direct
+        # launches are asynchronous: keep operands referenced until this thread's next launch replaces them
+        tls.keepalive = keep
         if launch_exit_hook is not None:
             launch_exit_hook(launch_metadata)
 

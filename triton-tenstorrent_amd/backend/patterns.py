@@ -497,16 +497,21 @@ def verify_named(name: str, ttir: str) -> dict | None:
     descs = len(re.findall(r"%[\w.]+\s*:\s*!tt\.tensordesc<", head))
     foreign = [k for k in c if k.startswith("math.")]
     if name in ("matmul_kernel_tma", "matmul_kernel_tma_fp8_scaled"):
+        # no tt.trans: upstream Triton's tutorial kernel of the same name and signature loads B as [N, K] and
+        # multiplies by its transpose; the reference took that transpose out (09-persistent-matmul.py:139) and the
+        # prebuilt kernel computes A.B
         ok = (n("tt.dot") == 1 and n("tt.descriptor_load") == 2 and n("tt.descriptor_store") == 1 and descs == 3
               and n("tt.load") == 0 and n("tt.store") == 0 and not foreign and n("arith.addf") == 0
-              and n("arith.mulf") <= (2 if name.endswith("fp8_scaled") else 0))
+              and n("tt.trans") == 0 and n("arith.mulf") <= (2 if name.endswith("fp8_scaled") else 0))
         if not ok:
-            raise bad("expected one tt.dot over two descriptor loads, one descriptor store and no epilogue")
+            raise bad("expected one tt.dot over two descriptor loads with B as [K, N] (no transpose), one descriptor "
+                      "store and no epilogue")
     elif name == "matmul_kernel_fused":
         ok = (n("tt.dot") == 1 and n("tt.descriptor_load") in (2, 3) and n("tt.descriptor_store") == 1 and descs == 4
-              and n("tt.load") == 0 and n("tt.store") == 0 and all(k in ("math.erf", "math.exp", "math.tanh") for k in foreign))
+              and n("tt.load") == 0 and n("tt.store") == 0 and n("tt.trans") == 0
+              and all(k in ("math.erf", "math.exp", "math.tanh") for k in foreign))
         if not ok:
-            raise bad("expected one tt.dot, a bias descriptor and one descriptor store")
+            raise bad("expected one tt.dot with B as [K, N] (no transpose), a bias descriptor and one descriptor store")
     elif name == "matmul_kernel":
         body = _body(ttir)
         # the reference's kernel reads tile-major buffers and never uses the strides of its signature

@@ -22,6 +22,11 @@ supplies: ``dlopen``, look the kernel up, marshal the arguments by the launcher'
 (backend/driver.py:141-159: constexprs skipped, tensors as pointers), give every worker one contiguous
 ``[block_start, block_end)`` and run one host thread per (worker, thread_id).
 
+The same launcher is reached through the plugin surface: ``TTUtils.load_binary`` given an ELF image (what the
+reference's ``make_library`` stage produces, backend/compiler.py:452-466) loads it with ``load_image`` and hands back
+a ``HostFunction``, and ``TTLauncher.__call__`` launches that on host tensors with ``launch_host`` (the launcher's
+own argument walk, descriptors decomposed as Triton decomposes them).
+
 It runs host code on host memory and nothing else: it is not a fallback for the gfx950 kernels (those fail loudly
 without their library or a GPU), it refuses device tensors, and it never loads anything but the file it is given
 and ``libttamd_cpuabi.so`` (the barrier).
@@ -129,11 +134,18 @@ class CPUKernel:
                 out.append(a)
         return out, keep
 
-    def launch(self, grid: Sequence[int], *args, shared: int = 0, num_warps: int = 1, workers: int | None = None):
+    def launch(self, grid: Sequence[int], *args, shared: int = 0, num_warps: int = 1, workers: int | None = None,
+               persistent: bool = True):
         """Run programs ``[0, gridX*gridY*gridZ)``: worker w gets ``block_range(blocks, workers, w)`` and runs it on
         ``num_warps`` host threads (``thread_id`` 0 .. num_warps-1; the cpu/ path has one thread per warp,
         backend/compiler.py:131-134) that share the worker's shared memory and barrier.  Returns when every
-        thread has; an exception in argument marshalling is raised before anything runs."""
+        thread has; an exception in argument marshalling is raised before anything runs.
+
+        ``persistent``: the kernel carries the loop over ``[block_start, block_end)`` that MakePersistentKernel
+        wraps around its body, so it is called once per (worker, thread) with the worker's whole range.  A kernel
+        built WITHOUT that pass runs the one block ``block_start`` per call (GPUOpToLLVM.cpp:121-129): say
+        ``persistent=False`` and it is called once per block, with ``[b, b + 1)``, the threads of a team meeting at
+        the team's barrier between blocks (they share the worker's shared memory)."""
         g = [int(x) for x in grid] + [1, 1, 1]
         gx, gy, gz = g[:3]
         if min(gx, gy, gz) < 0 or gx * gy * gz >= 2**31:
@@ -153,7 +165,15 @@ class CPUKernel:
 
         def run(ids, smem, barrier):
             try:
-                self._fn(*cargs, C.addressof(launch_sz), C.addressof(ids), smem, barrier)
+                if persistent:
+                    self._fn(*cargs, C.addressof(launch_sz), C.addressof(ids), smem, barrier)
+                    return
+                first, last = ids[0], ids[1]
+                for b in range(first, last):
+                    ids[0], ids[1] = b, b + 1
+                    self._fn(*cargs, C.addressof(launch_sz), C.addressof(ids), smem, barrier)
+                    if num_warps > 1 and b + 1 < last:
+                        sup._cpu_barrier(barrier)      # nobody starts block b+1 on shared memory that block b still reads
             except BaseException as e:      # ctypes.ArgumentError and the like: report, do not lose the thread
                 errors.append(e)
 
@@ -206,3 +226,82 @@ class CPULibrary:
 
 def load_library(path: str | os.PathLike) -> CPULibrary:
     return CPULibrary(path)
+
+
+def is_elf_image(kernel) -> bool:
+    """Is this ``load_binary`` payload a shared object (as opposed to the JSON record of a prebuilt gfx950 kernel)?"""
+    return isinstance(kernel, (bytes, bytearray, memoryview)) and bytes(kernel[:4]) == b"\x7fELF"
+
+
+def load_image(image: bytes) -> CPULibrary:
+    """A shared object handed over as bytes, the way the reference's launcher hands one to its runtime
+    (``device.load_library(kernel, len(kernel))``, backend/driver.py:72).  The image goes into an anonymous
+    in-memory file that ``dlopen`` maps; nothing is left on disk."""
+    if not is_elf_image(image):
+        raise ValueError("not an ELF image")
+    fd = os.memfd_create("ttamd_cpu_kernel", 0)
+    try:
+        with os.fdopen(os.dup(fd), "wb") as f:
+            f.write(bytes(image))
+        return CPULibrary(f"/proc/self/fd/{fd}")
+    finally:
+        os.close(fd)        # the mapping made by dlopen keeps the pages
+
+
+def expand_signature(sig_types: Sequence[str]) -> list[str]:
+    """Launch signature -> the types that cross the C ABI, one per value of the launcher's argument walk
+    (backend/driver.py:141-159): a rank-r ``tensordesc<dtype[...]>`` becomes ``*dtype``, r shapes and r strides as
+    i64, the padding flag as i1, then r shapes as i32 and r strides as i64, which is how Triton decomposes a
+    descriptor that has no hardware form (triton/backends/amd/driver.py:229-256)."""
+    out: list[str] = []
+    for ty in sig_types:
+        if isinstance(ty, str) and ty.startswith("tensordesc<"):
+            dtype = ty[len("tensordesc<"):].split("[")[0]
+            r = ty.count(",") + 1
+            out += ["*" + dtype] + ["i64"] * (2 * r) + ["i1"] + ["i32"] * r + ["i64"] * r
+        else:
+            out.append(ty)
+    return out
+
+
+class HostFunction:
+    """What ``TTUtils.load_binary`` returns as ``function`` for an ELF image: the kernel's name in a loaded
+    library.  The launch signature is the launcher's, so the typed kernel is made (and kept) at the first launch."""
+
+    host = True
+
+    def __init__(self, library: CPULibrary, name: str):
+        self.library, self.name = library, name
+        self._typed: dict = {}
+        if not hasattr(library.handle, name):
+            raise LookupError(f"{library.path}: no kernel '{name}'")
+
+    def typed(self, flat_types: Sequence[str]) -> CPUKernel:
+        key = tuple(flat_types)
+        k = self._typed.get(key)
+        if k is None:
+            k = self._typed[key] = CPUKernel(self.library, self.name, key)
+        return k
+
+    def __repr__(self):
+        return f"<HostFunction {self.name}>"
+
+
+def launch_host(function: HostFunction, sig_types: Sequence[str], grid: Sequence[int], user_args: Sequence[Any],
+                num_warps: int, shared: int, persistent: bool = True) -> None:
+    """``TTLauncher.__call__`` for a host kernel: the reference's argument walk (constexprs skipped, a tensor as
+    its address, a descriptor as base, shape, strides, padding flag, shape, strides), then ``CPUKernel.launch``."""
+    from .tensor_descriptor import is_tensor_descriptor
+    flat_types = [t for t in expand_signature(sig_types) if t != "constexpr"]
+    flat: list = []
+    for ty, a in zip(sig_types, user_args):
+        if ty == "constexpr":
+            continue
+        if is_tensor_descriptor(a):
+            shape, strides = [int(d) for d in a.shape], [int(x) for x in a.strides]
+            flat += [a.base, *shape, *strides, a.padding == "nan", *shape, *strides]
+        else:
+            flat.append(a)
+    if len(flat) != len(flat_types):
+        raise ValueError(f"{function.name}: the arguments flatten to {len(flat)} values, the signature to {len(flat_types)}")
+    function.typed(flat_types).launch(grid, *flat, shared=int(shared), num_warps=max(1, int(num_warps)), persistent=persistent)

@@ -833,7 +833,7 @@ extern "C" {
 GEMM_TILE_ALL_EPI(gemm_tile_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
 
-// the same kernels for M any, N % 8 == 0, K % 32 == 0
+// the same kernels for M any, N % 8 == 0, K % 8 == 0 (a last 32-deep step that ends past K is cleared in LDS)
 #define GEMM_TILE_RAGGED(name, IN, OUT, EPI)                                                       \
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \

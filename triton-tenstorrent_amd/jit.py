@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import functools
 import json
+import threading
 from types import SimpleNamespace
 from typing import Any, Callable, Sequence
 
@@ -76,6 +77,9 @@ class Config:
         self.kwargs, self.num_warps, self.num_stages, self.pre_hook = dict(kwargs), num_warps, num_stages, pre_hook
 
 
+_MISSING = object()
+_PLAIN_VALUES = (int, float, str, bool, type(None))      # constexpr values a plan compares with ==
+
 _driver: TTDriver | None = None
 _STOCK_GET_STREAM = TTDriver.get_current_stream      # a driver whose stream lookup was replaced is asked, not bypassed
 _raw_stream = None      # (current device, its current stream) without building torch.cuda.Stream objects
@@ -117,11 +121,15 @@ class PrebuiltKernel:
         self.defaults = dict(defaults or {})
         self.fn = SimpleNamespace(arg_names=self.arg_names, __name__=name)
         self._cache: dict = {}
-        # repeat launches: (number of positional arguments, keyword arguments, device, closure, the configuration's
-        # pre_hook or None, the arguments after the positional ones by name for that hook and for a callable grid,
-        # the launch arguments among them in order or None)
+        # repeat launches: (number of positional arguments, the keyword arguments that are not launch arguments
+        # (constexprs, num_warps ...) with their values, device, closure, the configuration's pre_hook or None, the
+        # arguments after the positional ones by name for that hook and for a callable grid, the launch arguments
+        # among them in order as (name, given by keyword?, value at the launch that built the plan) or None, the
+        # number of keyword arguments).  The tuple is replaced as a whole and never modified, and everything a launch
+        # writes (the closure's descriptor blocks, the operands kept alive) is per thread: any thread may take a plan
+        # that another one built.
         self._plan = None
-        self._keep = None
+        self._tls = threading.local()
         n_lead = next((i for i, n in enumerate(self.arg_names) if n in self.constexprs), len(self.arg_names))
         # a plan needs "launch arguments first, positionally; constexprs after them, by keyword or default"
         self._lead = n_lead if all(n in self.constexprs for n in self.arg_names[n_lead:]) else None
@@ -150,26 +158,52 @@ class PrebuiltKernel:
             raise TypeError(f"{self.name}() missing arguments: {missing}")
         return {n: bound[n] for n in self.arg_names}
 
+    @property
+    def _keep(self):
+        """The operands of the calling thread's last repeat launch."""
+        return getattr(self._tls, "keep", None)
+
+    def _plan_applies(self, plan, kwargs):
+        """-> (True, launch arguments given by keyword in their positions) when this call's keyword arguments are
+        the plan's: the same names, the same VALUES for those that select the kernel (constexprs, compared only
+        where they are plain Python values), and whatever the caller passes now for the launch arguments among
+        them (a tensor given by keyword is a different tensor every call)."""
+        for k, v in plan[1].items():
+            w = kwargs.get(k, _MISSING)
+            if w is not v and (type(w) is not type(v) or type(v) not in _PLAIN_VALUES or w != v):
+                return False, None
+        tail = plan[6]
+        if tail is None:
+            return True, None
+        try:
+            return True, tuple([kwargs[n] if from_kw else v for n, from_kw, v in tail])
+        except KeyError:
+            return False, None
+
     def run(self, *args, grid, **kwargs):
         plan = self._plan
-        if (plan is not None and TTDriver.get_current_stream is _STOCK_GET_STREAM and len(args) == plan[0] and kwargs == plan[1] and (type(grid) is tuple or callable(grid))
+        if (plan is not None and TTDriver.get_current_stream is _STOCK_GET_STREAM and len(args) == plan[0]
+                and len(kwargs) == plan[7] and (type(grid) is tuple or callable(grid))
                 and PrebuiltKernel.launch_enter_hook is None and PrebuiltKernel.launch_exit_hook is None):
             device, stream = _raw_stream()
-            if device == plan[2]:
+            ok, by_keyword = self._plan_applies(plan, kwargs) if device == plan[2] else (False, None)
+            if ok:
                 g = grid
                 if plan[4] is not None or type(g) is not tuple:
                     # the configuration's pre_hook and a callable grid see every argument by name, as on the ordinary path
                     named = dict(zip(self.arg_names, args))
                     named.update(plan[5])
+                    if by_keyword is not None:
+                        for (n, _, _), v in zip(plan[6], by_keyword):
+                            named[n] = v
                     if plan[4] is not None:
                         plan[4](named)
                     if type(g) is not tuple:
                         g = g(named)
-                # launch arguments that came by keyword (equal to the ones the plan was built with: see the guard) go
-                # to the closure in their positions
-                full = args if plan[6] is None else args + plan[6]
+                # launch arguments that came by keyword go to the closure in their positions
+                full = args if by_keyword is None else args + by_keyword
                 if type(g) is tuple and plan[3](full, g, stream):
-                    self._keep = args   # launches are asynchronous: operands stay referenced until the next one
+                    self._tls.keep = full   # launches are asynchronous: operands stay referenced until this thread's next one
                     return self
         user_grid = grid
         bound = self._bind(args, kwargs)
@@ -213,6 +247,7 @@ class PrebuiltKernel:
                 and (type(user_grid) is tuple or callable(user_grid)) and stream == _raw_stream()[1]):
             hook = config.pre_hook if config is not None else None
             rest = {n: bound[n] for n in self.arg_names[len(args):]}
-            by_keyword = tuple(bound[n] for n in self.arg_names[len(args):self._lead]) or None
-            self._plan = (len(args), dict(kwargs), device, direct, hook, rest, by_keyword)
+            tail = tuple((n, n in kwargs, bound[n]) for n in self.arg_names[len(args):self._lead]) or None
+            selecting = {k: v for k, v in kwargs.items() if k not in self.arg_names[len(args):self._lead]}
+            self._plan = (len(args), selecting, device, direct, hook, rest, tail, len(kwargs))
         return self
