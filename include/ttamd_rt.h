@@ -345,6 +345,13 @@ TTAMD_API int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const 
                 int32_t N_CTX, int32_t HEAD_DIM, int32_t BLOCK_M, int32_t BLOCK_N,
                 int32_t STAGE, const uint32_t grid[3], void *stream);
 
+/* Diagnostic, no counterpart in the reference: what core clock does the part grant under the 16-bit macro-tile GEMM?
+ * arm != 0 makes the NEXT launch of that kernel (tt_matmul_kernel_tma / _fused on a shape of whole 256x256x128 macro
+ * tiles) synchronous and records workgroup 0's core-clock cycles and the 100 MHz wall ticks of its run; reading
+ * (may be null) receives the last record, {0, 0} when there is none: clock in GHz = reading[0] / reading[1] / 10.
+ * The kernels are bounded by power, so their rate follows this clock, which differs from box to box. */
+TTAMD_API int rt_gemm_clock_probe(int32_t arm, uint64_t reading[2]);
+
 /* Name of the device kernel the last tt_* call on this thread launched (for
  * profiles and tests that assert which path ran). */
 TTAMD_API const char *tt_last_kernel_name(void);

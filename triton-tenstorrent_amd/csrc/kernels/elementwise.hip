@@ -20,6 +20,7 @@
 // and 6750 at one vector per lane, a read-only one 7100-7170 at either.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "elementwise_geom.h"
 
@@ -27,7 +28,6 @@ namespace {
 
 using ewgeom::kThreads;
 using ewgeom::kVec;
-using ewgeom::kVecHeavy;
 
 template <typename T> struct Vec4 { typedef T type __attribute__((ext_vector_type(4))); };
 
@@ -137,41 +137,43 @@ __device__ __forceinline__ void binary_scalar_body(const T *x, const T *y, T *ou
 }
 
 // ---- sin ------------------------------------------------------------------
-// k = rint(x * 2/pi); r = x - k*pi/2 by a three-constant Cody-Waite reduction
-// carried out with fused multiply-adds (each k*piece product enters the fma
-// unrounded); minimax polynomials for sin and
-// cos on [-pi/4, pi/4]; quadrant select.  Valid while k*pi/2's third piece
-// still resolves the result: |x| < 2^17 here, beyond that the library routine
-// with its full Payne-Hanek reduction takes over (a wave-uniform rarity).
+// k = rint(x / pi); r = x - k*pi by a two-constant Cody-Waite reduction carried out with fused multiply-adds (x - k*p1
+// is exact: both are multiples of 2^-22 and the difference is below 2; the piece of pi left out after p2 is 3e-15, i.e.
+// k times that in r: 1.3e-10 at the top of the range); one odd minimax polynomial of degree 9 on [-pi/2, pi/2]
+// (|error| <= 5e-9); sin(x) = (-1)^k sin(r).  13 VALU operations per element, where the reduction to a quarter
+// period with a sine and a cosine polynomial and a select between them took 24: at two 16-byte vectors per lane
+// that arithmetic showed beside the memory time.  Max |error| 1.3e-7 against the correctly rounded result over
+// |x| < 2^17 (the bar of the parity tests is 2e-6); near a multiple of pi the error is absolute, not relative.
+// Beyond 2^17 the library routine with its full Payne-Hanek reduction takes over (a wave-uniform rarity).
 __device__ __forceinline__ float sin_fast(float x) {
-  const float two_over_pi = 0.636619772367581343f;
-  const float p1 = 1.5707963705062866f;     // fp32(pi/2)
-  const float p2 = -4.371138828673793e-08f;  // fp32(pi/2 - p1)
-  const float p3 = -1.7151245100058819e-15f; // fp32(pi/2 - p1 - p2)
-  float kf = __builtin_rintf(x * two_over_pi);
+  const float one_over_pi = 0.318309886183790672f;
+  const float p1 = 3.1415927410125732f;       // fp32(pi)
+  const float p2 = -8.742277657347586e-08f;   // fp32(pi - p1)
+  const float kf = __builtin_rintf(x * one_over_pi);
   float r = __builtin_fmaf(-kf, p1, x);
   r = __builtin_fmaf(-kf, p2, r);
-  r = __builtin_fmaf(-kf, p3, r);
-  int q = (int)kf;
-  float r2 = r * r;
-  // sin(r) = r + r^3 * S(r^2)
-  float s = __builtin_fmaf(r2, 2.7183114939898219064e-06f, -1.98393348360966317347e-04f);
-  s = __builtin_fmaf(s, r2, 8.3333293858894631756e-03f);
-  s = __builtin_fmaf(s, r2, -1.66666666416265235595e-01f);
-  s = __builtin_fmaf(s * r2, r, r);
-  // cos(r) = 1 + r^2 * C(r^2)
-  float c = __builtin_fmaf(r2, 2.43904487962774090654e-05f, -1.38867637746099294692e-03f);
-  c = __builtin_fmaf(c, r2, 4.16666233237390631894e-02f);
-  c = __builtin_fmaf(c, r2, -4.99999997251031003120e-01f);
-  c = __builtin_fmaf(c, r2, 1.0f);
-  float v = (q & 1) ? c : s;
-  return (q & 2) ? -v : v;
+  const uint32_t odd = (uint32_t)(int)kf << 31;
+  const float r2 = r * r;
+  // sin(r) = r + r^3 * P(r^2)
+  float p = __builtin_fmaf(r2, 2.599668732727878e-06f, -1.980644155992195e-04f);
+  p = __builtin_fmaf(p, r2, 8.333015255630016e-03f);
+  p = __builtin_fmaf(p, r2, -1.6666656732559204e-01f);
+  const float s = __builtin_fmaf(p * r2, r, r);
+  return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, s) ^ odd);
 }
 
 __device__ __forceinline__ float sin_any(float x) {
   const float ax = __builtin_fabsf(x);
+  float v = sin_fast(x);
+  // |x| >= 2^17 (inf and NaN included): the library routine.  The branch is on a whole wavefront's vote, so that it IS
+  // a branch: written as a select between the two results, the compiler evaluates the library routine's
+  // 300-instruction reduction for every element and picks afterwards (the kernel then needed two vectors per lane
+  // to hide its own arithmetic and still ran 3 % behind exp).
+  if (__builtin_amdgcn_ballot_w64(!(ax < 131072.0f)) != 0) {
+    asm volatile("" ::: "memory");   // (nothing in here may be hoisted out and evaluated for everybody)
+    if (!(ax < 131072.0f)) v = sinf(x);
+  }
   // below 2^-12 sin(x) rounds to x itself; returning x also keeps the sign of -0.0
-  float v = (ax < 131072.0f) ? sin_fast(x) : sinf(x);
   return ax < 2.44140625e-4f ? x : v;
 }
 
@@ -197,23 +199,23 @@ __device__ __forceinline__ float cos_fast(float x) {
   return (q & 2) ? -v : v;
 }
 
-// IEEE-754-2019 maximum / minimum (arith.maximumf / minimumf): NaN if either is NaN, -0 < +0
-__device__ __forceinline__ float ieee_maximum(float a, float b) {
-  if (a != a) return a;
-  if (b != b) return b;
-  if (a == b) return __builtin_signbit(a) ? b : a;
-  return a > b ? a : b;
-}
-__device__ __forceinline__ float ieee_minimum(float a, float b) {
-  if (a != a) return a;
-  if (b != b) return b;
-  if (a == b) return __builtin_signbit(a) ? a : b;
-  return a < b ? a : b;
-}
+// IEEE-754-2019 maximum / minimum (arith.maximumf / minimumf): NaN if either is NaN, -0 < +0.  gfx950 has the
+// operation as one instruction (v_maximum3_f32 / v_minimum3_f32, which the builtin selects); spelled out with
+// comparisons it was six VALU operations per element and wanted two vectors per lane.
+__device__ __forceinline__ float ieee_maximum(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float ieee_minimum(float a, float b) { return __builtin_elementwise_minimum(a, b); }
 
 struct SinOp { __device__ static float apply(float x) { return sin_any(x); } };
 struct CosOp {
-  __device__ static float apply(float x) { return __builtin_fabsf(x) < 131072.0f ? cos_fast(x) : cosf(x); }
+  __device__ static float apply(float x) {
+    const float ax = __builtin_fabsf(x);
+    float v = cos_fast(x);
+    if (__builtin_amdgcn_ballot_w64(!(ax < 131072.0f)) != 0) {   // a real branch on the wavefront's vote, as in sin_any
+      asm volatile("" ::: "memory");
+      if (!(ax < 131072.0f)) v = cosf(x);
+    }
+    return v;
+  }
 };
 struct AbsOp { __device__ static float apply(float x) { return __builtin_fabsf(x); } };
 struct CeilOp { __device__ static float apply(float x) { return __builtin_ceilf(x); } };
@@ -330,40 +332,40 @@ __device__ __forceinline__ void cast_body(const typename Op::in_t *x, typename O
   for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) out[i] = Op::apply(x[i]);
 }
 
-// 16-byte aligned operands: a lane turns 16 / sizeof(out) inputs (2 or 4 loads of 16 bytes) into one 16-byte
-// store; a workgroup owns one contiguous run of kThreads * UNROLL such items, the last one also the ragged end.
+// 16-byte aligned operands: a lane turns the four inputs of one 16-byte load into one 8- or 4-byte store, so that a
+// wavefront reads 1 KiB and writes 512 or 256 bytes, each in one contiguous run (whole cache lines for every load and
+// store instruction).  A workgroup owns one contiguous run of kThreads * UNROLL such items, the last one also the
+// ragged end.  (Gathering 16 bytes of output per lane instead made every load instruction touch every other 16 bytes of
+// twice the lines: fp32 -> bf16 at N = 2^28 ran at 6.0 TB/s that way.)
 template <typename Op, int UNROLL>
 __device__ __forceinline__ void cast_vec_body(const typename Op::in_t *__restrict__ x, typename Op::out_t *__restrict__ out,
                                               uint32_t n) {
   using In = typename Op::in_t;
   using Out = typename Op::out_t;
-  constexpr int E = 16 / (int)sizeof(Out);   // elements per item: 8 or 16
-  constexpr int LOADS = E / 4;
+  static_assert(sizeof(In) == 4 && (sizeof(Out) == 2 || sizeof(Out) == 1), "four inputs of four bytes per item");
   typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+  using Packed = typename std::conditional<sizeof(Out) == 2, u32x2_t, uint32_t>::type;
   union InV { u32x4_t q; In e[4]; };
-  union OutV { u32x4_t q; Out e[E]; };
-  const uint32_t nitem = n / E;
+  union OutV { Packed q; Out e[4]; };
+  const uint32_t nitem = n / 4;
   const u32x4_t *xv = reinterpret_cast<const u32x4_t *>(x);
-  u32x4_t *ov = reinterpret_cast<u32x4_t *>(out);
+  Packed *ov = reinterpret_cast<Packed *>(out);
   const uint32_t base = blockIdx.x * (kThreads * UNROLL);
   const uint32_t i = base + threadIdx.x;
   if (base + kThreads * UNROLL <= nitem) {
-    InV a[UNROLL][LOADS];
+    InV a[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-      for (int l = 0; l < LOADS; ++l) a[u][l].q = __builtin_nontemporal_load(xv + (size_t)(i + u * kThreads) * LOADS + l);
+    for (int u = 0; u < UNROLL; ++u) a[u].q = __builtin_nontemporal_load(xv + i + u * kThreads);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       OutV r;
 #pragma unroll
-      for (int l = 0; l < LOADS; ++l)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) r.e[l * 4 + e] = Op::apply(a[u][l].e[e]);
+      for (int e = 0; e < 4; ++e) r.e[e] = Op::apply(a[u].e[e]);
       __builtin_nontemporal_store(r.q, ov + i + u * kThreads);
     }
   } else {
-    for (uint32_t j = (size_t)base * E + threadIdx.x; j < n; j += kThreads) out[j] = Op::apply(x[j]);
+    for (uint32_t j = (size_t)base * 4 + threadIdx.x; j < n; j += kThreads) out[j] = Op::apply(x[j]);
   }
 }
 
@@ -402,8 +404,8 @@ __global__ __launch_bounds__(kThreads) void ew_add_i32_unaligned(const int *x, c
                                                                         uint32_t n) {                    \
     unary_scalar_body<Op>(x, out, n);                                                                    \
   }
-EW_UNARY(sin, SinOp, kVecHeavy)
-EW_UNARY(cos, CosOp, kVecHeavy)
+EW_UNARY(sin, SinOp, ewgeom::kVecTrig)
+EW_UNARY(cos, CosOp, ewgeom::kVecTrig)
 EW_UNARY(abs, AbsOp, kVec)
 EW_UNARY(ceil, CeilOp, kVec)
 EW_UNARY(floor, FloorOp, kVec)
@@ -443,10 +445,8 @@ EW_BINARY_CONST(min, MinOp)
 EW_BINARY(sub, SubOp, kVec)
 EW_BINARY(mul, MulOp, kVec)
 EW_BINARY(div, DivOp, kVec)
-// maximum / minimum carry a NaN and signed-zero rule (about six VALU operations per element): two vectors per lane,
-// as for sin and cos
-EW_BINARY(max, MaxOp, kVecHeavy)
-EW_BINARY(min, MinOp, kVecHeavy)
+EW_BINARY(max, MaxOp, kVec)
+EW_BINARY(min, MinOp, kVec)
 
 #define EW_CAST(name, Op, IN, OUT)                                                                          \
   __global__ __launch_bounds__(kThreads) void name(const IN *x, OUT *out, uint32_t n) {                     \

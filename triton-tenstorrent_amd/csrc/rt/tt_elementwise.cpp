@@ -122,7 +122,7 @@ int tt_sin_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_SI
   bool al = aligned16(x) && aligned16(out);
   void *args[] = {&x, &out, &n_eff};
   return launch("elementwise", al ? "ew_sin_f32" : "ew_sin_f32_unaligned",
-                dim3(streaming_grid(n_eff, al, ewgeom::kVecHeavy)), dim3(kThreads), 0, stream, args, 3);
+                dim3(streaming_grid(n_eff, al, ewgeom::kVecTrig)), dim3(kThreads), 0, stream, args, 3);
 }
 
 int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_elements, int32_t BLOCK_SIZE,
@@ -140,9 +140,8 @@ int tt_unary_kernel(int32_t op, const void *x, void *out, int32_t n_elements, in
   char name[48];
   snprintf(name, sizeof(name), "ew_%s_f32%s", names[op], al ? "" : "_unaligned");
   void *args[] = {&x, &out, &n_eff};
-  const bool heavy = op == TT_OP_SIN || op == TT_OP_COS;
-  return launch("elementwise", name, dim3(streaming_grid(n_eff, al, heavy ? ewgeom::kVecHeavy : kUnroll)), dim3(kThreads), 0,
-                stream, args, 3);
+  const int vec = (op == TT_OP_SIN || op == TT_OP_COS) ? ewgeom::kVecTrig : kUnroll;
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al, vec)), dim3(kThreads), 0, stream, args, 3);
 }
 
 int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_t n_elements,
@@ -160,8 +159,7 @@ int tt_binary_kernel(int32_t op, const void *x, const void *y, void *out, int32_
   char name[48];
   snprintf(name, sizeof(name), "ew_%s_f32%s", names[op], al ? "" : "_unaligned");
   void *args[] = {&x, &y, &out, &n_eff};
-  const bool heavy = op == TT_OP_MAXIMUM || op == TT_OP_MINIMUM;   // built with kVecHeavy vectors per lane
-  return launch("elementwise", name, dim3(streaming_grid(n_eff, al, heavy ? ewgeom::kVecHeavy : kUnroll)), dim3(kThreads), 0,
+  return launch("elementwise", name, dim3(streaming_grid(n_eff, al, kUnroll)), dim3(kThreads), 0,
                 stream, args, 4);
 }
 
@@ -204,7 +202,7 @@ int tt_cast_kernel(const void *x, void *out, int32_t n_elements, int32_t BLOCK_S
   void *args[] = {&x, &out, &n_eff};
   if (aligned16(x) && aligned16(out)) {
     // one workgroup per run of kThreads * kUnroll 16-byte stores, plus the ragged end
-    const uint32_t per_item = out_dtype == TT_I8 ? 16 : 8, per_wg = kThreads * kUnroll * per_item;
+    const uint32_t per_wg = kThreads * kUnroll * 4;   // four inputs per lane and vector
     return launch("elementwise", stem, dim3((uint32_t)cdiv64(n_eff, per_wg)), dim3(kThreads), 0, stream, args, 3);
   }
   char name[48];

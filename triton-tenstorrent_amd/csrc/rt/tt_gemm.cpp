@@ -1,6 +1,7 @@
 // tt_matmul_kernel_tma / tt_matmul_kernel_fused / tt_matmul_kernel_tma_fp8_scaled / tt_matmul_kernel:
 // launch validation and kernel selection for the tile-matmul family.
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 
@@ -10,6 +11,10 @@
 using namespace ttamd;
 
 namespace {
+
+// rt_gemm_clock_probe: armed for one launch; the last reading {core-clock cycles, 100 MHz ticks} of workgroup 0
+std::atomic<int> g_probe_armed{0};
+std::atomic<unsigned long long> g_probe_last[2];
 
 // Workgroups of the persistent macro-tile kernels: one per CU, or one per tile when there are fewer tiles.
 // The plain kernels (`splits`) finish a tail of at most grid/2 macro tiles as half tiles on twice the
@@ -137,7 +142,8 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
     // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
     static unsigned long long *probe_buf = nullptr;
-    const bool probe = env_int("TTAMD_GEMM_CLOCK_PROBE", 0) != 0;
+    const bool armed = g_probe_armed.exchange(0) != 0;     // rt_gemm_clock_probe(1, ...): this launch only
+    const bool probe = armed || env_int("TTAMD_GEMM_CLOCK_PROBE", 0) != 0;
     if (probe && !probe_buf && hipMalloc((void **)&probe_buf, 16) != hipSuccess) probe_buf = nullptr;
     g.probe = probe ? probe_buf : nullptr;
     void *fargs[] = {&g};
@@ -145,7 +151,11 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     if (lrc == 0 && g.probe) {
       unsigned long long h[2] = {0, 0};
       if (hipStreamSynchronize((hipStream_t)stream) == hipSuccess &&
-          hipMemcpy(h, probe_buf, 16, hipMemcpyDeviceToHost) == hipSuccess && h[1])
+          hipMemcpy(h, probe_buf, 16, hipMemcpyDeviceToHost) == hipSuccess && h[1]) {
+        g_probe_last[0] = h[0];
+        g_probe_last[1] = h[1];
+      }
+      if (h[1] && !armed)
         fprintf(stderr, "[ttamd] %s: workgroup 0 ran %llu core cycles in %.1f us -> %.3f GHz\n", fast_name, h[0],
                 h[1] / 100.0, h[0] / (h[1] * 10.0));
     }
@@ -179,6 +189,15 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
 } // namespace
 
 extern "C" {
+
+int rt_gemm_clock_probe(int32_t arm, uint64_t reading[2]) {
+  if (arm) g_probe_armed.store(1);
+  if (reading) {
+    reading[0] = g_probe_last[0].load();
+    reading[1] = g_probe_last[1].load();
+  }
+  return RT_OK;
+}
 
 int tt_matmul_kernel_tma(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c, int32_t M,
                          int32_t N, int32_t K, int32_t BLOCK_SIZE_M, int32_t BLOCK_SIZE_N,

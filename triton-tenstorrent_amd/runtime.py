@@ -104,6 +104,7 @@ SYMBOLS = {
     "tt_matmul_kernel": (C.c_int, [_vp, _vp, _vp, _i32, _i32, _i32] + [C.c_int64] * 6 + [_i32] * 6 + [_G, _vp]),
     "tt_attn_fwd": (C.c_int, [_f32, _vp, _i32, _i32, _DP, _DP, _DP, _DP, _i32, _i32, _i32, _i32, _i32, _G, _vp]),
     "tt_last_kernel_name": (C.c_char_p, []),
+    "rt_gemm_clock_probe": (C.c_int, [_i32, C.POINTER(C.c_uint64)]),
 }
 
 _lib = None
@@ -165,6 +166,14 @@ def device_props() -> dict:
 
 def last_kernel_name() -> str:
     return load().tt_last_kernel_name().decode()
+
+
+def gemm_clock_probe(arm: bool = False):
+    """``arm``: the next launch of the 16-bit macro-tile GEMM records its clock (and is synchronous).  Returns the
+    last record as (core cycles, 100 MHz ticks, GHz) or None."""
+    r = (C.c_uint64 * 2)()
+    check(load().rt_gemm_clock_probe(1 if arm else 0, r))
+    return (int(r[0]), int(r[1]), r[0] / r[1] / 10.0) if r[1] else None
 
 
 def grid3(gx: int, gy: int = 1, gz: int = 1):
