@@ -191,7 +191,28 @@ def main() -> int:
             # the MFMA peak at the granted clock, and the kernel against that
             extra["gemm_bf16_8192"]["peak_at_granted_clock_TFLOPs"] = round(PEAK_BF16_TFLOPS * ghz / (props["clock_khz"] / 1e6), 1)
             extra["gemm_bf16_8192"]["frac_at_granted_clock"] = round(value / (PEAK_BF16_TFLOPS * ghz / (props["clock_khz"] / 1e6)), 4)
-        del a, b, c, ad, bd, cd
+        # ... and the ceiling to lay it against: the same MFMAs alone (no LDS, no copies, no barrier) on the
+        # benchmark's own operand values, one wavefront per SIMD on every CU, and the clock the box grants under THAT
+        import ctypes as C
+        lib = rt.init(0)
+        mod, kh = C.c_void_p(), C.c_void_p()
+        rt.check(lib.rt_builtin_module(b"gemm", C.byref(mod)))
+        rt.check(lib.rt_get_kernel(mod, b"gemm_mfma_ceiling_bf16", C.byref(kh)))
+        sink = torch.zeros(4, device="cuda")
+        probe = torch.zeros(2, device="cuda", dtype=torch.int64)
+        iters = 3000
+        vals = [C.c_int(iters), C.c_void_p(a.data_ptr()), C.c_void_p(sink.data_ptr()), C.c_void_p(probe.data_ptr())]
+        kargs = (C.c_void_p * 4)(*[C.cast(C.pointer(v), C.c_void_p) for v in vals])     # (src: 64 x 16 x 256 fragments of A)
+        cus = props["multiprocessor_count"]
+        g3, b3 = rt.grid3(cus), rt.grid3(256)
+        avg_c, per_c, _ = _events_time(lambda: rt.check(lib.rt_launch(kh, g3, b3, 0, C.c_void_p(stream), kargs, 4)),
+                                       max(5, steps // 2), 3, stream)
+        extra["gemm_bf16_8192"]["mfma_only_TFLOPs"] = round(4 * cus * iters * 2.0 ** 20 / (avg_c * 1e-3) / 1e12, 1)
+        pr = probe.tolist()
+        if pr[1]:
+            extra["gemm_bf16_8192"]["mfma_only_clock_GHz"] = round(pr[0] / pr[1] / 10.0, 3)
+        extra["gemm_bf16_8192"]["kernel_over_mfma_only"] = round(value / extra["gemm_bf16_8192"]["mfma_only_TFLOPs"], 4)
+        del a, b, c, ad, bd, cd, sink, probe
         # shapes that are not whole 256x256x128 macro tiles run the same kernel's clamping instantiation
         ragged = {}
         for (m_, n_, k_) in ((8000, 8192, 8192), (8192, 8192, 8160)):

@@ -632,3 +632,26 @@ def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
     for _ in range(2):
         assert torch.equal(K.matmul_fp8_scaled(qa, qb, sa, sb), first)
     assert K.matmul_kernel_tma_fp8_scaled._plan is not None
+
+
+@pytest.mark.gpu
+def test_clock_probe_reports_a_plausible_core_clock_and_leaves_results_alone():
+    """rt_gemm_clock_probe arms ONE launch of the 16-bit macro-tile GEMM: that launch records workgroup 0's core
+    cycles and wall ticks (the clock granted under load), computes what it always computes, and the launches after
+    it are not probed."""
+    torch.manual_seed(5)
+    a = (torch.randn(4096, 4096, device="cuda") / 64).to(torch.bfloat16)
+    b = (torch.randn(4096, 4096, device="cuda") / 64).to(torch.bfloat16)
+    want = K.matmul_tma(a, b)
+    assert rt.last_kernel_name() == "gemm_tile_bf16_epi0"
+    for _ in range(10):
+        K.matmul_tma(a, b)
+    rt.gemm_clock_probe(arm=True)
+    got = K.matmul_tma(a, b)
+    torch.cuda.synchronize()
+    cycles, ticks, ghz = rt.gemm_clock_probe()
+    assert cycles > 0 and ticks > 0 and 0.4 < ghz < 2.6, (cycles, ticks, ghz)
+    assert torch.equal(got, want)
+    K.matmul_tma(a, b)                       # not armed any more: the record stays as it is
+    torch.cuda.synchronize()
+    assert rt.gemm_clock_probe()[:2] == (cycles, ticks)

@@ -882,4 +882,48 @@ GEMM_TILED(gemm_tiled_f16_epi3, EPI_LEAKY_RELU)
 GEMM_TILED_RAGGED(gemm_tiledragged_f16_epi0, EPI_NONE)
 GEMM_TILED_RAGGED(gemm_tiledragged_f16_epi3, EPI_LEAKY_RELU)
 
+// Diagnostic, launched by bench.py only: what the part sustains for this kernel's MFMAs alone.  One wavefront per SIMD
+// holds eight A and eight B fragments taken from `src` (so that the operand statistics are the benchmark's: MFMAs on
+// zeros draw far less power and run at the full clock) and issues the 64 MFMAs of a K step, in the kernel's order and
+// on AGPR accumulators, `iters` times: no LDS, no copies, no barrier.  The kernels above are bounded by power, so this
+// figure, at the clock the box grants under it, is the ceiling they can be laid against (2^20 flops per wavefront and
+// iteration; 64 x 16 x 256 fragments of 16 bytes are read from `src`).
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mfma_ceiling_bf16(int iters, const bf16x8 *src,
+                                                                                                      float *sink,
+                                                                                                      unsigned long long *probe) {
+  // probe: workgroup 0 leaves {core-clock cycles, 100 MHz ticks} of its run there (the clock granted under this loop)
+  const long long probe_c0 = clock64(), probe_w0 = wall_clock64();
+  bf16x8 a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = src[((blockIdx.x & 63) * 16 + i) * 256 + threadIdx.x];
+    b[i] = src[((blockIdx.x & 63) * 16 + 8 + i) * 256 + threadIdx.x];
+  }
+  f32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int n = 0; n < 64; ++n) {
+      const int i = n >> 3, j = (i & 1) ? 7 - (n & 7) : (n & 7);   // odd row blocks walk backwards, as in the K step
+      fast::MFMA<DT_BF16>::run(b[j], a[i], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  float t = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) t += acc[i][j][e];
+  if (t == 12345.678f) sink[0] = t;   // (keeps the accumulators alive; never true in practice)
+  if (probe && blockIdx.x == 0 && threadIdx.x == 0) {
+    probe[0] = (unsigned long long)(clock64() - probe_c0);
+    probe[1] = (unsigned long long)(wall_clock64() - probe_w0);
+  }
+}
+
 } // extern "C"
