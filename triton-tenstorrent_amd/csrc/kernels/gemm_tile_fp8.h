@@ -410,8 +410,16 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
             *(uint32_t *)((uint8_t *)g.c + mi * g.ldc + n) = q;
           }
         } else {
-          // 16-byte stores as in the 16-bit kernel: the lane pair (l, l+32) exchanges its middle column groups
-          // (v_permlane32_swap), so the lower lane holds columns 0-7 and the upper lane 8-15 of each 16
+          // 16-byte stores, four lanes to a row's 64 contiguous bytes.  A lane holds columns 8g + 4hi .. +3 (g = 0..3) of
+          // row l % 32 of the 32x32 block.  First the lane pair (l, l+32) exchanges its middle column groups
+          // (v_permlane32_swap): the lower lane then holds columns 0-7 and 16-23, the upper one 8-15 and 24-31.  Then
+          // sixteen-lane rows 0 / 1 and 2 / 3 of the wavefront exchange (v_permlane16_swap: odd rows of its first
+          // operand <-> even rows of its second) the second piece of the lanes that hold block row r < 16 with the first
+          // piece of the lanes that hold block row r + 16: afterwards every lane's first piece belongs to block row
+          // l % 16 and its second to block row l % 16 + 16, at columns {0, 16, 8, 24}[l / 16] .. +7, so that one store
+          // instruction writes sixteen rows in segments of 64 bytes (32-byte segments before: the writes that reached
+          // memory were 1.15 times the bytes of C).
+          u32x4 pc[2];      // after the swaps: [0] block row l % 16, [1] block row l % 16 + 16
 #pragma unroll
           for (int q = 0; q < 2; ++q) {
             u32x2 p[2];
@@ -428,9 +436,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
             }
             asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p[0].x), "+v"(p[1].x));
             asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(p[0].y), "+v"(p[1].y));
-            const int64_t n = n0 + wn * 128 + j * 32 + q * 16 + hi * 8;
-            if (RAGGED && (mi >= g.M || n >= g.N)) continue;     // N is a multiple of 16
-            *(u32x4 *)((uint16_t *)g.c + mi * g.ldc + n) = (u32x4){p[0].x, p[0].y, p[1].x, p[1].y};
+            pc[q] = (u32x4){p[0].x, p[0].y, p[1].x, p[1].y};   // columns q*16 + hi*8 .. +7 of block row l % 32
+          }
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(pc[0].x), "+v"(pc[1].x));
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(pc[0].y), "+v"(pc[1].y));
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(pc[0].z), "+v"(pc[1].z));
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(pc[0].w), "+v"(pc[1].w));
+          const int64_t n = n0 + wn * 128 + j * 32 + ((lane >> 4) & 1) * 16 + hi * 8;
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const int64_t mr = m0 + wm * (32 * MB) + i * 32 + half * 16 + (lane & 15);
+            if (RAGGED && (mr >= g.M || n >= g.N)) continue;     // N is a multiple of 16
+            *(u32x4 *)((uint16_t *)g.c + mr * g.ldc + n) = pc[half];
           }
         }
       }
