@@ -179,15 +179,20 @@ def main() -> int:
         # The kernel is bounded by power, so its rate follows the core clock the box grants under it (1.6-1.8 GHz
         # against the 2.4 GHz the peak is quoted at), and boxes differ.  One untimed launch behind a run of ordinary
         # ones reports workgroup 0's core cycles and wall ticks: with it two lines from two boxes can be compared.
-        for _ in range(20):
+        readings = []
+        for _ in range(5):          # five probed launches, each behind a run of ordinary ones; the median clock
+            for _ in range(8):
+                gemm_step()
+            rt.gemm_clock_probe(arm=True)
             gemm_step()
-        rt.gemm_clock_probe(arm=True)
-        gemm_step()
-        torch.cuda.synchronize()
-        reading = rt.gemm_clock_probe()
-        if reading is not None:
-            ghz = reading[2]
+            torch.cuda.synchronize()
+            r = rt.gemm_clock_probe()
+            if r is not None:
+                readings.append(r[2])
+        if readings:
+            ghz = statistics.median(readings)
             extra["gemm_bf16_8192"]["clock_under_load_GHz"] = round(ghz, 3)
+            extra["gemm_bf16_8192"]["clock_under_load_GHz_minmax"] = [round(min(readings), 3), round(max(readings), 3)]
             # the MFMA peak at the granted clock, and the kernel against that
             extra["gemm_bf16_8192"]["peak_at_granted_clock_TFLOPs"] = round(PEAK_BF16_TFLOPS * ghz / (props["clock_khz"] / 1e6), 1)
             extra["gemm_bf16_8192"]["frac_at_granted_clock"] = round(value / (PEAK_BF16_TFLOPS * ghz / (props["clock_khz"] / 1e6)), 4)

@@ -48,13 +48,31 @@ def test_transcendental_unary_within_two_ulp(op):
         assert np.all(err <= 2 * np.spacing(np.abs(want[fin])))
 
 
+@pytest.mark.parametrize("op", ["cos", "sin"])
+def test_trig_on_both_sides_of_the_library_threshold(op):
+    """Below 2^17 the kernels reduce the argument themselves; from 2^17 on, inf and NaN included, a wavefront
+    branches to the library routine for the lanes that need it.  Blocks in which no lane, some lanes and every lane
+    take that branch, and the values right at the threshold."""
+    g = torch.Generator().manual_seed(17)
+    small = (torch.rand(64 * 300, generator=g) * 2 - 1) * 1.3e5
+    large = torch.randn(64 * 300, generator=g) * 1e7
+    mixed = torch.where(torch.rand(64 * 300, generator=g) < 0.03, large, small)
+    edge = torch.tensor([131071.99, 131072.0, 131072.01, -131071.99, -131072.0, 1e30, -1e30, float("inf"), float("nan")])
+    x = torch.cat([small, mixed, large, edge])
+    got = K.unary(op, x.cuda()).cpu().numpy()
+    want = orc.unary(op, x.numpy())
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    fin = np.isfinite(want)
+    assert np.max(np.abs(got[fin].astype(np.float64) - want[fin].astype(np.float64))) <= 2e-6
+
+
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "maximum", "minimum"])
 def test_binary_bit_exact(op):
     got = K.binary(op, X.cuda(), Y.cuda()).cpu().numpy()
     assert _bits_equal(got, orc.binary(op, X.numpy(), Y.numpy()))
     # signed zeros and NaN of maximum / minimum, both operand orders
-    a = torch.tensor([0.0, -0.0, float("nan"), 1.0, -0.0], dtype=torch.float32)
-    b = torch.tensor([-0.0, 0.0, 1.0, float("nan"), -0.0], dtype=torch.float32)
+    a = torch.tensor([0.0, -0.0, float("nan"), 1.0, -0.0, float("inf"), float("-inf"), float("nan")], dtype=torch.float32)
+    b = torch.tensor([-0.0, 0.0, 1.0, float("nan"), -0.0, float("nan"), 5.0, float("inf")], dtype=torch.float32)
     got = K.binary(op, a.cuda(), b.cuda()).cpu().numpy()
     assert _bits_equal(got, orc.binary(op, a.numpy(), b.numpy()))
 
