@@ -310,6 +310,23 @@ def test_an_elf_image_goes_through_load_binary_and_the_launcher(tmp_path):
     assert not cpu_abi.is_elf_image(b'{"kernel": "add_kernel"}')
 
 
+def test_two_images_loaded_one_after_the_other_are_two_libraries(tmp_path):
+    """dlopen answers a path name it has seen with the library it loaded then, so images must never share one."""
+    libs = []
+    for value in (11, 22):
+        src, so = tmp_path / f"k{value}.c", tmp_path / f"libk{value}.so"
+        src.write_text("#include <stdint.h>\nvoid which(int32_t *out, int32_t *launch_sz, int32_t *launch_id, int8_t *smem, void *barrier) "
+                       f"{{ (void)launch_sz; (void)launch_id; (void)smem; (void)barrier; out[0] = {value}; }}\n")
+        subprocess.run(["gcc", "-shared", "-fPIC", "-O2", "-std=c99", str(src), "-o", str(so)], check=True)
+        libs.append(cpu_abi.load_image(so.read_bytes()))
+    outs = []
+    for lib_ in libs:
+        o = torch.zeros(1, dtype=torch.int32)
+        lib_.get_kernel("which", ["*i32"]).launch((1, ), o)
+        outs.append(int(o[0]))
+    assert outs == [11, 22]
+
+
 def test_the_elf_route_loads_neither_the_gpu_library_nor_the_oracle(tmp_path):
     src, so = tmp_path / "k.c", tmp_path / "libk.so"
     src.write_text(KERNELS_C)

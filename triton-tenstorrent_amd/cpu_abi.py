@@ -235,17 +235,20 @@ def is_elf_image(kernel) -> bool:
 
 def load_image(image: bytes) -> CPULibrary:
     """A shared object handed over as bytes, the way the reference's launcher hands one to its runtime
-    (``device.load_library(kernel, len(kernel))``, backend/driver.py:72).  The image goes into an anonymous
-    in-memory file that ``dlopen`` maps; nothing is left on disk."""
+    (``device.load_library(kernel, len(kernel))``, backend/driver.py:72).  The image is written to a file of its own
+    in the temporary directory, mapped by ``dlopen`` and unlinked at once: the mapping keeps the pages, nothing is left
+    on disk, and two images never meet under one path name (``dlopen`` answers a path it has seen before with the
+    library it loaded then)."""
+    import tempfile
     if not is_elf_image(image):
         raise ValueError("not an ELF image")
-    fd = os.memfd_create("ttamd_cpu_kernel", 0)
+    fd, path = tempfile.mkstemp(prefix="ttamd_cpu_kernel_", suffix=".so")
     try:
-        with os.fdopen(os.dup(fd), "wb") as f:
+        with os.fdopen(fd, "wb") as f:
             f.write(bytes(image))
-        return CPULibrary(f"/proc/self/fd/{fd}")
+        return CPULibrary(path)
     finally:
-        os.close(fd)        # the mapping made by dlopen keeps the pages
+        os.unlink(path)
 
 
 def expand_signature(sig_types: Sequence[str]) -> list[str]:
