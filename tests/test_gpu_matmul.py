@@ -472,6 +472,26 @@ def test_full_size_8192_properties():
     assert torch.equal(K.matmul_tma(a * 2, b), c * 2)
 
 
+def test_streaming_stores_of_an_output_beyond_the_memory_side_cache():
+    """A C of more than 256 MiB with K <= 2048 leaves the kernel in cache-bypassing stores (another instantiation
+    of the epilogue): small integers make every element exact, so the whole 512 MiB output is compared, ragged
+    edge included."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for (M, N, K_), kernel in (((16384, 16384, 256), "gemm_tile_bf16_epi0"), ((16380, 16392, 136), "gemm_ragged_bf16_epi0")):
+        a = torch.randint(-3, 4, (M, K_), device="cuda", generator=g).to(torch.bfloat16)
+        b = torch.randint(-3, 4, (K_, N), device="cuda", generator=g).to(torch.bfloat16)
+        cbuf = torch.full((M, N + 8), 7.5, device="cuda", dtype=torch.bfloat16)
+        c = cbuf[:, :N]
+        ad, bd, cd = (TensorDescriptor.from_tensor(t, [32, 32]) for t in (a, b, c))
+        K.matmul_kernel_tma[(-(-M // 128) * -(-N // 128), )](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False)
+        assert rt.last_kernel_name() == kernel
+        for r0 in range(0, M, 4096):          # (by slabs: the float reference of a slab is 256 MiB)
+            r1 = min(r0 + 4096, M)
+            assert torch.equal(c[r0:r1], (a[r0:r1].float() @ b.float()).to(torch.bfloat16))   # (sums < 2^24: exact in fp32)
+        assert torch.all(cbuf[:, N:] == 7.5)
+        del a, b, c, cbuf
+
+
 # ---- the fp8 fast path (scaled 32x32x64 MFMA, transposing byte reads) --------
 @pytest.mark.parametrize("M,N,K_", [(256, 256, 256), (512, 768, 512), (1024, 1024, 1024), (256, 512, 2048)])
 def test_fp8_fast_path(M, N, K_):

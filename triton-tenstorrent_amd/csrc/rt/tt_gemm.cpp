@@ -133,7 +133,9 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   // whose rows can be fetched in 16-byte pieces (N and K multiples of 8; a last K step that ends past K has its
   // copies redirected into the matrix and the surplus cleared in shared memory).
   const bool ragged_shape = !fast_shape && N % 8 == 0 && K % 8 == 0 && g.lda < (1 << 23) && g.ldb < (1 << 23);
-  if (full_grid && half_io && (fast_shape || ragged_shape) && fast_align && !nan_shows && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+  // (these kernels do not multiply by g.scale: no entry point sends 16-bit operands with another scale than 1)
+  if (full_grid && half_io && g.scale == 1.0f && (fast_shape || ragged_shape) && fast_align && !nan_shows &&
+      !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     char fast_name[64];
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
              epi);
