@@ -556,6 +556,21 @@ def test_fp8_full_size_8192_properties():
     assert torch.equal(K.matmul_fp8_scaled(qa, eye, 1.0, 1.0), qa.to(torch.bfloat16))   # e4m3 values are exact in bf16
 
 
+def test_fp8_streaming_stores_of_an_output_beyond_the_memory_side_cache():
+    """The fp8 kernels' cache-bypassing variants (a 16-bit C of more than 256 MiB, K <= 4096): small integers, so
+    the whole 512 MiB output is compared bit for bit, whole tiles and clamped."""
+    g = torch.Generator(device="cuda").manual_seed(6)
+    for (M, N, K_), kernel in (((16384, 16384, 256), "gemm_tile_fp8_bf16_stream"), ((16380, 16400, 192), "gemm_ragged_fp8_bf16_stream")):
+        a = torch.randint(-4, 5, (M, K_), device="cuda", generator=g).float()
+        b = torch.randint(-4, 5, (K_, N), device="cuda", generator=g).float()
+        c = K.matmul_fp8_scaled(a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn), 0.5, 4.0)
+        assert rt.last_kernel_name() == kernel
+        for r0 in range(0, M, 4096):
+            r1 = min(r0 + 4096, M)
+            assert torch.equal(c[r0:r1], ((a[r0:r1] @ b) * 2).to(torch.bfloat16))   # (sums < 2^24: exact in fp32)
+        del a, b, c
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_nan_padded_descriptors(dtype):
     """`padding="nan"` (reference backend/driver.py:322-329): elements of A and B outside the matrix read as NaN.

@@ -108,6 +108,28 @@ def test_error_paths_return_codes():
     torch.cuda.synchronize()
 
 
+def test_first_large_launch_on_a_new_stream():
+    """The buffer of partial results of a stream is allocated and cleared at the stream's first large launch; the
+    clearing is ordered in that stream (a clear in the null stream is not waited for by a non-blocking stream and
+    could reset the arrival counter under the first launch).  Eight new streams, the first launch of each checked."""
+    rng = np.random.default_rng(11)
+    x = rng.integers(-2**31, 2**31 - 1, 1 << 20, dtype=np.int64).astype(np.int32)
+    xg = torch.from_numpy(x).cuda()
+    want = orc.reduce1d(x, "sum", orc.I32)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(8)]
+    outs = []
+    for st in streams:
+        with torch.cuda.stream(st):
+            outs.append(K.reduce1d("sum", xg))
+            outs.append(K.reduce1d("sum", xg))
+    torch.cuda.synchronize()
+    for got in outs:
+        assert got.cpu().numpy()[0] == want
+    for st in streams:
+        assert rt.load().rt_release_stream(C.c_void_p(st.cuda_stream)) == rt.RT_OK
+
+
 def test_large_blocks_across_workgroups_streams_and_repeats():
     """A block of 128 KiB and more is folded by several workgroups through a per-stream buffer of partial results:
     repeated launches on one stream, launches on two streams at once, an operand off the 16-byte grid (one

@@ -39,7 +39,12 @@ typedef __attribute__((address_space(3))) void lds_void;
 // the stores are clipped.
 // MB = 2: the half-tile pass over the tail of the persistent loop, as in the 16-bit kernel: a workgroup computes a
 // 128x256 half of a macro tile, each wavefront 64x128 (2x4 accumulators), two A slabs and six copies per step.
-template <int OUT_DT, bool RAGGED = false, int MB = 4>
+// STREAM: the stores of a 16-bit C go past the caches: the host's choice for an output that the 256 MiB memory-side
+// cache does not hold (a plain store leaves its line there and in the L2, and a C beyond that size only evicts
+// operands on its way through: 16384 x 16384 x 1024 runs 28 % faster with streaming stores and x 4096 8.6 %, x 8192
+// the same; 8192^3, whose C fits, slower).  The variants are kernels of their own: the two forms of the epilogue
+// inside one kernel cost the benchmark shapes 1-2 %.
+template <int OUT_DT, bool RAGGED = false, int MB = 4, bool STREAM = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -447,7 +452,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
           for (int half = 0; half < 2; ++half) {
             const int64_t mr = m0 + wm * (32 * MB) + i * 32 + half * 16 + (lane & 15);
             if (RAGGED && (mr >= g.M || n >= g.N)) continue;     // N is a multiple of 16
-            *(u32x4 *)((uint16_t *)g.c + mr * g.ldc + n) = pc[half];
+            if constexpr (STREAM)
+              __builtin_nontemporal_store(pc[half], (u32x4 *)((uint16_t *)g.c + mr * g.ldc + n));
+            else
+              *(u32x4 *)((uint16_t *)g.c + mr * g.ldc + n) = pc[half];
           }
         }
       }
@@ -460,33 +468,37 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
 extern "C" {
 
-#define GEMM_TILE_FP8(name, OUT)                                                                    \
+#define GEMM_TILE_FP8(name, OUT, STREAM)                                                            \
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                    \
-    fast8::body<OUT, false, 4>(g, ring);                                                             \
-    fast8::body<OUT, false, 2>(g, ring);                                                             \
+    fast8::body<OUT, false, 4, STREAM>(g, ring);                                                     \
+    fast8::body<OUT, false, 2, STREAM>(g, ring);                                                     \
   }
 
-GEMM_TILE_FP8(gemm_tile_fp8_bf16, DT_BF16)
-GEMM_TILE_FP8(gemm_tile_fp8_f16, DT_F16)
-GEMM_TILE_FP8(gemm_tile_fp8_fp8, DT_FP8)
+GEMM_TILE_FP8(gemm_tile_fp8_bf16, DT_BF16, false)
+GEMM_TILE_FP8(gemm_tile_fp8_f16, DT_F16, false)
+GEMM_TILE_FP8(gemm_tile_fp8_fp8, DT_FP8, false)
+GEMM_TILE_FP8(gemm_tile_fp8_bf16_stream, DT_BF16, true)
+GEMM_TILE_FP8(gemm_tile_fp8_f16_stream, DT_F16, true)
 
-#define GEMM_RAGGED_FP8(name, OUT)                                                                  \
+#define GEMM_RAGGED_FP8(name, OUT, STREAM)                                                          \
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                    \
-    fast8::body<OUT, true, 4>(g, ring);                                                              \
-    fast8::body<OUT, true, 2>(g, ring);                                                              \
+    fast8::body<OUT, true, 4, STREAM>(g, ring);                                                      \
+    fast8::body<OUT, true, 2, STREAM>(g, ring);                                                      \
   }
-GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16, DT_BF16)
-GEMM_RAGGED_FP8(gemm_ragged_fp8_f16, DT_F16)
-GEMM_RAGGED_FP8(gemm_ragged_fp8_fp8, DT_FP8)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16, DT_BF16, false)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_f16, DT_F16, false)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_fp8, DT_FP8, false)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16_stream, DT_BF16, true)
+GEMM_RAGGED_FP8(gemm_ragged_fp8_f16_stream, DT_F16, true)
 
 } // extern "C"

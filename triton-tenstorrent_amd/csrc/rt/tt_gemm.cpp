@@ -175,9 +175,11 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = persistent_grid(tiles, true);
     void *fargs[] = {&g};
-    char fp8_name[48];
-    snprintf(fp8_name, sizeof(fp8_name), "gemm_%s_fp8_%s", fp8_shape ? "tile" : "ragged",
-             out == TT_BF16 ? "bf16" : out == TT_F16 ? "f16" : "fp8");
+    char fp8_name[64];
+    // a 16-bit C that the 256 MiB memory-side cache does not hold is stored past the caches while K is short
+    const bool past_caches = out != TT_FP8E4M3 && (int64_t)M * N * 2 > (256ll << 20) && K <= 4096;
+    snprintf(fp8_name, sizeof(fp8_name), "gemm_%s_fp8_%s%s", fp8_shape ? "tile" : "ragged",
+             out == TT_BF16 ? "bf16" : out == TT_F16 ? "f16" : "fp8", past_caches ? "_stream" : "");
     return launch("gemm", fp8_name, dim3(wgs), dim3(256), 0, stream, fargs, 1);
   }
 

@@ -34,7 +34,10 @@ void *partials_for(void *stream) {
   if (it != g_bufs.end()) return it->second;
   void *p = nullptr;
   if (hipMalloc(&p, ttamd::kReduceScratchBytes) != hipSuccess) return nullptr;
-  if (hipMemset(p, 0, ttamd::kReduceScratchBytes) != hipSuccess) {
+  // Cleared in the stream that will use it: hipMemset runs in the null stream, which a non-blocking stream does not
+  // wait for, so the first launch's workgroups could take their tickets before the counter was put to zero under
+  // them (no workgroup then sees the last ticket, nothing is stored, and the counter stays off for the launches after).
+  if (hipMemsetAsync(p, 0, ttamd::kReduceScratchBytes, (hipStream_t)stream) != hipSuccess) {
     (void)hipFree(p);
     return nullptr;
   }
