@@ -249,9 +249,11 @@ def test_causal_mask_is_the_sources_at_block_m_32(S, D, kernel):
 
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("Z,H,S,D", [(2, 32, 2304, 128), (1, 40, 3328, 128), (3, 3, 768, 128), (2, 32, 2272, 128),
-                                     (1, 33, 4000, 128), (5, 8, 1056, 128), (2, 32, 2304, 64), (3, 11, 3328, 64), (1, 5, 512, 64)])
+                                     (1, 33, 4000, 128), (5, 8, 1056, 128), (2, 32, 2304, 64), (3, 11, 3328, 64), (1, 5, 512, 64),
+                                     (2, 32, 1152, 256), (1, 40, 1664, 256), (3, 3, 384, 256), (1, 5, 128, 256)])
 def test_items_chained_inside_a_workgroup(causal, Z, H, S, D):
-    """The head dim 128 and 64 kernels walk (head, pair of query blocks) items on a persistent grid and lets each item's last
+    """The head dim 128, 64 and 256 kernels walk (head, pair of query blocks) items on a persistent grid (256-query blocks;
+    128-query blocks at head dim 256) and let each item's last
     copies fetch the first key blocks of the next one, which may belong to another head.  Shapes with more items
     than CUs (288 and 280 against 256), an odd number of query blocks (9, 13: the middle block is an item on its own,
     so items of one and of two blocks alternate), a head count that is not a multiple of 8, and lengths that are not
@@ -265,7 +267,7 @@ def test_items_chained_inside_a_workgroup(causal, Z, H, S, D):
     v = (v.float() + torch.arange(Z * H, device="cuda").view(Z, H, 1, 1).float() * 0.25).to(torch.bfloat16)
     sm = D ** -0.5
     o, M = K.attention(q, k, v, causal, sm, return_lse=True)
-    assert rt.last_kernel_name() == (f"attn_tile_d{D}" if S % 256 == 0 else f"attn_ragged_d{D}")
+    assert rt.last_kernel_name() == (f"attn_tile_d{D}" if S % (128 if D == 256 else 256) == 0 else f"attn_ragged_d{D}")
     heads = sorted({0, 1, Z * H // 2, Z * H - 2, Z * H - 1, 7, 8} & set(range(Z * H)))
     rows = torch.arange(S, device="cuda")
     for hh in heads:
@@ -276,6 +278,36 @@ def test_items_chained_inside_a_workgroup(causal, Z, H, S, D):
         ref = torch.softmax(s, -1) @ v[z, h].double()
         assert (o[z, h].double() - ref).abs().max() <= O_ATOL * max(1.0, float(v[z, h].float().abs().max()))
         assert (M[z, h].double() - torch.logsumexp(s, -1) / np.log(2.0)).abs().max() <= M_ATOL
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("S,D,kernel", [(1024, 128, "attn_tile_d128"), (1024, 256, "attn_tile_d256"), (1024, 64, "attn_tile_d64")])
+def test_row_maxima_that_climb_slowly_and_in_jumps(causal, S, D, kernel):
+    """The pipelined kernels keep a row's exponent reference until some row of the wavefront outgrows it by 2^8 and
+    only then rescale (a stated difference from a literal evaluation).  Scores that rise by 0.1 log2 units per key
+    (6.4 per 64-key block: several blocks pass between two rescales, and p reaches 2^8 in between), with a jump of 60
+    units at key 700 and another of 20 at key 900, against float64."""
+    from triton_tenstorrent_amd import runtime as rt
+    g = torch.Generator().manual_seed(S + D)
+    q = torch.randn(1, 2, S, D, generator=g) * 0.05
+    k = torch.randn(1, 2, S, D, generator=g) * 0.05
+    ramp = 0.1 / 1.44269504 * torch.arange(S).float()
+    ramp[700:] += 60 / 1.44269504
+    ramp[900:] += 20 / 1.44269504
+    q[..., 0] = 1.0
+    k[..., 0] = ramp
+    v = torch.randn(1, 2, S, D, generator=g)
+    q, k, v = (t.to(torch.bfloat16).cuda() for t in (q, k, v))
+    o, M = K.attention(q, k, v, causal, 1.0, return_lse=True)
+    assert rt.last_kernel_name() == kernel
+    rows = torch.arange(S, device="cuda")
+    for h in range(2):
+        s_ = q[0, h].double() @ k[0, h].double().T
+        if causal:
+            s_ = s_.masked_fill(rows[:, None] < rows[None, :], float("-inf"))
+        ref = torch.softmax(s_, -1) @ v[0, h].double()
+        assert (o[0, h].double() - ref).abs().max() <= O_ATOL
+        assert (M[0, h].double() - torch.logsumexp(s_, -1) / np.log(2.0)).abs().max() <= M_ATOL
 
 
 def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
