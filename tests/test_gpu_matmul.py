@@ -473,11 +473,10 @@ def test_full_size_8192_properties():
 
 
 def test_streaming_stores_of_an_output_beyond_the_memory_side_cache():
-    """A C of more than 256 MiB with K <= 2048 leaves the kernel in cache-bypassing stores (another instantiation
-    of the epilogue): small integers make every element exact, so the whole 512 MiB output is compared, ragged
-    edge included."""
+    """A C of more than 256 MiB with K <= 2048 goes to the kernels whose stores bypass the caches: small integers
+    make every element exact, so the whole 512 MiB output is compared, ragged edge included."""
     g = torch.Generator(device="cuda").manual_seed(5)
-    for (M, N, K_), kernel in (((16384, 16384, 256), "gemm_tile_bf16_epi0"), ((16380, 16392, 136), "gemm_ragged_bf16_epi0")):
+    for (M, N, K_), kernel in (((16384, 16384, 256), "gemm_tile_bf16_epi0_stream"), ((16380, 16392, 136), "gemm_ragged_bf16_epi0_stream")):
         a = torch.randint(-3, 4, (M, K_), device="cuda", generator=g).to(torch.bfloat16)
         b = torch.randint(-3, 4, (K_, N), device="cuda", generator=g).to(torch.bfloat16)
         cbuf = torch.full((M, N + 8), 7.5, device="cuda", dtype=torch.bfloat16)

@@ -79,54 +79,30 @@ template <int IN_DT> struct MFMA;
 // out the last MFMAs before it reads (see there).
 template <> struct MFMA<DT_BF16> {
   typedef bf16x8 vec;
-  // Z: the first MFMA into an accumulator of a tile takes 0 as its addend instead of the register (which is
-  // still named as read and written, so the allocation is the same as for every other MFMA of the loop)
-  template <bool Z = false> static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
-    if constexpr (Z)
-      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "+a"(c) : "v"(a), "v"(b));
-    else
-      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
   // The MFMA and, behind it, one direct-to-LDS copy (m0: its LDS destination, written by the compiler in front of
   // the statement): the MFMA is the wait state that the copy needs after a write to m0.
-  template <bool Z = false>
   static __device__ __forceinline__ void run_copy(vec a, vec b, f32x4 &c, uint32_t m0v, uint32_t voff, const uint8_t *src) {
-    if constexpr (Z)
-      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0\n\tglobal_load_lds_dwordx4 %4, %5"
-                   : "+a"(c)
-                   : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
-                   : "memory");
-    else
-      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
-                   : "+a"(c)
-                   : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
-                   : "memory");
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
+                 : "memory");
   }
 };
 template <> struct MFMA<DT_F16> {
   typedef f16x8 vec;
-  // Z: the first MFMA into an accumulator of a tile takes 0 as its addend instead of the register (which is
-  // still named as read and written, so the allocation is the same as for every other MFMA of the loop)
-  template <bool Z = false> static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
-    if constexpr (Z)
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "+a"(c) : "v"(a), "v"(b));
-    else
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  static __device__ __forceinline__ void run(vec a, vec b, f32x4 &c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
   // The MFMA and, behind it, one direct-to-LDS copy (m0: its LDS destination, written by the compiler in front of
   // the statement): the MFMA is the wait state that the copy needs after a write to m0.
-  template <bool Z = false>
   static __device__ __forceinline__ void run_copy(vec a, vec b, f32x4 &c, uint32_t m0v, uint32_t voff, const uint8_t *src) {
-    if constexpr (Z)
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0\n\tglobal_load_lds_dwordx4 %4, %5"
-                   : "+a"(c)
-                   : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
-                   : "memory");
-    else
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
-                   : "+a"(c)
-                   : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
-                   : "memory");
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
+                 : "+a"(c)
+                 : "v"(a), "v"(b), "{m0}"(m0v), "v"(voff), "s"(src)
+                 : "memory");
   }
 };
 
@@ -232,8 +208,17 @@ struct Ring {
 // the chip four workgroups to a tile.  A quarter's step moves 20 KiB for a quarter of the flops and its fragment
 // reads (18 per wavefront and 16 MFMAs) keep the LDS busier than the matrix pipe, so it runs at about two thirds of
 // the macro tile's rate: worth it only where the alternative is idle CUs.
+//
+// STREAM: the stores of C go past the caches.  A plain store leaves its line in the L2 and in the 256 MiB
+// memory-side cache, which drain it while the next tile multiplies; that is right while C fits there.  A larger C
+// only evicts operands on its way through, which shows where K is short and operands are re-read soon:
+// 16384 x 16384 x 1024 runs 8.5 % faster with streaming stores and x 2048 3.7 %, x 4096 0.6 % slower, 8192^3 0.5 %
+// slower and 8192 x 8192 x 1024 (a C of 128 MiB) 15 % slower.  The host picks the streaming kernels for a C beyond
+// 256 MiB at K <= 2048.  They are kernels of their own (plain epilogue only): with both forms of the stores inside
+// one kernel, several instantiations spilled copy offsets whose reloads the compiler then waits for inside the K
+// loop, with every copy in flight counted in (tile-major 8192^3: 1585 -> 1482 TFLOP/s).
 template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false,
-          bool QUARTERS = false>
+          bool QUARTERS = false, bool STREAM = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   static_assert(MB == 4 || ((MB == 2 || (MB == 1 && QUARTERS)) && SPLIT_TAIL), "part tiles exist for the tail passes only");
   // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
@@ -336,7 +321,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // The LDS reads of one step, in the order the MFMAs will want them:
   // b0.lo b0.hi a0 b1.lo b1.hi ... b7.lo b7.hi a1 ... a(NA-1)
   // (J: ring index of the stage, a constant wherever this is called)
-  auto rd = [&](Frags &f, const uint8_t *stage, int J, int r) __attribute__((always_inline)) {
+  auto rd = [&](Frags &f, const uint8_t *stage, int J, int r) {
     if constexpr (APAIR) {
       if (r == 2 || r >= 17) {
         const int i = r == 2 ? 0 : r - 16;
@@ -355,11 +340,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     }
   };
   // MFMA number n (0..NM-1) of a step, row-block major: needs a[n/8] and each b once per row block
-  // (z_: the tile's first step, whose MFMAs start the accumulators instead of adding to them)
-  auto mm = [&](Frags &f, int n, auto z_) __attribute__((always_inline)) {
+  auto mm = [&](Frags &f, int n) {
     // (odd row blocks walk the columns backwards: every MFMA then shares one operand with the one before it)
     const int i = n >> 3, j = (i & 1) ? 7 - (n & 7) : (n & 7);
-    X::template run<decltype(z_)::value>(f.b[j].v, f.a[i], acc[i][j]);
+    X::run(f.b[j].v, f.a[i], acc[i][j]);
   };
   // One direct-to-LDS copy: lane l's 16 bytes land at dst_slab + wave*1024 + 16*l.
   // Written as assembly on purpose: the compiler's own bookkeeping of such copies is
@@ -367,7 +351,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // unrelated), which would flatten the multi-step prefetch.  Completion is tracked by
   // hand instead: copies retire in issue order, and each step's barrier waits with
   // s_waitcnt vmcnt(n) for exactly the copies that the following reads depend on.
-  auto dma_plain = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) __attribute__((always_inline)) {
+  auto dma_plain = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
     // (m0 is the compiler's to write: it then sees a scalar instruction between the MFMA before and this statement
     // and does not pad with a wait state of its own; the one M0 needs before the copy reads it stays in here)
@@ -377,10 +361,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
                  : "memory");
   };
   // MFMA number n of a step and a copy in one statement (inside the K loop every copy rides behind an MFMA)
-  auto mm_copy = [&](Frags &f, int n, const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab, auto z_) __attribute__((always_inline)) {
+  auto mm_copy = [&](Frags &f, int n, const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
     const int i = n >> 3, j = (i & 1) ? 7 - (n & 7) : (n & 7);
     const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(dst_slab + lds_wave);
-    X::template run_copy<decltype(z_)::value>(f.b[j].v, f.a[i], acc[i][j], m0v, voff, src_uniform);
+    X::run_copy(f.b[j].v, f.a[i], acc[i][j], m0v, voff, src_uniform);
   };
 
   // RAGGED with K not a multiple of 32: the last step of every tile holds columns (A) and rows (B) past K:
@@ -459,12 +443,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // tile and the next and (RAGGED) between data and the page of zeros are not made at run time, and a copy's
   // source is one scalar address per operand and step plus the thread's offset for that slab
   // (f, n: the MFMA that the copy is issued behind, n < 0: none)
-  auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_, Frags &f, int n, auto z_) __attribute__((always_inline)) {
+  auto dma_single = [&](int kk, uint8_t *stage, int i, auto inner_, Frags &f, int n) {
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
     auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
-      if (n >= 0) mm_copy(f, n, src_uniform, voff, dst_slab, z_);
+      if (n >= 0) mm_copy(f, n, src_uniform, voff, dst_slab);
       else dma_plain(src_uniform, voff, dst_slab);
     };
     if constexpr (inner) {
@@ -507,12 +491,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   };
 
   // APAIR: copy number i (0..7) of the pair of steps (kk, kk+1), kk even, into pair buffer P
-  auto dma_pair = [&](int kk, int P, int i, auto inner_, Frags &f, int n, auto z_) __attribute__((always_inline)) {
+  auto dma_pair = [&](int kk, int P, int i, auto inner_, Frags &f, int n) {
     constexpr bool inner = decltype(inner_)::value;
     const bool over = !inner && kk >= nk;
     const int k = over ? kk - nk : kk;
     auto dma_one = [&](const uint8_t *src_uniform, uint32_t voff, uint8_t *dst_slab) {
-      if (n >= 0) mm_copy(f, n, src_uniform, voff, dst_slab, z_);
+      if (n >= 0) mm_copy(f, n, src_uniform, voff, dst_slab);
       else dma_plain(src_uniform, voff, dst_slab);
     };
     uint8_t *dst = ring.s[2 * P + (i >> 2)] + (i & 3) * 4096;
@@ -562,10 +546,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   //   pipeline's input queue, and its MFMAs stall with it.  (Placement matters little here: two MFMAs or four
   //   before the barrier, reads on every second MFMA, copies every third to seventh MFMA from the 7th to the 30th
   //   on all measured within 1 % of each other, 1477-1497 TFLOP/s on 8192^3; two reads per MFMA cost 1.5 %.)
-  auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_, auto z_) __attribute__((always_inline)) {
+  auto step = [&](auto I_, int k, Frags &c, Frags &p, auto inner_) {
     constexpr int I = decltype(I_)::value;
     uint8_t *cur = ring.s[I], *nxt = ring.s[(I + 1) % R];
-    mm(c, 0, z_);
+    mm(c, 0);
     FENCE();
     if constexpr (RAGGED && !decltype(inner_)::value) {
       if constexpr (APAIR && (I & 1)) {
@@ -612,7 +596,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         if (2 * (n - 1) < NR) rd(p, nxt, (I + 1) % R, 2 * (n - 1));
         if (2 * (n - 1) + 1 < NR) rd(p, nxt, (I + 1) % R, 2 * (n - 1) + 1);
         if (n % 3 == 0) {
-          dma_single(k + R, cur, n / 3 - 1, inner_, c, n, z_);
+          dma_single(k + R, cur, n / 3 - 1, inner_, c, n);
           with_copy = true;
         }
       } else {
@@ -621,29 +605,29 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           if constexpr (I & 1) {
             if (n >= 26 && n <= 59 && (n - 26) % 3 == 0) {
               const int c12 = (n - 26) / 3;
-              if (c12 < 8) dma_pair(k + 3, (I - 1) >> 1, c12, inner_, c, n, z_);
-              else dma_single(k + R, cur, MB + c12 - 8, inner_, c, n, z_);
+              if (c12 < 8) dma_pair(k + 3, (I - 1) >> 1, c12, inner_, c, n);
+              else dma_single(k + R, cur, MB + c12 - 8, inner_, c, n);
               with_copy = true;
             }
           } else {
             if (n >= 30 && n <= 54 && (n - 30) % 8 == 0) {
-              dma_single(k + R, cur, MB + (n - 30) / 8, inner_, c, n, z_);
+              dma_single(k + R, cur, MB + (n - 30) / 8, inner_, c, n);
               with_copy = true;
             }
           }
         } else if constexpr (MB == 4) {
           if (n >= 25 && n <= 60 && n % 5 == 0) {
-            dma_single(k + R, cur, n / 5 - 5, inner_, c, n, z_);
+            dma_single(k + R, cur, n / 5 - 5, inner_, c, n);
             with_copy = true;
           }
         } else {
           if (n % 5 == 0 && n <= 30) {
-            dma_single(k + R, cur, n / 5 - 1, inner_, c, n, z_);
+            dma_single(k + R, cur, n / 5 - 1, inner_, c, n);
             with_copy = true;
           }
         }
       }
-      if (!with_copy) mm(c, n, z_);   // (a copy took MFMA n with it)
+      if (!with_copy) mm(c, n);   // (a copy took MFMA n with it)
       FENCE();
     }
   };
@@ -661,20 +645,20 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   if constexpr (APAIR) {
     // in the order the steps of a turn issue them: pair (0,1), B 0, B 1, B 2, pair (2,3), B 3
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dma_pair(0, 0, i, std::false_type{}, f0, -1, std::false_type{});
+    for (int i = 0; i < 8; ++i) dma_pair(0, 0, i, std::false_type{}, f0, -1);
 #pragma unroll
     for (int s = 0; s < 3; ++s)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) dma_single(s, ring.s[s], MB + i, std::false_type{}, f0, -1, std::false_type{});
+      for (int i = 0; i < 4; ++i) dma_single(s, ring.s[s], MB + i, std::false_type{}, f0, -1);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) dma_pair(2, 1, i, std::false_type{}, f0, -1, std::false_type{});
+    for (int i = 0; i < 8; ++i) dma_pair(2, 1, i, std::false_type{}, f0, -1);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma_single(3, ring.s[3], MB + i, std::false_type{}, f0, -1, std::false_type{});
+    for (int i = 0; i < 4; ++i) dma_single(3, ring.s[3], MB + i, std::false_type{}, f0, -1);
   } else {
 #pragma unroll
     for (int s = 0; s < R; ++s)
 #pragma unroll
-      for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{}, f0, -1, std::false_type{});
+      for (int i = 0; i < MB + 4; ++i) dma_single(s, ring.s[s], i, std::false_type{}, f0, -1);
   }
   static_assert(DMA_PER_STEP == 8 && R == 4, "the hand-written vmcnt waits assume MB + 4 copies per step and 4 stages");
   if (RAGGED && k_tail && nk_real == 1) {   // a single data step: it is the one that ends past K
@@ -704,45 +688,40 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     int tm, tn, part;
     item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, part);
     const int64_t m0 = (int64_t)tm * BM + part * (64 * MB), n0 = (int64_t)tn * BN;
-    // The accumulators are not cleared: the MFMAs of the tile's first step take 0 as their addend (z_ of step).
-    // These statements emit nothing; they tell the compiler that the registers hold a new value from here on.
 #pragma unroll
     for (int i = 0; i < NA; ++i)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) asm volatile("" : "=a"(acc[i][j]));
+      for (int j = 0; j < 8; ++j) acc[i][j] = (f32x4){0, 0, 0, 0};
 
     int k = 0;
-    // one turn of the ring; `first`: the turn a tile starts with
-    auto turn = [&](auto inner_, auto first_) __attribute__((always_inline)) {
-      step(std::integral_constant<int, 0>{}, k, f0, f1, inner_, first_);
-      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, inner_, std::false_type{});
-      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, inner_, std::false_type{});
-      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, inner_, std::false_type{});
-      k += R;
-    };
     // turns of the ring whose copies (up to step k + 2R - 1) all carry this tile's data
     // (row-major operands whose last step ends past K: that step's copies need the redirection above, so it stays
     // out of these turns)
     const int nk_inner = nk_real - ((!TILED && k_tail) ? 1 : 0);
-    // The turns that do not qualify copy the next tile's first steps (this tile's again when there is none: a
-    // harmless refetch); RAGGED: where that tile lies is worked out only in front of them.
-    auto next_tile = [&]() __attribute__((always_inline)) {
-      if constexpr (RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
-    };
-    // The first turn is the one instantiation with the zero addend, and so takes the general form of the copies
-    // whether it qualifies or not.
-    const bool long_k = 2 * R <= nk_inner;
-    if (!long_k) next_tile();
-    turn(std::false_type{}, std::true_type{});
-    if (long_k) {
-      if (RAGGED && APAIR && __builtin_amdgcn_readfirstlane(vo_cur.last_row) >= BM - 1) {
-        // (a tile whose 256 rows all exist: the copies of A need no clamping)
-        while (k + 2 * R <= nk_inner) turn(std::integral_constant<int, 2>{}, std::false_type{});
+    if (RAGGED && APAIR && __builtin_amdgcn_readfirstlane(vo_cur.last_row) >= BM - 1) {
+      // (a tile whose 256 rows all exist: the copies of A need no clamping)
+      for (; k + 2 * R <= nk_inner; k += R) {
+        step(std::integral_constant<int, 0>{}, k, f0, f1, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::integral_constant<int, 2>{});
+        step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::integral_constant<int, 2>{});
       }
-      while (k + 2 * R <= nk_inner) turn(std::true_type{}, std::false_type{});
-      next_tile();
     }
-    while (k < nk) turn(std::false_type{}, std::false_type{});
+    for (; k + 2 * R <= nk_inner; k += R) {
+      step(std::integral_constant<int, 0>{}, k, f0, f1, std::true_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::true_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::true_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::true_type{});
+    }
+    // the remaining turns copy the next tile's first steps (this tile's again when there is none: a harmless
+    // refetch); RAGGED: where that tile lies is worked out only now
+    if constexpr (RAGGED) tile_bases(t + (int)gridDim.x < total ? t + (int)gridDim.x : t, a_nxt, b_nxt, vo_nxt);
+    for (; k < nk; k += R) {
+      step(std::integral_constant<int, 0>{}, k, f0, f1, std::false_type{});
+      step(std::integral_constant<int, 1>{}, k + 1, f1, f0, std::false_type{});
+      step(std::integral_constant<int, 2>{}, k + 2, f0, f1, std::false_type{});
+      step(std::integral_constant<int, 3>{}, k + 3, f1, f0, std::false_type{});
+    }
     // the ring already holds the next tile's first steps; move the tile window on
     a_cur = a_nxt;
     b_cur = b_nxt;
@@ -770,18 +749,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         brow[j] = *(const f32x4 *)((const float *)g.bias + (RAGGED ? min(n0 + wn * 128 + j * 16 + G4 * 4, (int64_t)g.N - 4)
                                                                    : n0 + wn * 128 + j * 16 + G4 * 4));
     }
-    // stream_: the stores bypass the caches.  A plain store leaves its line in the L2 and in the memory-side cache,
-    // which is what a C of up to that cache's size wants (the L2 drains it while the next tile multiplies); a C
-    // beyond that size only pushes the operands out on its way through, which shows where K is short:
-    // 16384 x 16384 x 1024 runs 8.5 % faster with streaming stores and x 2048 2.5 %, 8192^3 0.5 % slower and
-    // 8192 x 8192 x 1024 15 % slower.
-    auto store_tile = [&](auto stream_) __attribute__((always_inline)) {
     // the four columns n .. n+3 of row mi that this lane holds for (i, j), after scale, epilogue and rounding
     auto packed = [&](int i, int j, int64_t mi, int64_t n) {
       float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float x = acc[i][j][e];   // (g.scale is 1 for 16-bit operands: the host sends no other launch here)
+        const float x = acc[i][j][e] * g.scale;
         if constexpr (EPI == EPI_BIAS_ROW_GELU)
           v[e] = gelu_erf(x + brow[j][e]);
         else if constexpr (EPI == EPI_BIAS_ROW)
@@ -813,14 +786,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
           const int64_t nl = nb + G4 * 4, nh = nb + 16 + G4 * 4;
           u32x2 p0 = packed(i, 2 * jp, mb, RAGGED ? min(nl, (int64_t)g.N - 4) : nl);
           u32x2 p1 = packed(i, 2 * jp + 1, mb, RAGGED ? min(nh, (int64_t)g.N - 4) : nh);
-          const auto sx = __builtin_amdgcn_permlane16_swap(p0.x, p1.x, false, false);
-          const auto sy = __builtin_amdgcn_permlane16_swap(p0.y, p1.y, false, false);
-          p0 = (u32x2){sx[0], sy[0]};
-          p1 = (u32x2){sx[1], sy[1]};
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p0.x), "+v"(p1.x));
+          asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(p0.y), "+v"(p1.y));
           const int64_t n = nb + (G4 & 1) * 16 + (G4 >> 1) * 8;
           if (RAGGED && (mi >= g.M || n >= g.N)) continue;
           const int64_t coff = TILED ? (((mi >> 5) * ntn + (n >> 5)) << 10) + (mi & 31) * 32 + (n & 31) : mi * g.ldc + n;
-          if constexpr (decltype(stream_)::value)
+          if constexpr (STREAM)
             __builtin_nontemporal_store((u32x4){p0.x, p0.y, p1.x, p1.y}, (u32x4 *)((uint16_t *)g.c + coff));
           else
             *(u32x4 *)((uint16_t *)g.c + coff) = (u32x4){p0.x, p0.y, p1.x, p1.y};
@@ -841,13 +812,6 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         }
       }
     }
-    };
-    if constexpr (RAGGED && TILED) {
-      store_tile(std::false_type{});
-    } else {
-      if ((int64_t)g.M * g.N * 2 > (256ll << 20) && g.K <= 2048) store_tile(std::true_type{});
-      else store_tile(std::false_type{});
-    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the trailing refetches must land before the LDS is released
   if (MB == 4 && g.probe && blockIdx.x == 0 && tid == 0) {
@@ -860,45 +824,47 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
 extern "C" {
 
-#define GEMM_TILE(name, IN, OUT, EPI)                                                              \
+#define GEMM_TILE(name, IN, OUT, EPI, STREAM)                                                      \
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, OUT, EPI, false, false, 4, true, true>(g, ring);                                 \
-    fast::body<IN, OUT, EPI, false, false, 2, true, true>(g, ring);                                 \
-    fast::body<IN, OUT, EPI, false, false, 1, true, true>(g, ring);                                 \
+    fast::body<IN, OUT, EPI, false, false, 4, true, true, STREAM>(g, ring);                         \
+    fast::body<IN, OUT, EPI, false, false, 2, true, true, STREAM>(g, ring);                         \
+    fast::body<IN, OUT, EPI, false, false, 1, true, true, STREAM>(g, ring);                         \
   }
-#define GEMM_TILE_ALL_EPI(prefix, IN, OUT)             \
-  GEMM_TILE(prefix##_epi0, IN, OUT, EPI_NONE)           \
-  GEMM_TILE(prefix##_epi1, IN, OUT, EPI_BIAS_FULL)      \
-  GEMM_TILE(prefix##_epi2, IN, OUT, EPI_BIAS_ROW_GELU)  \
-  GEMM_TILE(prefix##_epi3, IN, OUT, EPI_LEAKY_RELU)     \
-  GEMM_TILE(prefix##_epi4, IN, OUT, EPI_BIAS_ROW)
+#define GEMM_TILE_ALL_EPI(prefix, IN, OUT)                    \
+  GEMM_TILE(prefix##_epi0, IN, OUT, EPI_NONE, false)           \
+  GEMM_TILE(prefix##_epi1, IN, OUT, EPI_BIAS_FULL, false)      \
+  GEMM_TILE(prefix##_epi2, IN, OUT, EPI_BIAS_ROW_GELU, false)  \
+  GEMM_TILE(prefix##_epi3, IN, OUT, EPI_LEAKY_RELU, false)     \
+  GEMM_TILE(prefix##_epi4, IN, OUT, EPI_BIAS_ROW, false)       \
+  GEMM_TILE(prefix##_epi0_stream, IN, OUT, EPI_NONE, true)
 
 GEMM_TILE_ALL_EPI(gemm_tile_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
 
 // the same kernels for M any, N % 8 == 0, K % 8 == 0 (a last 32-deep step that ends past K is cleared in LDS)
-#define GEMM_TILE_RAGGED(name, IN, OUT, EPI)                                                       \
+#define GEMM_TILE_RAGGED(name, IN, OUT, EPI, STREAM)                                               \
   __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
     __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
     __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
     fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, OUT, EPI, false, true, 4, true, true>(g, ring);                                  \
-    fast::body<IN, OUT, EPI, false, true, 2, true, true>(g, ring);                                  \
-    fast::body<IN, OUT, EPI, false, true, 1, true, true>(g, ring);                                  \
+    fast::body<IN, OUT, EPI, false, true, 4, true, true, STREAM>(g, ring);                          \
+    fast::body<IN, OUT, EPI, false, true, 2, true, true, STREAM>(g, ring);                          \
+    fast::body<IN, OUT, EPI, false, true, 1, true, true, STREAM>(g, ring);                          \
   }
-#define GEMM_TILE_RAGGED_ALL_EPI(prefix, IN, OUT)             \
-  GEMM_TILE_RAGGED(prefix##_epi0, IN, OUT, EPI_NONE)           \
-  GEMM_TILE_RAGGED(prefix##_epi1, IN, OUT, EPI_BIAS_FULL)      \
-  GEMM_TILE_RAGGED(prefix##_epi2, IN, OUT, EPI_BIAS_ROW_GELU)  \
-  GEMM_TILE_RAGGED(prefix##_epi3, IN, OUT, EPI_LEAKY_RELU)     \
-  GEMM_TILE_RAGGED(prefix##_epi4, IN, OUT, EPI_BIAS_ROW)
+#define GEMM_TILE_RAGGED_ALL_EPI(prefix, IN, OUT)                    \
+  GEMM_TILE_RAGGED(prefix##_epi0, IN, OUT, EPI_NONE, false)           \
+  GEMM_TILE_RAGGED(prefix##_epi1, IN, OUT, EPI_BIAS_FULL, false)      \
+  GEMM_TILE_RAGGED(prefix##_epi2, IN, OUT, EPI_BIAS_ROW_GELU, false)  \
+  GEMM_TILE_RAGGED(prefix##_epi3, IN, OUT, EPI_LEAKY_RELU, false)     \
+  GEMM_TILE_RAGGED(prefix##_epi4, IN, OUT, EPI_BIAS_ROW, false)       \
+  GEMM_TILE_RAGGED(prefix##_epi0_stream, IN, OUT, EPI_NONE, true)
 GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
 

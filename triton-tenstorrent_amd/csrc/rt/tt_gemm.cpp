@@ -133,12 +133,12 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   // whose rows can be fetched in 16-byte pieces (N and K multiples of 8; a last K step that ends past K has its
   // copies redirected into the matrix and the surplus cleared in shared memory).
   const bool ragged_shape = !fast_shape && N % 8 == 0 && K % 8 == 0 && g.lda < (1 << 23) && g.ldb < (1 << 23);
-  // (these kernels do not multiply by g.scale: no entry point sends 16-bit operands with another scale than 1)
-  if (full_grid && half_io && g.scale == 1.0f && (fast_shape || ragged_shape) && fast_align && !nan_shows &&
-      !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
+  if (full_grid && half_io && (fast_shape || ragged_shape) && fast_align && !nan_shows && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     char fast_name[64];
-    snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
-             epi);
+    // a C that the 256 MiB memory-side cache does not hold is stored past the caches while K is short (plain epilogue)
+    const bool past_caches = epi == TT_EPI_NONE && (int64_t)M * N * 2 > (256ll << 20) && K <= 2048;
+    snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d%s", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
+             epi, past_caches ? "_stream" : "");
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
     const uint32_t wgs = persistent_grid(tiles, true, true);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
