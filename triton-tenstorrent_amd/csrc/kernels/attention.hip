@@ -542,8 +542,7 @@ ATTN_RAGGED(64)
     __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
     fastattn::body<D, RAGGED, 4>(a, lds0, lds1);                                           \
   }
-// (whole 128-query blocks at head dim 256: attn_tile_d256 in attention_pipe256.h)
-ATTN_TILE4(attn_ragged_d256, 256, true)
+// (head dim 256: attn_tile_d256 and attn_ragged_d256 in attention_pipe256.h)
 
 } // extern "C"
 

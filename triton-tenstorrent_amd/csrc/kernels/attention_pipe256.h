@@ -1,5 +1,6 @@
-// attn_tile_d256: _attn_fwd (examples/fused-attn/06-fused-attention.py:33-90, 143-215) at head dim 256 on whole
-// 128-query blocks, as the software pipeline of attention_pipe.h re-cut for one wavefront per SIMD.
+// attn_tile_d256, attn_ragged_d256: _attn_fwd (examples/fused-attn/06-fused-attention.py:33-90, 143-215) at head dim
+// 256 on whole 128-query blocks and on any length that is a whole number of 32-query tiles, as the software pipeline
+// of attention_pipe.h re-cut for one wavefront per SIMD.
 //
 // At this head dim a wavefront's O^T is 128 registers and its Q 64, so a workgroup is four wavefronts of 32 queries,
 // one per SIMD, each with the whole register file: O^T and Q live in AGPRs, scores and fragments in VGPRs, and every
@@ -87,7 +88,15 @@ __device__ __forceinline__ void mfma_o_copy(f32x16 &o, bf16x8 v, bf16x8 p, uint3
 // PREFETCHED, next_head, next_qblk: as in pipeattn::body (blocks 0, 1, 2 of this item are already in stages 0, 1, 2;
 // this item's trailing copies fetch the first key blocks of the next item; its Q is loaded before this item's
 // results are stored).
-template <bool PREFETCHED>
+//
+// RAGGED: N_CTX is a whole number of 32-query tiles but not of 128-query blocks.  Key blocks are 32 keys, so every
+// block of the sequence is whole and no key needs masking for the length's sake.  A wavefront whose tile lies past
+// the end computes and stores nothing but keeps up with the barriers and its share of the copies; an item's stream
+// of blocks is padded to a multiple of four periods (the padding refetches the item's last block into a stage that
+// nobody reads), so that the next item's first blocks land in stages 0, 1, 2 as they do for whole blocks; and an
+// item with fewer than three blocks has the others of its first three fetched from its last one.  Q is loaded when
+// the item starts.
+template <bool PREFETCHED, bool RAGGED = false>
 __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int head, const int qblk, const int next_head,
                                      const int next_qblk, Frag (&qf)[DK]) {
   const int tid = threadIdx.x, lane = tid & 63;
@@ -99,8 +108,13 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   const int my_q = qw + c32;
   const int64_t base = (int64_t)head * a.n_ctx;
   const float qk_scale = a.sm_scale * 1.44269504f;
-  const int nblk = a.causal ? (q0 + BM) / BN : a.n_ctx / BN;     // key blocks of this item
-  const int L = a.causal ? qw / BN : nblk - 1;                   // this wavefront's last block (the masked one when causal)
+  const bool live = !RAGGED || qw < a.n_ctx;                     // wave-uniform
+  const int nreal = (a.causal ? (RAGGED ? min(q0 + BM, a.n_ctx) : q0 + BM) : a.n_ctx) / BN;   // key blocks of this item
+  const int nblk = RAGGED ? (nreal + 3) & ~3 : nreal;            // periods the workgroup goes through (a multiple of 4)
+  const int L = a.causal ? qw / BN : nreal - 1;                  // this wavefront's last block (the masked one when causal)
+  // RAGGED: the real blocks of the item that follows (this item's own when none does)
+  const int next_q0 = (next_qblk >= 0 ? next_qblk : qblk) * BM;
+  const int next_nreal = RAGGED ? (a.causal ? min(next_q0 + BM, a.n_ctx) : a.n_ctx) / BN : 3;
 
   // ---- copies: 256 threads x 16 B = 4 KiB = 8 rows per instruction round, four rounds per K or V tile ----
   const int crow = tid / CH, cpos = tid % CH;
@@ -125,20 +139,34 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
                  : "memory", "m0");
   };
   const int64_t kstep = (int64_t)BN * a.ldk * 2, vstep = (int64_t)BN * a.ldv * 2;
+  // where period blk of this item's stream fetches from: its own block blk (RAGGED: the last real one for the padding
+  // periods and for an item of fewer than three blocks), past the stream the next item's first blocks (RAGGED: as
+  // many as that item has)
+  auto block_src = [&](int blk, const uint8_t *&kb, const uint8_t *&vb) __attribute__((always_inline)) {
+    const bool own = blk < nblk;
+    const int64_t b = own ? (RAGGED ? min(blk, nreal - 1) : blk) : (RAGGED ? min(blk - nblk, next_nreal - 1) : blk - nblk);
+    kb = (own ? kg : kg_next) + b * kstep;
+    vb = (own ? vg : vg_next) + b * vstep;
+  };
   // piece r (0-3: the four 8-row rounds of K; 4-7: of V) of block blk into the stage at byte offset stage_o
   auto dma_piece = [&](int blk, int stage_o, int r) __attribute__((always_inline)) {
-    const bool own = blk < nblk;
-    const int64_t b = own ? blk : blk - nblk;
-    if (r < 4) dma_one((own ? kg : kg_next) + b * kstep, k_voff[r], lds + stage_o + r * 4096);
-    else dma_one((own ? vg : vg_next) + b * vstep, v_voff[r - 4], lds + VBASE + stage_o + (r - 4) * 4096);
+    const uint8_t *kb, *vb;
+    block_src(blk, kb, vb);
+    if (r < 4) dma_one(kb, k_voff[r], lds + stage_o + r * 4096);
+    else dma_one(vb, v_voff[r - 4], lds + VBASE + stage_o + (r - 4) * 4096);
   };
   // the same from two running pointers (K and V rows of the block that is fetched next), stepped after the last piece
   // of a block and switched to the next item's keys when this item's run out
-  const uint8_t *kp = kg + 3 * kstep, *vp = vg + 3 * vstep;   // block 3: blocks 0..2 are the prologue's (or the item before's)
+  const uint8_t *kp, *vp;   // block 3 at first: blocks 0..2 are the prologue's (or the item before's)
+  block_src(3, kp, vp);
   auto dma_step = [&](int blk) __attribute__((always_inline)) {
-    const bool wrap = blk + 1 == nblk;
-    kp = wrap ? kg_next : kp + kstep;
-    vp = wrap ? vg_next : vp + vstep;
+    if constexpr (RAGGED) {
+      block_src(blk + 1, kp, vp);
+    } else {
+      const bool wrap = blk + 1 == nblk;
+      kp = wrap ? kg_next : kp + kstep;
+      vp = wrap ? vg_next : vp + vstep;
+    }
   };
   auto dma_run = [&](int blk, int stage_o, int r) __attribute__((always_inline)) {
     if (r < 4) dma_one(kp, k_voff[r], lds + stage_o + r * 4096);
@@ -183,7 +211,10 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
     for (int b = 0; b < 3; ++b)
 #pragma unroll
       for (int r = 0; r < 8; ++r) dma_piece(b, b * STG, r);
-    const uint16_t *qrow = a.q + (base + my_q) * a.ldq;
+  }
+  if constexpr (!PREFETCHED || RAGGED) {   // (otherwise the item before this one loaded them)
+    // (RAGGED: a wavefront past the end loads the last row that exists and never uses it)
+    const uint16_t *qrow = a.q + (base + (RAGGED ? min(my_q, a.n_ctx - 1) : my_q)) * a.ldq;
 #pragma unroll
     for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
   }
@@ -202,16 +233,18 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   asm volatile("" : "=v"(s0));
   asm volatile("" : "=v"(s1));
   asm volatile("" : "=v"(sb));
-#pragma unroll
-  for (int i = 0; i < DK; ++i) {
-    f32x16 &dst = (i & 1) ? sb : s0;
-    if (i < 2) mfma_s<true>(dst, rdK(lds, i), qf[i].v);
-    else mfma_s<false>(dst, rdK(lds, i), qf[i].v);
-  }
   bf16x8 kpre[GK], vpre[GV];   // first fragment group of the coming phase, requested during the phase before
+  if (live) {
 #pragma unroll
-  for (int i = 0; i < GK; ++i) kpre[i] = rdK(lds + STG, i);
-  P256_IDLE_V(sb);             // S^T(0) is read at once
+    for (int i = 0; i < DK; ++i) {
+      f32x16 &dst = (i & 1) ? sb : s0;
+      if (i < 2) mfma_s<true>(dst, rdK(lds, i), qf[i].v);
+      else mfma_s<false>(dst, rdK(lds, i), qf[i].v);
+    }
+#pragma unroll
+    for (int i = 0; i < GK; ++i) kpre[i] = rdK(lds + STG, i);
+    P256_IDLE_V(sb);             // S^T(0) is read at once
+  }
 
   // One block period of this wavefront.  LAST: no next block to start on; MASKED: the block on the diagonal.
   // cur_o, nxt_o, nn_o: byte offsets of the stages of blocks j, j+1, j+2; free_o: of the stage block j+3 goes into.
@@ -364,32 +397,35 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   int j = 0, cur_o = 0;
   auto nx = [&](int o) { return (o + STG) & (NST * STG - 1); };
   __builtin_amdgcn_s_setprio(3);
-  for (; j + 4 <= L; j += 4) {       // stage offsets known at compile time, score registers alternating
-    period(j, 0, STG, 2 * STG, 3 * STG, s0, s1, F, F);
-    period(j + 1, STG, 2 * STG, 3 * STG, 0, s1, s0, F, F);
-    period(j + 2, 2 * STG, 3 * STG, 0, STG, s0, s1, F, F);
-    period(j + 3, 3 * STG, 0, STG, 2 * STG, s1, s0, F, F);
-  }
-  // what is left (at most three blocks and the last one) runs with the stage offsets in registers
-  const int rest = L - j;
-  if (rest & 1) {
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
-    s0 = s1;
+  if (live) {
+    for (; j + 4 <= L; j += 4) {       // stage offsets known at compile time, score registers alternating
+      period(j, 0, STG, 2 * STG, 3 * STG, s0, s1, F, F);
+      period(j + 1, STG, 2 * STG, 3 * STG, 0, s1, s0, F, F);
+      period(j + 2, 2 * STG, 3 * STG, 0, STG, s0, s1, F, F);
+      period(j + 3, 3 * STG, 0, STG, 2 * STG, s1, s0, F, F);
+    }
+    // what is left (at most three blocks and the last one) runs with the stage offsets in registers
+    const int rest = L - j;
+    if (rest & 1) {
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
+      s0 = s1;
+      cur_o = nx(cur_o);
+      ++j;
+    }
+    if (rest & 2) {
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
+      cur_o = nx(cur_o);
+      ++j;
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s1, s0, F, F);
+      cur_o = nx(cur_o);
+      ++j;
+    }
+    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, T);
     cur_o = nx(cur_o);
     ++j;
   }
-  if (rest & 2) {
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
-    cur_o = nx(cur_o);
-    ++j;
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s1, s0, F, F);
-    cur_o = nx(cur_o);
-    ++j;
-  }
-  period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, T);
-  cur_o = nx(cur_o);
-  ++j;
-  // done: keep up with the others' barriers and this wavefront's share of the copies; cur_o is the stage of block j
+  // done (or, RAGGED, never started): keep up with the others' barriers and this wavefront's share of the copies;
+  // cur_o is the stage of block j
   for (; j < nblk; ++j) {
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
@@ -398,11 +434,14 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the trailing copies land before the stages are reused or released
   P256_IDLE_ACC(acc);                                // the last P.V MFMAs have written back before the accumulators are read
-  if (next_qblk >= 0) {   // the next item's Q, on its way while this item's results are stored
-    const uint16_t *qrow = a.q + ((int64_t)next_head * a.n_ctx + next_qblk * BM + wave * 32 + c32) * a.ldq;
+  if constexpr (!RAGGED) {
+    if (next_qblk >= 0) {   // the next item's Q, on its way while this item's results are stored
+      const uint16_t *qrow = a.q + ((int64_t)next_head * a.n_ctx + next_qblk * BM + wave * 32 + c32) * a.ldq;
 #pragma unroll
-    for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+      for (int s = 0; s < DK; ++s) qf[s].u = *(const u16x8 *)(qrow + s * 16 + hi * 8);
+    }
   }
+  if (!live) return;
   // ---- epilogue ----
   if (hi == 0) a.m[base + my_q] = m_i + __builtin_log2f(l_i);
   uint16_t *orow = a.o + (base + my_q) * a.ldo;
@@ -428,8 +467,8 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 
 // Persistent, as attn_pipe: gridDim.x workgroups walk the (head, pair of query blocks) items in the order the
 // dispatcher would have dealt one-item workgroups, a workgroup's items back to back.
-__device__ __forceinline__ void attn_pipe256(const AttnArgs &a, uint8_t *lds) {
-  const int qblocks = a.rows / pipe256::BM;
+template <bool RAGGED> __device__ __forceinline__ void attn_pipe256(const AttnArgs &a, uint8_t *lds) {
+  const int qblocks = RAGGED ? (a.rows + pipe256::BM - 1) / pipe256::BM : a.rows / pipe256::BM;
   const int per_head = (qblocks + 1) / 2, total = per_head * a.heads;
   auto decode = [&](int n, int &head, int &p) {
     int id = n;
@@ -455,13 +494,13 @@ __device__ __forceinline__ void attn_pipe256(const AttnArgs &a, uint8_t *lds) {
   int n2 = n, head2 = head, p2 = p, which2 = which;
   bool more = advance(n2, head2, p2, which2);
   pipeattn::Frag qf[pipe256::DK];   // Q fragments of the running item; its end refills them for the next
-  pipe256::body<false>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head,
+  pipe256::body<false, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head,
                        more ? (which2 ? p2 : qblocks - 1 - p2) : -1, qf);
   asm volatile("s_barrier" ::: "memory");   // nobody reads this item's stages any more; the next item's first blocks have landed
   while (more) {
     n = n2; head = head2; p = p2; which = which2;
     more = advance(n2, head2, p2, which2);
-    pipe256::body<true>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head,
+    pipe256::body<true, RAGGED>(a, lds, head, which ? p : qblocks - 1 - p, more ? head2 : head,
                         more ? (which2 ? p2 : qblocks - 1 - p2) : -1, qf);
     asm volatile("s_barrier" ::: "memory");
   }
@@ -471,7 +510,13 @@ extern "C" {
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_tile_d256(AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[pipe256::NST * 2 * pipe256::TILE];
-  attn_pipe256(a, lds);
+  attn_pipe256<false>(a, lds);
+}
+
+// the same for sequence lengths that are whole 32-query tiles but not whole 128-query blocks
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void attn_ragged_d256(AttnArgs a) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[pipe256::NST * 2 * pipe256::TILE];
+  attn_pipe256<true>(a, lds);
 }
 
 } // extern "C"
