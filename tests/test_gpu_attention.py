@@ -251,7 +251,8 @@ def test_causal_mask_is_the_sources_at_block_m_32(S, D, kernel):
 @pytest.mark.parametrize("Z,H,S,D", [(2, 32, 2304, 128), (1, 40, 3328, 128), (3, 3, 768, 128), (2, 32, 2272, 128),
                                      (1, 33, 4000, 128), (5, 8, 1056, 128), (2, 32, 2304, 64), (3, 11, 3328, 64), (1, 5, 512, 64),
                                      (2, 32, 1152, 256), (1, 40, 1664, 256), (3, 3, 384, 256), (1, 5, 128, 256),
-                                     (2, 32, 1056, 256), (1, 33, 2016, 256), (5, 8, 544, 256), (1, 3, 32, 256), (2, 3, 96, 256)])
+                                     (2, 32, 1056, 256), (1, 33, 2016, 256), (5, 8, 544, 256), (1, 3, 32, 256), (2, 3, 96, 256),
+                                     (2, 32, 2272, 64), (1, 33, 4000, 64), (5, 8, 1056, 64), (1, 3, 32, 64), (2, 3, 96, 64), (1, 2, 224, 64)])
 def test_items_chained_inside_a_workgroup(causal, Z, H, S, D):
     """The head dim 128, 64 and 256 kernels walk (head, pair of query blocks) items on a persistent grid (256-query blocks;
     128-query blocks at head dim 256) and let each item's last

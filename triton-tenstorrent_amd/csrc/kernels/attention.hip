@@ -533,7 +533,7 @@ ATTN_TILE(32)
     fastattn::body<D, true>(a, lds0, lds1);                                                \
   }
 ATTN_RAGGED(32)
-ATTN_RAGGED(64)
+// (head dim 64: attn_ragged_d64 in attention_pipe.h)
 
 // head dim 256: four wavefronts, 128 queries per workgroup
 #define ATTN_TILE4(name, D, RAGGED)                                                        \

@@ -96,7 +96,7 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   constexpr int PPT = BN / RPP;                // such pieces per K or V tile
   constexpr int SLOTS = D / 8;                 // MFMAs per phase: 2*DK = 4*DT
   constexpr int SPS = 16 / SLOTS;              // softmax work items per MFMA slot
-  static_assert(D == 128 || (D == 64 && !RAGGED), "LDS swizzles exist for 256- and 128-byte rows; ragged lengths at 256 only");
+  static_assert(D == 128 || D == 64, "LDS swizzles exist for 256- and 128-byte rows");
   static_assert((NST & (NST - 1)) == 0, "the stage ring wraps with a mask");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -123,6 +123,9 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   const int v_chunk = cpos ^ ((D == 128 ? (crow & 3) : ((crow >> 1) & 1)) << 2);   // V: at c ^ ((r & 3) << 2), 128-byte rows: c ^ (((r >> 1) & 1) << 2)
   const uint32_t k_voff = (uint32_t)(((int64_t)crow * a.ldk + k_chunk * 8) * 2);
   const uint32_t v_voff = (uint32_t)(((int64_t)crow * a.ldv + v_chunk * 8) * 2);
+  // (RAGGED at 128-byte rows: the same with rows 32-63 of a tile fetched from rows 0-31, for a half block at the end)
+  const uint32_t k_voff_half = (uint32_t)(((int64_t)(crow & 31) * a.ldk + k_chunk * 8) * 2);
+  const uint32_t v_voff_half = (uint32_t)(((int64_t)(crow & 31) * a.ldv + v_chunk * 8) * 2);
   const uint8_t *kg = (const uint8_t *)(a.k + base * a.ldk);
   const uint8_t *vg = (const uint8_t *)(a.v + base * a.ldv);
   const uint8_t *kg_next = (const uint8_t *)(a.k + (int64_t)next_head * a.n_ctx * a.ldk);
@@ -143,9 +146,21 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
     // (RAGGED: periods nblk .. nstream-1 are padding and refetch the last block; any 32 rows that do not exist are
     // fetched from the last 32 that do)
     int64_t row0 = (int64_t)(own ? (RAGGED ? min(blk, nblk - 1) : blk) : blk - nstream) * BN + (r % PPT) * RPP;
-    if (RAGGED) row0 = min(row0, (int64_t)last_rows);
-    if (r < PPT) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, k_voff, lds + stage_o + (r % PPT) * 8192);
-    else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, v_voff, lds + VBASE + stage_o + (r % PPT) * 8192);
+    uint32_t kvo = k_voff, vvo = v_voff;
+    if constexpr (RAGGED && RPP == 64) {
+      // (128-byte rows: one copy instruction is a whole 64-row tile.  A block at or past the end is fetched from the
+      // last one that starts inside the sequence, and where that one is a half block its threads of rows 32-63
+      // fetch rows 0-31 again)
+      row0 = min(row0, (int64_t)((a.n_ctx - 1) / 64) * 64);
+      if (row0 + 64 > a.n_ctx) {
+        kvo = k_voff_half;
+        vvo = v_voff_half;
+      }
+    } else if (RAGGED) {
+      row0 = min(row0, (int64_t)last_rows);
+    }
+    if (r < PPT) dma_one((own ? kg : kg_next) + row0 * a.ldk * 2, kvo, lds + stage_o + (r % PPT) * 8192);
+    else dma_one((own ? vg : vg_next) + row0 * a.ldv * 2, vvo, lds + VBASE + stage_o + (r % PPT) * 8192);
   };
   // The same for whole blocks only, from two running pointers (K and V rows of the block that is fetched next) instead
   // of a 64-bit product per piece: the pieces of a block are issued in order and the pointers step after the last one,
@@ -510,6 +525,12 @@ __global__ __launch_bounds__(512) void attn_ragged_d128(AttnArgs a) {
 __global__ __launch_bounds__(512) void attn_tile_d64(AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 64 * 2];
   attn_pipe<64, false>(a, lds);
+}
+
+// and for lengths that are whole 32-query tiles but not whole 256-query blocks
+__global__ __launch_bounds__(512) void attn_ragged_d64(AttnArgs a) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[pipeattn::NST * 2 * 64 * 64 * 2];
+  attn_pipe<64, true>(a, lds);
 }
 
 } // extern "C"

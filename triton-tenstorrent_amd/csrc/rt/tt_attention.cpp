@@ -71,10 +71,10 @@ extern "C" int tt_attn_fwd(float sm_scale, float *M, int32_t Z, int32_t H, const
     void *fargs[] = {&a};
     const int queries = HEAD_DIM == 256 ? 128 : 256;   // per workgroup: 4 or 8 wavefronts of 32
     uint32_t wgs = (uint32_t)(cdiv64(N_CTX, queries) * (int64_t)Z * H);
-    // head dims 128 and 256, and head dim 64 on whole blocks: an item is the pair of query blocks i and n-1-i of a head, and
+    // head dims 64, 128 and 256: an item is the pair of query blocks i and n-1-i of a head, and
     // the grid is persistent: one workgroup per CU walks its share of the items back to back (fewer workgroups when
     // there are fewer items)
-    if (HEAD_DIM == 128 || HEAD_DIM == 256 || (HEAD_DIM == 64 && N_CTX % queries == 0)) {
+    if (HEAD_DIM != 32) {
       const int64_t items = cdiv64(cdiv64(N_CTX, queries), 2) * (int64_t)Z * H;
       wgs = (uint32_t)std::min<int64_t>(items, props()->multiprocessor_count);
     }
