@@ -229,8 +229,8 @@ constexpr int BN = 64;
 // the last key block may hold 32 keys only: its copies fetch the rows past N_CTX from the last row instead, the
 // second 32-key tile is left out of both products and its scores count as -inf.
 //
-// WAVES = 4 (head dim 256): 128 queries per workgroup, one wavefront per SIMD with the whole register file
-// (O^T alone is 128 registers and Q 64 at that head dim), and all four wavefronts share the copies.
+// WAVES = 4: 128 queries per workgroup, one wavefront per SIMD with the whole register file, all four wavefronts
+// sharing the copies (how head dim 256 ran before attention_pipe256.h; no kernel instantiates it now).
 // Issue priority of a wavefront over a block: 3 through the two MFMA phases, 1 through the softmax, 2 at the end of
 // the block, never the default 0.  Measured A/B in one process (causal / not causal TFLOP/s): head dim 256 (one
 // wavefront per SIMD) 575 -> 667 / 658 -> 766, and a constant priority of 3 does the same there, so what counts is
@@ -535,13 +535,6 @@ ATTN_TILE(32)
 ATTN_RAGGED(32)
 // (head dim 64: attn_ragged_d64 in attention_pipe.h)
 
-// head dim 256: four wavefronts, 128 queries per workgroup
-#define ATTN_TILE4(name, D, RAGGED)                                                        \
-  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(AttnArgs a) { \
-    __shared__ __attribute__((aligned(1024))) uint8_t lds0[2 * 64 * D * 2];                \
-    __shared__ __attribute__((aligned(1024))) uint8_t lds1[2 * 64 * D * 2];                \
-    fastattn::body<D, RAGGED, 4>(a, lds0, lds1);                                           \
-  }
 // (head dim 256: attn_tile_d256 and attn_ragged_d256 in attention_pipe256.h)
 
 } // extern "C"
