@@ -312,6 +312,33 @@ def test_row_maxima_that_climb_slowly_and_in_jumps(causal, S, D, kernel):
         assert (M[0, h].double() - torch.logsumexp(s_, -1) / np.log(2.0)).abs().max() <= M_ATOL
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Z,H,S,sm", [(3, 2, 1216, 0.125), (2, 4, 1184, 0.0625), (1, 6, 160, 0.125), (2, 3, 1152, 0.125)])
+def test_the_wavefront_that_ends_an_item_reads_finished_accumulators(causal, Z, H, S, sm):
+    """Head dim 256.  The last wavefront of a full 128-query block runs its last block period and goes straight to
+    the epilogue, with no idle period in between; in the other periods outside the main loop (a number of key blocks
+    that is not a multiple of four leaves up to three) the compiler may move accumulator tiles between register
+    sets.  Wherever such a read follows the MFMA that writes the tile, the MFMA carries its wait states itself.
+    A length with nine full blocks and a part (every block but the last is full while the launch takes the ragged
+    kernel), one more ragged length, a short one and a whole one: every row of every head against float64, and three
+    launches on the same operands give the same bits."""
+    from triton_tenstorrent_amd import runtime as rt
+    g = torch.Generator(device="cuda").manual_seed(S + Z)
+    q, k, v = (torch.randn(Z, H, S, 256, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+    o, M = K.attention(q, k, v, causal, sm, return_lse=True)
+    assert rt.last_kernel_name() == ("attn_tile_d256" if S % 128 == 0 else "attn_ragged_d256")
+    for _ in range(2):
+        o2, M2 = K.attention(q, k, v, causal, sm, return_lse=True)
+        assert torch.equal(o2, o) and torch.equal(M2, M)
+    s = (q.double() @ k.double().transpose(-1, -2)) * sm
+    if causal:
+        rows = torch.arange(S, device="cuda")
+        s = s.masked_fill(rows[:, None] < rows[None, :], float("-inf"))
+    ref = torch.softmax(s, -1) @ v.double()
+    assert (o.double() - ref).abs().max() <= O_ATOL
+    assert (M.double() - torch.logsumexp(s, -1) / np.log(2.0)).abs().max() <= M_ATOL
+
+
 def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
     """From the second call of a shape on, `_attn_fwd` is launched through a cached closure (N_CTX and the block
     sizes arrive by keyword and are part of what makes two calls alike).  Batch, heads, operands and the mask may

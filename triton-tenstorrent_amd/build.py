@@ -11,6 +11,7 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
@@ -38,8 +39,8 @@ def hipcc() -> str:
     return exe
 
 
-def _run(cmd: list[str]) -> None:
-    r = subprocess.run(cmd, capture_output=True, text=True)
+def _run(cmd: list[str], cwd: str | None = None) -> None:
+    r = subprocess.run(cmd, capture_output=True, text=True, cwd=cwd)
     if r.returncode != 0:
         sys.stderr.write(" ".join(cmd) + "\n" + r.stdout + r.stderr)
         raise RuntimeError(f"build step failed: {cmd[0]} ... {cmd[-1]}")
@@ -49,9 +50,23 @@ def _run(cmd: list[str]) -> None:
 
 
 def build_code_object(name: str, extra: list[str] | None = None) -> Path:
+    """Compile kernels/<name>.hip and check the assembly listing of that same compilation (kept with -save-temps
+    in a directory of its own, deleted afterwards) for reads of an MFMA result that the compiler placed too close
+    behind an inline-assembly MFMA: see listing_check."""
+    from . import listing_check
     BUILD.mkdir(exist_ok=True)
     out = BUILD / f"{name}.hsaco"
-    _run([hipcc(), "--genco", *DEVICE_FLAGS, *(extra or []), str(CSRC / "kernels" / f"{name}.hip"), "-o", str(out)])
+    with tempfile.TemporaryDirectory(prefix=f"ttamd_{name}_") as tmp:
+        _run([hipcc(), "--genco", *DEVICE_FLAGS, "-save-temps", *(extra or []), str(CSRC / "kernels" / f"{name}.hip"),
+              "-o", str(out)], cwd=tmp)
+        listings = list(Path(tmp).glob(f"{name}-hip-amdgcn-*{ARCH}.s"))
+        if len(listings) != 1:
+            raise RuntimeError(f"{name}: expected one {ARCH} listing from -save-temps, found {len(listings)}")
+        bad = listing_check.check_listing(listings[0].read_text())
+    if bad:
+        out.unlink()
+        lines = [f"{k}: {len(v)} (first: {v[0]})" for k, v in bad.items()]
+        raise RuntimeError(f"{name}.hip: an MFMA result is touched too early in\n  " + "\n  ".join(lines))
     return out
 
 

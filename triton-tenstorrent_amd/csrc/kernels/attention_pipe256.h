@@ -71,18 +71,37 @@ template <bool ZERO> __device__ __forceinline__ void mfma_s(f32x16 &s, bf16x8 k,
   else
     asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(k), "a"(q));
 }
+// Idle states behind an MFMA, inside its statement, for the places where the compiler may put code of its own that
+// reads the result right behind the statement: it does not know that the statement holds an MFMA and leaves none of
+// the wait states that a read of an MFMA's result needs (eleven for this MFMA).  Two kinds of such places exist.  In
+// the periods outside the main loop (the up to three left over and the last one of an item) the register allocator
+// may move each 16-register accumulator tile to VGPRs directly behind the MFMA that writes it last, as it did in the
+// ragged kernel.  And where control flow joins behind a period, it copies accumulator registers between the
+// register sets the paths use.  Without the idle states such copies hold what the tile held before the MFMA: wrong
+// output values in some d-tiles of some rows, with the right M.
+#define P256_TAIL "\n\ts_nop 7\n\ts_nop 7"
 // O^T += V^T . P^T: accumulators in AGPRs
-__device__ __forceinline__ void mfma_o(f32x16 &o, bf16x8 v, bf16x8 p) {
-  asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(o) : "v"(v), "v"(p));
+template <bool TAIL> __device__ __forceinline__ void mfma_o(f32x16 &o, bf16x8 v, bf16x8 p) {
+  if constexpr (TAIL)
+    asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" P256_TAIL : "+a"(o) : "v"(v), "v"(p));
+  else
+    asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(o) : "v"(v), "v"(p));
 }
 
 // the same with one direct-to-LDS copy behind it (m0, its LDS destination, is written by the compiler in front of
 // the statement: the MFMA is the wait state that the copy needs after a write to m0)
+template <bool TAIL>
 __device__ __forceinline__ void mfma_o_copy(f32x16 &o, bf16x8 v, bf16x8 p, uint32_t m0v, uint32_t voff, const uint8_t *src) {
-  asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
-               : "+a"(o)
-               : "v"(v), "v"(p), "{m0}"(m0v), "v"(voff), "s"(src)
-               : "memory");
+  if constexpr (TAIL)
+    asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5" P256_TAIL
+                 : "+a"(o)
+                 : "v"(v), "v"(p), "{m0}"(m0v), "v"(voff), "s"(src)
+                 : "memory");
+  else
+    asm volatile(P256_PAD "v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tglobal_load_lds_dwordx4 %4, %5"
+                 : "+a"(o)
+                 : "v"(v), "v"(p), "{m0}"(m0v), "v"(voff), "s"(src)
+                 : "memory");
 }
 
 // PREFETCHED, next_head, next_qblk: as in pipeattn::body (blocks 0, 1, 2 of this item are already in stages 0, 1, 2;
@@ -249,9 +268,13 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
   // One block period of this wavefront.  LAST: no next block to start on; MASKED: the block on the diagonal.
   // cur_o, nxt_o, nn_o: byte offsets of the stages of blocks j, j+1, j+2; free_o: of the stage block j+3 goes into.
   // sc holds S^T(j) on entry, sn receives S^T(j+1).
+  // tail_: 0 in the main loop; 1: the period may be followed by something else than the next period (its last MFMA
+  // leaves idle states); 2: a period outside the main loop (every P.V MFMA leaves them): see P256_TAIL
   auto period = [&](int j, int cur_o, int nxt_o, int nn_o, int free_o, f32x16 &sc, f32x16 &sn, auto last_,
-                    auto masked_) __attribute__((always_inline)) {
+                    auto masked_, auto tail_) __attribute__((always_inline)) {
     constexpr bool LAST = decltype(last_)::value, MASKED = decltype(masked_)::value;
+    constexpr int TAIL = decltype(tail_)::value;
+    static_assert(!LAST || TAIL == 2, "");
     const uint8_t *cur = lds + cur_o, *nxt = lds + nxt_o;
     bf16x8 kf[2 * GK], vf[2 * GV];
     float rmax0 = -__builtin_inff(), rmax1 = -__builtin_inff(), m_ij, alpha, l_ij = 0.0f;
@@ -373,10 +396,13 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
       if (i % 2 == 1) {
         const int r = i / 2;
         const uint32_t m0v = (uint32_t)(uintptr_t)(lds_void *)(lds + (r < 4 ? 0 : VBASE) + free_o + (r & 3) * 4096 + lds_wave);
-        mfma_o_copy(acc[t], vf[i % (2 * GV)], pf[k4].v, m0v, r < 4 ? k_voff[r] : v_voff[r - 4], r < 4 ? kp : vp);
+        if (TAIL == 2 || (TAIL == 1 && i == 2 * DT - 1))
+          mfma_o_copy<true>(acc[t], vf[i % (2 * GV)], pf[k4].v, m0v, r < 4 ? k_voff[r] : v_voff[r - 4], r < 4 ? kp : vp);
+        else
+          mfma_o_copy<false>(acc[t], vf[i % (2 * GV)], pf[k4].v, m0v, r < 4 ? k_voff[r] : v_voff[r - 4], r < 4 ? kp : vp);
         if (r == 7) dma_step(j + 3);
       } else {
-        mfma_o(acc[t], vf[i % (2 * GV)], pf[k4].v);
+        mfma_o<TAIL == 2>(acc[t], vf[i % (2 * GV)], pf[k4].v);
       }
       if (!LAST && i == 2 * DT - 4) {
 #pragma unroll
@@ -394,33 +420,36 @@ __device__ __forceinline__ void body(const AttnArgs &a, uint8_t *lds, const int 
 
   const std::false_type F{};
   const std::true_type T{};
+  const std::integral_constant<int, 0> T0{};
+  const std::integral_constant<int, 1> T1{};
+  const std::integral_constant<int, 2> T2{};
   int j = 0, cur_o = 0;
   auto nx = [&](int o) { return (o + STG) & (NST * STG - 1); };
   __builtin_amdgcn_s_setprio(3);
   if (live) {
     for (; j + 4 <= L; j += 4) {       // stage offsets known at compile time, score registers alternating
-      period(j, 0, STG, 2 * STG, 3 * STG, s0, s1, F, F);
-      period(j + 1, STG, 2 * STG, 3 * STG, 0, s1, s0, F, F);
-      period(j + 2, 2 * STG, 3 * STG, 0, STG, s0, s1, F, F);
-      period(j + 3, 3 * STG, 0, STG, 2 * STG, s1, s0, F, F);
+      period(j, 0, STG, 2 * STG, 3 * STG, s0, s1, F, F, T0);
+      period(j + 1, STG, 2 * STG, 3 * STG, 0, s1, s0, F, F, T0);
+      period(j + 2, 2 * STG, 3 * STG, 0, STG, s0, s1, F, F, T0);
+      period(j + 3, 3 * STG, 0, STG, 2 * STG, s1, s0, F, F, T1);
     }
     // what is left (at most three blocks and the last one) runs with the stage offsets in registers
     const int rest = L - j;
     if (rest & 1) {
-      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F, T2);
       s0 = s1;
       cur_o = nx(cur_o);
       ++j;
     }
     if (rest & 2) {
-      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F);
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, F, F, T2);
       cur_o = nx(cur_o);
       ++j;
-      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s1, s0, F, F);
+      period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s1, s0, F, F, T2);
       cur_o = nx(cur_o);
       ++j;
     }
-    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, T);
+    period(j, cur_o, nx(cur_o), nx(nx(cur_o)), nx(nx(nx(cur_o))), s0, s1, T, T, T2);
     cur_o = nx(cur_o);
     ++j;
   }
