@@ -252,8 +252,9 @@ typedef enum tt_reduce_op {
 TTAMD_API int tt_reduce1d_kernel(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype,
                        int32_t acc_dtype, int32_t out_dtype, int32_t propagate_nan,
                        const uint32_t grid[3], void *stream);
-/* Frees what the library allocated for `stream` on the current device (the buffer above), after waiting for the
- * stream; call it before destroying a stream that ran large reductions.  No counterpart in the reference. */
+/* Frees what the library allocated for `stream` on the current device (the buffer above and the workspace of
+ * tt_matmul_kernel_tma / _fused, below), after waiting for the stream; call it before destroying a stream that ran
+ * large reductions or matmuls of few tiles.  No counterpart in the reference. */
 TTAMD_API int rt_release_stream(void *stream);
 /* The same reductions, same arguments and results, for callers that cannot allocate device memory: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
@@ -273,7 +274,13 @@ TTAMD_API int tt_reduce1d_kernel_noalloc(int32_t op, const void *x, void *z, int
  * examples/matmul_tensor_descriptor/09-persistent-matmul.py:102-145.
  * A [M,K] and B [K,N] (not transposed) row-major, fp32 accumulate, one
  * round-to-nearest-even cast to c->dtype.  grid[0] logical programs, one per
- * BLOCK_SIZE_M x BLOCK_SIZE_N tile in GROUP_SIZE_M-swizzled order. */
+ * BLOCK_SIZE_M x BLOCK_SIZE_N tile in GROUP_SIZE_M-swizzled order.
+ * A 16-bit launch (this entry point and _fused) whose C has few 256x256 tiles under a long K (at most half the CUs
+ * busy even with 64-row pieces of tiles, K a multiple of 256) is computed in slices of K: the slices' fp32 sums pass
+ * through a workspace of at most 64 MiB that the library keeps per (device, stream), allocated by the first such
+ * call on the stream (hipMalloc), grown by a call that needs more (the stream is drained first) and freed by
+ * rt_release_stream; the sums are added in slice order, so results do not change from launch to launch, and the
+ * epilogue is applied to the whole sum.  A call on a stream that is recording a graph never takes that route. */
 TTAMD_API int tt_matmul_kernel_tma(const tt_desc2d *a, const tt_desc2d *b, const tt_desc2d *c,
                          int32_t M, int32_t N, int32_t K, int32_t BLOCK_SIZE_M,
                          int32_t BLOCK_SIZE_N, int32_t BLOCK_SIZE_K, int32_t GROUP_SIZE_M,

@@ -1,6 +1,8 @@
 """GPU parity: the tile-matmul family through the launcher and the C ABI against the CPU
 oracle.  Tolerance (bf16/fp16/fp8 inputs, fp32 accumulate): abs(err) <= 1e-2*abs(ref) + 1e-4
 against the fp64-accumulated oracle, and PCC >= 0.9999 (the reference's bar is 0.97)."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -314,8 +316,113 @@ def test_matmul_errors():
 def test_fast_path_matches_oracle(M, N, K_, dtype):
     a, b = _ab(M, N, K_, dtype, seed=M + N + K_)
     c = K.matmul_tma(a.cuda(), b.cuda())
-    assert rt.last_kernel_name().startswith("gemm_tile_"), rt.last_kernel_name()
+    # (four tiles under K = 2048: the launch that is finished in slices of K)
+    assert rt.last_kernel_name().startswith("gemm_splitk_reduce_" if K_ == 2048 else "gemm_tile_"), rt.last_kernel_name()
     _check(c, a, b)
+
+
+# ---- few tiles under a long K: slices of K as work items, fp32 sums through a workspace -------------------------
+@pytest.mark.parametrize("M,N,K_", [(64, 256, 2048), (1, 512, 4096), (200, 520, 2048), (256, 256, 4096), (300, 264, 3072),
+                                    (130, 1024, 8192), (700, 256, 2560)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_k_slices_match_oracle(M, N, K_, dtype):
+    """Shapes of one to twelve macro tiles with K a multiple of 256: matrices of one row of tiles with 1, 64, 130, 200
+    and 256 live rows (one to four live quarters per tile), two and three rows of tiles, N not a whole tile.  The
+    result is the fp32 sum over all of K rounded once, as without slices, so the same bounds hold; two launches give
+    the same bits (the slabs are added in slice order)."""
+    a, b = _ab(M, N, K_, dtype, seed=M + N + K_)
+    c = K.matmul_tma(a.cuda(), b.cuda())
+    assert rt.last_kernel_name() == ("gemm_splitk_reduce_bf16" if dtype == torch.bfloat16 else "gemm_splitk_reduce_f16")
+    _check(c, a, b)
+    assert torch.equal(K.matmul_tma(a.cuda(), b.cuda()), c)
+
+
+def test_k_slices_small_integers_bit_exact_and_output_strides():
+    g = torch.Generator().manual_seed(5)
+    M, N, K_ = 190, 520, 4096
+    a = torch.randint(-4, 5, (M, K_), generator=g).to(torch.bfloat16)
+    b = torch.randint(-4, 5, (K_, N), generator=g).to(torch.bfloat16)
+    cbuf = torch.full((M + 3, N + 24), 7.5, dtype=torch.bfloat16, device="cuda")
+    c = cbuf[:M, :N]
+    from triton_tenstorrent_amd.tensor_descriptor import TensorDescriptor as TD
+    ad, bd, cd = TD.from_tensor(a.cuda(), [128, 64]), TD.from_tensor(b.cuda(), [64, 128]), TD.from_tensor(c, [128, 128])
+    K.matmul_kernel_tma[(2 * 5, )](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False, BLOCK_SIZE_M=128,
+                                   BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, GROUP_SIZE_M=8)
+    assert rt.last_kernel_name() == "gemm_splitk_reduce_bf16"
+    assert np.array_equal(bits(c), orc.matmul(bits(a), bits(b), BM=64, BN=64, BK=64))
+    # nothing outside the [M, N] window of the output buffer was written
+    assert torch.all(cbuf[M:, :] == 7.5) and torch.all(cbuf[:, N:] == 7.5)
+
+
+@pytest.mark.parametrize("epilogue", [None, "gelu", "bias_row", "leaky_relu"])
+def test_k_slices_epilogues(epilogue):
+    """The epilogue is applied by the kernel that adds the slabs, on the whole sum: same results as in one pass."""
+    M, N, K_ = 100, 520, 4096
+    a, b = _ab(M, N, K_, seed=31)
+    gen = torch.Generator().manual_seed(32)
+    if epilogue is None:
+        bias = torch.randn(M, N, generator=gen).to(torch.bfloat16)
+        okw = dict(bias=bits(bias), epi=orc.EPI_BIAS_FULL)
+    else:
+        bias = torch.randn(N, generator=gen) * 0.02
+        okw = dict(bias=bias.numpy(), epi={"gelu": orc.EPI_BIAS_ROW_GELU, "bias_row": orc.EPI_BIAS_ROW,
+                                          "leaky_relu": orc.EPI_LEAKY_RELU}[epilogue])
+        if epilogue == "leaky_relu":
+            okw.pop("bias")
+    c = K.matmul_fused(a.cuda(), b.cuda(), bias.cuda(), epilogue=epilogue)
+    assert rt.last_kernel_name() == "gemm_splitk_reduce_bf16"
+    ref = orc.from_bf16(orc.matmul(bits(a), bits(b), acc64=True, **okw))
+    assert close_bf16(decode(c), ref, RTOL, 1e-2 if epilogue is None else ATOL)
+
+
+def test_k_slices_workspace_per_stream_growth_release_and_graphs():
+    """The workspace belongs to a (device, stream) pair: launches on two streams do not share one, a launch that
+    needs more than the stream's has grows it, rt_release_stream gives it back (and the next launch takes a new
+    one), and a launch that is being recorded into a graph runs in one pass and holds no address of the library's."""
+    shapes = [(64, 256, 2048), (200, 1024, 4096), (64, 256, 2048)]      # small, larger, small again
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    data = [[_ab(M, N, K_, seed=7 * i + j) for j, (M, N, K_) in enumerate(shapes)] for i in range(2)]
+    dev = [[(a.cuda(), b.cuda()) for a, b in row] for row in data]
+    torch.cuda.synchronize()
+    out = [[None] * len(shapes) for _ in range(2)]
+    for j in range(len(shapes)):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                out[i][j] = K.matmul_tma(*dev[i][j])
+                assert rt.last_kernel_name() == "gemm_splitk_reduce_bf16"
+    torch.cuda.synchronize()
+    for i in range(2):
+        for j in range(len(shapes)):
+            _check(out[i][j], *data[i][j])
+    for st in streams:
+        assert rt.load().rt_release_stream(C.c_void_p(st.cuda_stream)) == rt.RT_OK
+    with torch.cuda.stream(streams[0]):
+        c = K.matmul_tma(*dev[0][1])
+    streams[0].synchronize()
+    assert torch.equal(c, out[0][1])
+    assert rt.load().rt_release_stream(C.c_void_p(streams[0].cuda_stream)) == rt.RT_OK
+    # under capture: one pass, same bounds; replays agree with each other
+    a, b = dev[1][1]
+    cg = torch.empty(a.shape[0], b.shape[1], dtype=torch.bfloat16, device="cuda")
+    ad, bd, cd = (TensorDescriptor.from_tensor(t, blk) for t, blk in ((a, [128, 64]), (b, [64, 128]), (cg, [128, 128])))
+    M, K_ = a.shape
+    N = b.shape[1]
+    grid = ((M + 127) // 128 * ((N + 127) // 128), )
+    st = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        K.matmul_kernel_tma[grid](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False, BLOCK_SIZE_M=128,
+                                  BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, GROUP_SIZE_M=8)      # warm: modules loaded
+        st.synchronize()
+        with torch.cuda.graph(graph, stream=st):
+            K.matmul_kernel_tma[grid](ad, bd, cd, M, N, K_, FP8_OUTPUT=False, WARP_SPECIALIZE=False, BLOCK_SIZE_M=128,
+                                      BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, GROUP_SIZE_M=8)
+            assert rt.last_kernel_name() == "gemm_ragged_bf16_epi0"
+    for _ in range(3):
+        cg.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        _check(cg, *data[1][1])
 
 
 def test_fast_path_small_integers_bit_exact():

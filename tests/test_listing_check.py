@@ -57,3 +57,12 @@ def test_the_window_follows_the_passes_of_the_form():
 def test_kernels_of_a_listing_are_checked_one_by_one():
     text = "\n".join(kernel(MFMA, "\tv_accvgpr_read_b32 v1, a0") + ["clean:", MFMA, "\ts_endpgm", ".Lfunc_end1:"])
     assert list(lc.check_listing(text)) == ["k"]
+
+
+def test_compiler_waits_for_memory_inside_an_mfma_loop_are_counted():
+    loop = [".LBB0_1:"] + [MFMA] * 32
+    asm_wait = ["\t;;#ASMSTART", "\ts_waitcnt vmcnt(16) lgkmcnt(0)", "\t;;#ASMEND"]
+    assert lc.vmcnt_waits_in_mfma_blocks(kernel(*loop, *asm_wait)) == 0
+    assert lc.vmcnt_waits_in_mfma_blocks(kernel(*loop, *asm_wait, "\ts_waitcnt vmcnt(0)")) == 1
+    # outside the loops (a block with few MFMAs) the compiler may wait as it likes
+    assert lc.vmcnt_waits_in_mfma_blocks(kernel(*loop, ".LBB0_2:", MFMA, "\ts_waitcnt vmcnt(0)")) == 0

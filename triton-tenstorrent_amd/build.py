@@ -62,7 +62,13 @@ def build_code_object(name: str, extra: list[str] | None = None) -> Path:
         listings = list(Path(tmp).glob(f"{name}-hip-amdgcn-*{ARCH}.s"))
         if len(listings) != 1:
             raise RuntimeError(f"{name}: expected one {ARCH} listing from -save-temps, found {len(listings)}")
-        bad = listing_check.check_listing(listings[0].read_text())
+        text = listings[0].read_text()
+        bad = listing_check.check_listing(text)
+        # not an error, but worth a line: the hand-scheduled K loops should hold no wait of the compiler's for memory
+        for kernel, lines in listing_check.split_kernels(text).items():
+            n = listing_check.vmcnt_waits_in_mfma_blocks(lines) if kernel.startswith(("gemm_tile", "gemm_ragged", "gemm_splitk_b", "gemm_splitk_f")) else 0
+            if n:
+                sys.stderr.write(f"[build] {kernel}: {n} compiler-placed vmcnt wait(s) inside an MFMA loop (a spill in the K loop?)\n")
     if bad:
         out.unlink()
         lines = [f"{k}: {len(v)} (first: {v[0]})" for k, v in bad.items()]

@@ -123,5 +123,37 @@ __global__ __launch_bounds__(256) void gemm_anytiled_bf16_f16(GemmArgs g) { gemm
 
 } // extern "C"
 
+// Second half of a launch whose K was cut into slices (gemm_splitk_* in gemm_tile.h): g.a is the workspace of
+// g.ksplit slabs of M x N fp32 sums.  A thread adds the slabs of eight neighbouring columns in slice order (so the
+// result does not depend on which workgroup finished when), applies scale and epilogue as the one-pass kernels do
+// and stores sixteen bytes of C.  N is a multiple of 8.
+template <int OUT_DT> __device__ __forceinline__ void splitk_reduce_body(const GemmArgs &g) {
+  const int64_t n8 = g.N / 8, groups = (int64_t)g.M * n8, slab = (int64_t)g.M * g.N;
+  const float *ws = (const float *)g.a;
+  for (int64_t it = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; it < groups; it += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t m = it / n8, n = (it - m * n8) * 8;
+    const float *p = ws + m * g.N + n;
+    f32x4 lo = *(const f32x4 *)p, hi = *(const f32x4 *)(p + 4);
+    for (int sl = 1; sl < g.ksplit; ++sl) {
+      lo += *(const f32x4 *)(p + sl * slab);
+      hi += *(const f32x4 *)(p + sl * slab + 4);
+    }
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = apply_epilogue<OUT_DT>(g, (e < 4 ? lo[e] : hi[e - 4]) * g.scale, m, n + e);
+    u32x4 pk;
+#pragma unroll
+    for (int w = 0; w < 4; ++w)    // rounded as the one-pass kernels round
+      pk[w] = OUT_DT == DT_BF16 ? pack_bf16x2(v[2 * w], v[2 * w + 1])
+                                : (uint32_t)f32_to_f16(v[2 * w]) | ((uint32_t)f32_to_f16(v[2 * w + 1]) << 16);
+    *(u32x4 *)((uint16_t *)g.c + m * g.ldc + n) = pk;
+  }
+}
+extern "C" {
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_bf16(GemmArgs g) { splitk_reduce_body<DT_BF16>(g); }
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_f16(GemmArgs g) { splitk_reduce_body<DT_F16>(g); }
+
+} // extern "C"
+
 #include "gemm_tile.h"
 #include "gemm_tile_fp8.h"

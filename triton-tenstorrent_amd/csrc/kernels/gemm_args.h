@@ -19,5 +19,7 @@ struct GemmArgs {
   uint16_t pad_a, pad_b;    // any-shape kernels: what an element of a / b outside the matrix reads as (16-bit operand bits):
                             // 0, or a NaN for descriptors with padding == "nan" (backend/driver.py:322-329)
   int32_t tiled;            // operands are tile-major buffers with tiles BM x BK, BK x BN, BM x BN (ld* unused)
+  int32_t ksplit;           // gemm_splitk_*: slices of K (K is a multiple of 128 * ksplit); c is then the workspace of
+                            // ksplit x M x N fp32 sums.  gemm_splitk_reduce_*: slabs to add; a is then the workspace
   unsigned long long *probe; // diagnostic: workgroup 0 stores {core-clock cycles, 100 MHz ticks} of its run, or null
 };

@@ -126,23 +126,29 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int &tm
 // (MB == 4) takes the whole rounds of the grid, or every tile when the tail is not worth splitting; the
 // half-tile pass (MB == 2) takes the two 128-row halves of each tail tile when those keep at most the whole grid
 // busy, and (QUARTERS) the quarter-tile pass (MB == 1) the four 64-row quarters when even they do.
+// `live_rows`: rows of a macro tile that exist, where that is the same for every tile (256 for whole tiles; M for a
+// clamping kernel whose matrix is a single row of tiles).  Halves and quarters that lie wholly past them are not
+// work items: a 64-row matrix is finished as one quarter per tile, not as four of which three store nothing.
 struct PassItems {
   int total;       // items of this pass
   int first_tile;  // MB < 4: id of the first tail tile
   int tail_tiles;
+  int parts;       // MB < 4: live parts of a tile (halves: 1..2, quarters: 1..4)
 };
 template <int MB, bool SPLIT_TAIL, bool QUARTERS = false>
-__device__ __forceinline__ PassItems pass_items(int total_tiles) {
-  PassItems p = {total_tiles, 0, 0};
+__device__ __forceinline__ PassItems pass_items(int total_tiles, int live_rows) {
+  PassItems p = {total_tiles, 0, 0, 1};
   if constexpr (SPLIT_TAIL) {
     const int whole = total_tiles / (int)gridDim.x * (int)gridDim.x;
     p.tail_tiles = total_tiles - whole;
-    const bool quarters = QUARTERS && p.tail_tiles > 0 && 4 * p.tail_tiles <= (int)gridDim.x;
-    const bool halves = !quarters && p.tail_tiles > 0 && 2 * p.tail_tiles <= (int)gridDim.x;
+    const int q_live = (live_rows + 63) >> 6, h_live = (live_rows + 127) >> 7;
+    const bool quarters = QUARTERS && p.tail_tiles > 0 && q_live * p.tail_tiles <= (int)gridDim.x;
+    const bool halves = !quarters && p.tail_tiles > 0 && h_live * p.tail_tiles <= (int)gridDim.x;
     if (MB == 4) {
       p.total = (quarters || halves) ? whole : total_tiles;
     } else {
-      p.total = MB == 2 ? (halves ? 2 * p.tail_tiles : 0) : (quarters ? 4 * p.tail_tiles : 0);
+      p.parts = MB == 2 ? h_live : q_live;
+      p.total = MB == 2 ? (halves ? h_live * p.tail_tiles : 0) : (quarters ? q_live * p.tail_tiles : 0);
       p.first_tile = whole;
     }
   }
@@ -158,14 +164,14 @@ __device__ __forceinline__ void item_tile(const PassItems &p, int item, int tile
     part = 0;
     tile_of(item, tiles_m, tiles_n, tm, tn);
   } else {
-    constexpr int PARTS = 4 / MB, SH = MB == 2 ? 1 : 2;
+    // (p.parts is the constant 4 / MB in the kernels for whole tiles: shifts and masks there)
     int j;
     if (p.tail_tiles % 8 == 0) {
-      j = (item >> (3 + SH)) * 8 + (item & 7);
-      part = (item >> 3) & (PARTS - 1);
+      j = (item >> 3) / p.parts * 8 + (item & 7);
+      part = (item >> 3) % p.parts;
     } else {
-      j = item >> SH;
-      part = item & (PARTS - 1);
+      j = item / p.parts;
+      part = item % p.parts;
     }
     tile_of(p.first_tile + j, tiles_m, tiles_n, tm, tn);
   }
@@ -217,23 +223,31 @@ struct Ring {
 // 256 MiB at K <= 2048.  They are kernels of their own (plain epilogue only): with both forms of the stores inside
 // one kernel, several instantiations spilled copy offsets whose reloads the compiler then waits for inside the K
 // loop, with every copy in flight counted in (tile-major 8192^3: 1585 -> 1482 TFLOP/s).
+//
+// SPLITK: K is cut into g.ksplit equal slices (whole steps each) and a work item is one slice of one macro tile;
+// slice s of tile (tm, tn) leaves its fp32 sums, nothing applied, in slab s of a workspace of ksplit x M x N floats
+// that g.c points at, and gemm_splitk_reduce adds the slabs in slice order and does the rest.  For a C of few macro
+// tiles under a long K: 128 x 8192 x 8192 has 32 tiles for 256 CUs, each streaming all of K on its own.
 template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false,
-          bool QUARTERS = false, bool STREAM = false>
+          bool QUARTERS = false, bool STREAM = false, bool SPLITK = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   static_assert(MB == 4 || ((MB == 2 || (MB == 1 && QUARTERS)) && SPLIT_TAIL), "part tiles exist for the tail passes only");
+  static_assert(!SPLITK || (RAGGED && !TILED && EPI == EPI_NONE && !STREAM), "slices of K: row-major, clamping");
+  const int gK = SPLITK ? g.K / g.ksplit : g.K;      // the K of one work item
   // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
   // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
   // real M and N (the padding of C is never written, as under the reference's store mask).
   const int Mf = TILED ? (g.M + 31) / 32 * 32 : g.M, Nf = TILED ? (g.N + 31) / 32 * 32 : g.N;   // fetchable extent
-  const int Kf = (TILED || RAGGED) ? (g.K + 31) / 32 * 32 : g.K;   // K in whole steps (row-major RAGGED: the last step may end past K)
+  const int Kf = (TILED || RAGGED) ? (gK + 31) / 32 * 32 : gK;   // K in whole steps (row-major RAGGED: the last step may end past K)
   using X = MFMA<IN_DT>;
   using vec = typename X::vec;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
-  const int total_tiles = tiles_m * tiles_n;
-  const PassItems items = pass_items<MB, SPLIT_TAIL, QUARTERS>(total_tiles);
+  const int tiles_mv = SPLITK ? tiles_m * g.ksplit : tiles_m;   // SPLITK: row tm + tiles_m * s of the item grid is slice s of tile row tm
+  const int total_tiles = tiles_mv * tiles_n;
+  const PassItems items = pass_items<MB, SPLIT_TAIL, QUARTERS>(total_tiles, (RAGGED && tiles_m == 1) ? g.M : BM);
   const int total = items.total;
   const int nk_real = Kf / BK;                                    // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
@@ -373,7 +387,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // (03-matrix-multiplication.py:340-342, 359-361), so a thread clears, in the stage that received the last data
   // step, the part of its OWN sixteen bytes of each slab that lies past K, once its copies have landed and before
   // the barrier that opens the stage for reading.
-  const int k_tail = RAGGED ? g.K & 31 : 0;                       // valid k of the last data step, 0 = all 32 (row-major: a multiple of 8)
+  const int k_tail = RAGGED ? gK & 31 : 0;                       // valid k of the last data step, 0 = all 32 (row-major: a multiple of 8)
   auto clear_past_k = [&](uint8_t *stage) {
     if constexpr (RAGGED) {
       typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
@@ -413,13 +427,22 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo, bool offsets = RAGGED) {
     int tm, tn, part;
-    item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, part);
+    item_tile<MB>(items, min(t, total - 1), tiles_mv, tiles_n, tm, tn, part);
+    int slice = 0;
+    if constexpr (SPLITK) {
+      slice = tm / tiles_m;
+      tm -= slice * tiles_m;
+    }
     int64_t row0 = (int64_t)tm * BM + part * (64 * MB);
     // RAGGED: a lower half that starts past the last row has nothing to fetch or store; it is pointed at the
     // upper half's rows (which exist) and its stores all fall to the clipping
     if (RAGGED && MB < 4 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
+    if constexpr (SPLITK) {
+      ap += (int64_t)slice * gK * 2;
+      bp += (int64_t)slice * gK * g.ldb * 2;
+    }
     if (RAGGED || offsets) {
       // per-thread offsets of the tile's copies from ap / bp, one per A slab (RAGGED: rows and column chunks
       // clamped into the matrix)
@@ -504,7 +527,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       // rows past M are fetched from the last row; a pair that ends past K (K is a multiple of 8) fetches the
       // chunks past K from the pair's first chunk, which exists, and clear_pair zeroes them once they have landed;
       // a pair that starts at or past K comes from the page of zeros
-      const int valid = inner ? 64 : min(max(g.K - 32 * k, 0), 64);
+      const int valid = inner ? 64 : min(max(gK - 32 * k, 0), 64);
       const int last_row = (over ? vo_nxt : vo_cur).last_row;
       if constexpr (decltype(inner_)::value == 2) {
         // a whole pair of a tile that lies inside the matrix (all but the last row of tiles; the caller knows):
@@ -554,7 +577,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if constexpr (RAGGED && !decltype(inner_)::value) {
       if constexpr (APAIR && (I & 1)) {
         // the pair about to open (its first step is the next one) ends past K: clear what lies past
-        const int valid = min(max(g.K - 32 * (k + 1 == nk ? 0 : k + 1), 0), 64);
+        const int valid = min(max(gK - 32 * (k + 1 == nk ? 0 : k + 1), 0), 64);
         if (valid > 0 && valid < 64) {
           asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
           clear_pair(((I + 1) % R) >> 1, valid);
@@ -666,10 +689,10 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     clear_past_k(ring.s[0]);
   }
   if constexpr (RAGGED && APAIR) {
-    if (g.K < 128 && (g.K & 63)) {          // one of the first tile's two pairs ends past K
+    if (gK < 128 && (gK & 63)) {          // one of the first tile's two pairs ends past K
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (g.K < 64) clear_pair(0, g.K);
-      else clear_pair(1, g.K - 64);
+      if (gK < 64) clear_pair(0, gK);
+      else clear_pair(1, gK - 64);
     }
   }
   // step 0 has landed when only the (R - 1) * (MB + 4) younger copies are left in flight
@@ -686,7 +709,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 
   for (; t < total; t += gridDim.x) {
     int tm, tn, part;
-    item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, part);
+    item_tile<MB>(items, t, tiles_mv, tiles_n, tm, tn, part);
+    int slice = 0;
+    if constexpr (SPLITK) {
+      slice = tm / tiles_m;
+      tm -= slice * tiles_m;
+    }
     const int64_t m0 = (int64_t)tm * BM + part * (64 * MB), n0 = (int64_t)tn * BN;
 #pragma unroll
     for (int i = 0; i < NA; ++i)
@@ -739,6 +767,20 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     // reads an accumulator: sixteen idle cycles cover the four passes of a 16x16x32.
     asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
     const int64_t m = m0 + wm * (32 * MB) + i16;
+    if constexpr (SPLITK) {
+      // the slice's sums as they are: a lane's four columns of a row are sixteen contiguous bytes of the slab
+      float *slab = (float *)g.c + (int64_t)slice * g.M * g.N;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int64_t mi = m + i * 16;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int64_t n = n0 + wn * 128 + j * 16 + G4 * 4;
+          if (mi < g.M && n < g.N) *(f32x4 *)(slab + mi * g.N + n) = acc[i][j];   // (N is a multiple of 8)
+        }
+      }
+      continue;
+    }
     // A row bias depends on n only: its 32 values for this lane are fetched once, all loads in flight
     // together, instead of one dependent load per use in the loop below.
     constexpr bool ROW_BIAS = EPI == EPI_BIAS_ROW || EPI == EPI_BIAS_ROW_GELU;
@@ -867,6 +909,21 @@ GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
   GEMM_TILE_RAGGED(prefix##_epi0_stream, IN, OUT, EPI_NONE, true)
 GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
+
+// slices of K as work items (see SPLITK in body), fp32 sums into the workspace
+#define GEMM_SPLITK(name, IN)                                                                      \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
+    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
+    fast::body<IN, IN, EPI_NONE, false, true, 4, true, true, false, true>(g, ring);                 \
+    fast::body<IN, IN, EPI_NONE, false, true, 2, true, true, false, true>(g, ring);                 \
+    fast::body<IN, IN, EPI_NONE, false, true, 1, true, true, false, true>(g, ring);                 \
+  }
+GEMM_SPLITK(gemm_splitk_bf16, DT_BF16)
+GEMM_SPLITK(gemm_splitk_f16, DT_F16)
 
 // matmul_kernel on tile-major fp16 buffers, plain and with leaky_relu
 #define GEMM_TILED(name, EPI)                                                                      \

@@ -50,7 +50,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
-  const fast::PassItems items = fast::pass_items<MB, true>(tiles_m * tiles_n);
+  const fast::PassItems items = fast::pass_items<MB, true>(tiles_m * tiles_n, fast::BM);
   const int total = items.total;
   const int nk_real = g.K / BK;                                   // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R

@@ -4,6 +4,9 @@
 #include <atomic>
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
 
 #include "tt_internal.h"
 #include "../kernels/gemm_args.h"
@@ -20,13 +23,69 @@ std::atomic<unsigned long long> g_probe_last[2];
 // The plain kernels (`splits`) finish a tail of at most grid/2 macro tiles as half tiles on twice the
 // workgroups, so a problem of at most CUs/2 tiles is launched with two workgroups per tile; those that also have
 // the quarter-tile pass (`quarters`) get four workgroups per tile for a problem of at most CUs/4 tiles.
-uint32_t persistent_grid(int64_t tiles, bool splits, bool quarters = false) {
+// `live_rows`: rows of a tile that exist when the matrix is a single row of tiles (else 256): halves and quarters
+// wholly past them are not work items, so a 64-row matrix gets one workgroup per tile in the quarter pass.
+int64_t live_parts(int64_t live_rows, int64_t rows_per_part) { return cdiv64(std::min<int64_t>(live_rows, 256), rows_per_part); }
+uint32_t persistent_grid(int64_t tiles, bool splits, bool quarters = false, int64_t live_rows = 256) {
   const int64_t cus = props()->multiprocessor_count;
   if (tiles >= cus) return (uint32_t)cus;
   const bool no_split = env_int("TTAMD_GEMM_NO_SPLIT", 0) != 0;
-  if (quarters && 4 * tiles <= cus && !no_split) return (uint32_t)(4 * tiles);
-  if (splits && 2 * tiles <= cus && !no_split) return (uint32_t)(2 * tiles);
+  if (quarters && live_parts(live_rows, 64) * tiles <= cus && !no_split) return (uint32_t)(live_parts(live_rows, 64) * tiles);
+  if (splits && live_parts(live_rows, 128) * tiles <= cus && !no_split) return (uint32_t)(live_parts(live_rows, 128) * tiles);
   return (uint32_t)tiles;
+}
+
+// K in slices (gemm_splitk_*): the slices' fp32 sums pass through a workspace of ksplit x M x N floats.  Launches on
+// one stream run in order and share one workspace; every (device, stream) pair gets its own on first use, grown when
+// a launch needs more (the stream is drained first) and kept until rt_release_stream or the end of the process.  A
+// launch that is being recorded into a graph does not take this path: the graph could be replayed on any stream,
+// beside eager launches on the one it was recorded on, with the workspace's address baked in.
+constexpr int64_t kSplitKMaxBytes = 64ll << 20;
+std::mutex g_ws_mu;
+struct Workspace { void *p; int64_t bytes; };
+std::map<std::pair<int, void *>, Workspace> g_ws;
+void *splitk_workspace(void *stream, int64_t bytes) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing((hipStream_t)stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  std::lock_guard<std::mutex> lk(g_ws_mu);
+  Workspace &w = g_ws[{dev, stream}];
+  if (w.bytes >= bytes) return w.p;
+  if (w.p) {
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess || hipFree(w.p) != hipSuccess) return nullptr;
+    w = {nullptr, 0};
+  }
+  void *p = nullptr;
+  if (hipMalloc(&p, (size_t)bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  w = {p, bytes};
+  return p;
+}
+
+// Slices of K for a launch of `tiles` macro tiles, or 1.  A problem of few tiles is finished as quarter tiles (64
+// rows by 256 columns, `parts` live ones per tile); where even those leave CUs idle and K is long, slices of K make
+// more of them: the largest power of two that still fits one round of the grid, keeps every slice at sixteen steps or
+// more and the workspace within bounds.  What it costs is one more launch and a pass over ksplit x M x N floats in
+// each direction (taken at 3 us and 4 TB/s); what it saves is (1 - 1/ksplit) of K/32 quarter-tile steps of about
+// 0.235 us.
+int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
+  const int64_t cus = props()->multiprocessor_count;
+  if (env_int("TTAMD_GEMM_NO_SPLITK", 0) || 2 * parts * tiles > cus) return 1;
+  int s = 1;
+  while (2 * s * parts * tiles <= cus && K % (2 * s * 128) == 0 && K / (2 * s) >= 512 &&
+         2 * s * M * N * 4 <= kSplitKMaxBytes)
+    s *= 2;
+  if (const int forced = env_int("TTAMD_GEMM_KSPLIT", 0)) s = (K % (forced * 128) == 0 && (int64_t)forced * M * N * 4 <= kSplitKMaxBytes) ? forced : 1;
+  if (s == 1) return 1;
+  const double saved_us = (double)(K / 32) * (1.0 - 1.0 / s) * 0.235;
+  const double cost_us = 3.0 + (double)s * M * N * 8 / 4.0e6;
+  return (saved_us > cost_us || env_int("TTAMD_GEMM_KSPLIT", 0)) ? s : 1;
 }
 
 int check_desc(const char *who, const char *what, const tt_desc2d *d, int64_t rows, int64_t cols) {
@@ -140,7 +199,28 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     snprintf(fast_name, sizeof(fast_name), "gemm_%s_%s_epi%d%s", fast_shape ? "tile" : "ragged", in == TT_BF16 ? "bf16" : "f16",
              epi, past_caches ? "_stream" : "");
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = persistent_grid(tiles, true, true);
+    const int64_t live_rows = M <= 256 ? M : 256;      // of a tile, where the matrix is a single row of tiles
+    const int ksplit = pick_ksplit(tiles, live_parts(live_rows, 64), M, N, K);
+    if (ksplit > 1) {
+      if (void *ws = splitk_workspace(stream, (int64_t)ksplit * M * N * 4)) {
+        GemmArgs part = g, sum = g;
+        part.c = ws;
+        part.ksplit = ksplit;
+        part.epi = TT_EPI_NONE;
+        void *pargs[] = {&part};
+        const uint32_t pwgs = persistent_grid(tiles * ksplit, true, true, live_rows);
+        int lrc = launch("gemm", in == TT_BF16 ? "gemm_splitk_bf16" : "gemm_splitk_f16", dim3(pwgs), dim3(256), 0, stream, pargs, 1);
+        if (lrc) return lrc;
+        sum.a = ws;
+        sum.ksplit = ksplit;
+        void *sargs[] = {&sum};
+        const int64_t groups = (int64_t)M * (N / 8);
+        const uint32_t swgs = (uint32_t)std::min<int64_t>(cdiv64(groups, 256), (int64_t)props()->multiprocessor_count * 8);
+        return launch("gemm", out == TT_BF16 ? "gemm_splitk_reduce_bf16" : "gemm_splitk_reduce_f16", dim3(swgs), dim3(256), 0,
+                      stream, sargs, 1);
+      }
+    }
+    const uint32_t wgs = persistent_grid(tiles, true, true, fast_shape ? 256 : live_rows);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
     // 100 MHz ticks; the launch is then synchronous and prints the effective clock.
     static unsigned long long *probe_buf = nullptr;
@@ -191,6 +271,15 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
 }
 
 } // namespace
+
+void *ttamd::gemm_take_workspace(int device, void *stream) {
+  std::lock_guard<std::mutex> lk(g_ws_mu);
+  auto it = g_ws.find({device, stream});
+  if (it == g_ws.end()) return nullptr;
+  void *p = it->second.p;
+  g_ws.erase(it);
+  return p;
+}
 
 extern "C" {
 

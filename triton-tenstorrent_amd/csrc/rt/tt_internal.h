@@ -34,6 +34,9 @@ constexpr size_t kReduceCounterAt = kReduceMaxGroups * 16, kReduceScratchBytes =
 int reduce1d_launch(int32_t op, const void *x, void *z, int32_t BLOCK, int32_t in_dtype, int32_t acc_dtype,
                     int32_t out_dtype, int32_t propagate_nan, const uint32_t grid[3], void *stream,
                     void *fixed_scratch);
+// Takes the workspace that K-sliced matmul launches on (device, stream) share out of the library's table and returns
+// it (null: none); the caller frees it once the stream has drained.
+void *gemm_take_workspace(int device, void *stream);
 // Resolves the address of the static scratch array on the current device; called by rt_init.
 int static_scratch_setup(int device);
 // Integer environment knob read once per name (tuning sweeps only).

@@ -139,13 +139,17 @@ extern "C" int rt_release_stream(void *stream) {
   {
     std::lock_guard<std::mutex> lk(g_mu);
     auto it = g_bufs.find({dev, stream});
-    if (it == g_bufs.end()) return RT_OK;
-    p = it->second;
-    g_bufs.erase(it);
+    if (it != g_bufs.end()) {
+      p = it->second;
+      g_bufs.erase(it);
+    }
   }
+  void *w = ttamd::gemm_take_workspace(dev, stream);
+  if (!p && !w) return RT_OK;
   hipError_t e = hipStreamSynchronize((hipStream_t)stream);
   if (e != hipSuccess) return hip_fail(e, "rt_release_stream: hipStreamSynchronize");
-  e = hipFree(p);
-  if (e != hipSuccess) return hip_fail(e, "rt_release_stream: hipFree");
+  for (void *q : {p, w}) {
+    if (q && (e = hipFree(q)) != hipSuccess) return hip_fail(e, "rt_release_stream: hipFree");
+  }
   return RT_OK;
 }
