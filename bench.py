@@ -227,6 +227,20 @@ def main() -> int:
             ragged[f"{m_}x{n_}x{k_}"] = {"kernel": rt.last_kernel_name(), "TFLOPs": round(2.0 * m_ * n_ * k_ / (avg_ms * 1e-3) / 1e12, 1)}
             del a, b
         extra["gemm_bf16_ragged_shapes"] = ragged
+        # few output tiles under a long K: computed in slices of K (two launches; the time is that of the pair).  These
+        # are bounded by the one pass over B: GB/s of A + B + C against the HBM peak
+        skinny = {}
+        for (m_, n_, k_) in ((16, 8192, 8192), (128, 8192, 8192), (64, 4096, 8192)):
+            a = (torch.randn(m_, k_, device="cuda") / math.sqrt(k_)).to(torch.bfloat16)
+            b = (torch.randn(k_, n_, device="cuda") / math.sqrt(k_)).to(torch.bfloat16)
+            avg_ms, per, _ = _events_time(lambda: K.matmul_tma(a, b), max(3, steps // 4), 2, stream)
+            byts = 2.0 * (m_ * k_ + k_ * n_ + m_ * n_)
+            skinny[f"{m_}x{n_}x{k_}"] = {"kernel": rt.last_kernel_name(), "us": round(avg_ms * 1e3, 1),
+                                         "TFLOPs": round(2.0 * m_ * n_ * k_ / (avg_ms * 1e-3) / 1e12, 1),
+                                         "GBs": round(byts / (avg_ms * 1e-3) / 1e9, 0),
+                                         "frac_of_hbm_peak": round(byts / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 3)}
+            del a, b
+        extra["gemm_bf16_few_tiles_long_k"] = skinny
 
     # ---------------- elementwise streaming, N = 2^28 ----------------------
     n_el = 1 << 28
