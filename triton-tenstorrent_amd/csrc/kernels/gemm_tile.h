@@ -135,10 +135,15 @@ struct PassItems {
   int tail_tiles;
   int parts;       // MB < 4: live parts of a tile (halves: 1..2, quarters: 1..4)
 };
-template <int MB, bool SPLIT_TAIL, bool QUARTERS = false>
+// ALLQ: every tile is finished as quarters (the kernels of the K slices, whose launches have no whole round).
+template <int MB, bool SPLIT_TAIL, bool QUARTERS = false, bool ALLQ = false>
 __device__ __forceinline__ PassItems pass_items(int total_tiles, int live_rows) {
   PassItems p = {total_tiles, 0, 0, 1};
-  if constexpr (SPLIT_TAIL) {
+  if constexpr (ALLQ) {
+    p.parts = (live_rows + 63) >> 6;
+    p.total = p.parts * total_tiles;
+    p.tail_tiles = total_tiles;
+  } else if constexpr (SPLIT_TAIL) {
     const int whole = total_tiles / (int)gridDim.x * (int)gridDim.x;
     p.tail_tiles = total_tiles - whole;
     const int q_live = (live_rows + 63) >> 6, h_live = (live_rows + 127) >> 7;
@@ -229,8 +234,12 @@ struct Ring {
 // that g.c points at, and gemm_splitk_reduce adds the slabs in slice order and does the rest.  For a C of few macro
 // tiles under a long K: 128 x 8192 x 8192 has 32 tiles for 256 CUs, each streaming all of K on its own.
 template <int IN_DT, int OUT_DT, int EPI, bool TILED = false, bool RAGGED = false, int MB = 4, bool SPLIT_TAIL = false,
-          bool QUARTERS = false, bool STREAM = false, bool SPLITK = false>
+          bool QUARTERS = false, bool STREAM = false, bool SPLITK = false, bool ALLQ = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
+  static_assert(!ALLQ || (MB == 1 && SPLITK), "quarters only: the K-slice kernels");
+  // where B's slabs start in a stage.  ALLQ: right behind the one A slab a quarter has, so that a stage is 20 KiB,
+  // the ring 80 KiB and two workgroups share a CU
+  constexpr int B_OFF = ALLQ ? 4096 : A_BYTES;
   static_assert(MB == 4 || ((MB == 2 || (MB == 1 && QUARTERS)) && SPLIT_TAIL), "part tiles exist for the tail passes only");
   static_assert(!SPLITK || (RAGGED && !TILED && EPI == EPI_NONE && !STREAM), "slices of K: row-major, clamping");
   const int gK = SPLITK ? g.K / g.ksplit : g.K;      // the K of one work item
@@ -247,7 +256,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
   const int tiles_mv = SPLITK ? tiles_m * g.ksplit : tiles_m;   // SPLITK: row tm + tiles_m * s of the item grid is slice s of tile row tm
   const int total_tiles = tiles_mv * tiles_n;
-  const PassItems items = pass_items<MB, SPLIT_TAIL, QUARTERS>(total_tiles, (RAGGED && tiles_m == 1) ? g.M : BM);
+  const PassItems items = pass_items<MB, SPLIT_TAIL, QUARTERS, ALLQ>(total_tiles, (RAGGED && tiles_m == 1) ? g.M : BM);
   const int total = items.total;
   const int nk_real = Kf / BK;                                    // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
@@ -311,7 +320,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) b_vs[i] = b_voff + (uint32_t)b_slab_off(i);
   // k = 8*G4 + 4h + q lies in slab h + 2*(G4>>1), row q + 4*(G4&1) of it; its swizzle is (q<<2) | ((G4&1)<<1)
-  const int b_base = A_BYTES + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
+  const int b_base = B_OFF + ((16 * (G4 >> 1) + 4 * (G4 & 1) + q) * 512) + ((wn * 16 + ((i16 >> 1) & 1)) << 4) +
                      ((i16 & 1) << 3);
   int b_pos[8];                                                             // half h: + h * 4096
 #pragma unroll
@@ -408,7 +417,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       // B: this thread's sixteen bytes of slab i lie in k row b_row0(i) + b_kk
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + A_BYTES + i * 4096 + lds_wave + lane * 16);
+        lds_u32x4 *p = (lds_u32x4 *)(lds_void *)(stage + B_OFF + i * 4096 + lds_wave + lane * 16);
         if (b_row0(i) + b_kk >= k_tail) *p = (u32x4){0, 0, 0, 0};
       }
     }
@@ -478,9 +487,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
       if (i < MB)
         dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
       else if constexpr (APAIR && !RAGGED)
-        dma_one(b_cur + (int64_t)k * b_kstep, b_vs[i - MB], stage + A_BYTES + (i - MB) * 4096);
+        dma_one(b_cur + (int64_t)k * b_kstep, b_vs[i - MB], stage + B_OFF + (i - MB) * 4096);
       else
-        dma_one(b_cur + (int64_t)k * b_kstep + b_slab_off(i - MB), vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
+        dma_one(b_cur + (int64_t)k * b_kstep + b_slab_off(i - MB), vo_cur.b, stage + B_OFF + (i - MB) * 4096);
     } else if constexpr (RAGGED) {
       const bool zero = k >= nk_real;                         // a padding step: both operands are zeros
       // row-major operands, last data step of a K that is not a whole number of steps: the 16-byte chunks of A past
@@ -501,15 +510,15 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
         const uint8_t *bp = zero ? zero_page
                                  : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (redirect ? (ib & 1) * b_rows4 : b_slab_off(ib));
         const uint32_t bv = redirect ? vo.b - (uint32_t)((wave >> 1) * 2 * b_rows4) : vo.b;
-        dma_one(bp, zero ? z_voff : bv, stage + A_BYTES + (i - MB) * 4096);
+        dma_one(bp, zero ? z_voff : bv, stage + B_OFF + (i - MB) * 4096);
       }
     } else if (i < MB) {
       const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
-      if constexpr (APAIR) dma_one(bp, b_vs[i - MB], stage + A_BYTES + (i - MB) * 4096);
-      else dma_one(bp + b_slab_off(i - MB), b_voff, stage + A_BYTES + (i - MB) * 4096);
+      if constexpr (APAIR) dma_one(bp, b_vs[i - MB], stage + B_OFF + (i - MB) * 4096);
+      else dma_one(bp + b_slab_off(i - MB), b_voff, stage + B_OFF + (i - MB) * 4096);
     }
   };
 
@@ -910,17 +919,15 @@ GEMM_TILE_ALL_EPI(gemm_tile_f16, DT_F16, DT_F16)
 GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_bf16, DT_BF16, DT_BF16)
 GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
 
-// slices of K as work items (see SPLITK in body), fp32 sums into the workspace
+// Slices of K as work items (see SPLITK in body), fp32 sums into the workspace.  Such a launch has at most one round
+// of quarter tiles, so the kernel is the quarter-tile body alone: 16 + 48 accumulator and fragment registers instead
+// of 256 + 128 and a ring of 4 x 20 KiB, i.e. two workgroups per CU.  That is what these launches want: the small
+// ones among them stream B once from memory, and twice the copies in flight per CU is 30 % more bandwidth there.
 #define GEMM_SPLITK(name, IN)                                                                      \
-  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void name(GemmArgs g) { \
-    __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast::STAGE];                            \
-    __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast::STAGE];                            \
-    __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast::STAGE];                            \
-    __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast::STAGE];                            \
-    fast::Ring ring = {{lds0, lds1, lds2, lds3}};                                                   \
-    fast::body<IN, IN, EPI_NONE, false, true, 4, true, true, false, true>(g, ring);                 \
-    fast::body<IN, IN, EPI_NONE, false, true, 2, true, true, false, true>(g, ring);                 \
-    fast::body<IN, IN, EPI_NONE, false, true, 1, true, true, false, true>(g, ring);                 \
+  __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void name(GemmArgs g) { \
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[4][20480];                                \
+    fast::Ring ring = {{lds[0], lds[1], lds[2], lds[3]}};                                           \
+    fast::body<IN, IN, EPI_NONE, false, true, 1, true, true, false, true, true>(g, ring);           \
   }
 GEMM_SPLITK(gemm_splitk_bf16, DT_BF16)
 GEMM_SPLITK(gemm_splitk_f16, DT_F16)

@@ -70,15 +70,16 @@ void *splitk_workspace(void *stream, int64_t bytes) {
 
 // Slices of K for a launch of `tiles` macro tiles, or 1.  A problem of few tiles is finished as quarter tiles (64
 // rows by 256 columns, `parts` live ones per tile); where even those leave CUs idle and K is long, slices of K make
-// more of them: the largest power of two that still fits one round of the grid, keeps every slice at sixteen steps or
-// more and the workspace within bounds.  What it costs is one more launch and a pass over ksplit x M x N floats in
+// more of them: the largest power of two up to 16 that gives at most one quarter tile per CU (the kernel fits two
+// on a CU, but past one per CU the growing workspace costs more than the slices save: 128 x 8192 x 8192 37, 44 and
+// 53 us with 4, 8 and 16 slices), keeps every slice at sixteen steps or more and the workspace within bounds.  What it costs is one more launch and a pass over ksplit x M x N floats in
 // each direction (taken at 3 us and 4 TB/s); what it saves is (1 - 1/ksplit) of K/32 quarter-tile steps of about
 // 0.235 us.
 int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
   const int64_t cus = props()->multiprocessor_count;
   if (env_int("TTAMD_GEMM_NO_SPLITK", 0) || 2 * parts * tiles > cus) return 1;
   int s = 1;
-  while (2 * s * parts * tiles <= cus && K % (2 * s * 128) == 0 && K / (2 * s) >= 512 &&
+  while (s < 16 && 2 * s * parts * tiles <= cus && K % (2 * s * 128) == 0 && K / (2 * s) >= 512 &&
          2 * s * M * N * 4 <= kSplitKMaxBytes)
     s *= 2;
   if (const int forced = env_int("TTAMD_GEMM_KSPLIT", 0)) s = (K % (forced * 128) == 0 && (int64_t)forced * M * N * 4 <= kSplitKMaxBytes) ? forced : 1;
@@ -208,7 +209,8 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
         part.ksplit = ksplit;
         part.epi = TT_EPI_NONE;
         void *pargs[] = {&part};
-        const uint32_t pwgs = persistent_grid(tiles * ksplit, true, true, live_rows);
+        // every tile as its live quarters, two workgroups per CU
+        const uint32_t pwgs = (uint32_t)std::min<int64_t>(live_parts(live_rows, 64) * tiles * ksplit, 2 * (int64_t)props()->multiprocessor_count);
         int lrc = launch("gemm", in == TT_BF16 ? "gemm_splitk_bf16" : "gemm_splitk_f16", dim3(pwgs), dim3(256), 0, stream, pargs, 1);
         if (lrc) return lrc;
         sum.a = ws;
