@@ -9,6 +9,8 @@
 //                clipped stores.  One wavefront owns one 32x32 piece of a
 //                logical tile and walks K with v_mfma_f32_32x32x16, operands
 //                straight from global memory.  Correctness path, not a fast one.
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace {
@@ -133,10 +135,37 @@ template <int OUT_DT> __device__ __forceinline__ void splitk_reduce_body(const G
   for (int64_t it = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; it < groups; it += (int64_t)gridDim.x * blockDim.x) {
     const int64_t m = it / n8, n = (it - m * n8) * 8;
     const float *p = ws + m * g.N + n;
-    f32x4 lo = *(const f32x4 *)p, hi = *(const f32x4 *)(p + 4);
-    for (int sl = 1; sl < g.ksplit; ++sl) {
-      lo += *(const f32x4 *)(p + sl * slab);
-      hi += *(const f32x4 *)(p + sl * slab + 4);
+    f32x4 lo, hi;
+    // the slabs' loads all in flight before the first addition (a loop of dependent loads took one memory round trip
+    // per slab); the additions stay in slice order
+    auto sum_of = [&](auto s_) __attribute__((always_inline)) {
+      constexpr int S = decltype(s_)::value;
+      f32x4 l[S], h[S];
+#pragma unroll
+      for (int sl = 0; sl < S; ++sl) {
+        l[sl] = *(const f32x4 *)(p + sl * slab);
+        h[sl] = *(const f32x4 *)(p + sl * slab + 4);
+      }
+      lo = l[0];
+      hi = h[0];
+#pragma unroll
+      for (int sl = 1; sl < S; ++sl) {
+        lo += l[sl];
+        hi += h[sl];
+      }
+    };
+    switch (g.ksplit) {
+    case 2: sum_of(std::integral_constant<int, 2>{}); break;
+    case 4: sum_of(std::integral_constant<int, 4>{}); break;
+    case 8: sum_of(std::integral_constant<int, 8>{}); break;
+    case 16: sum_of(std::integral_constant<int, 16>{}); break;
+    default:
+      lo = *(const f32x4 *)p;
+      hi = *(const f32x4 *)(p + 4);
+      for (int sl = 1; sl < g.ksplit; ++sl) {
+        lo += *(const f32x4 *)(p + sl * slab);
+        hi += *(const f32x4 *)(p + sl * slab + 4);
+      }
     }
     float v[8];
 #pragma unroll
