@@ -73,7 +73,7 @@ void *splitk_workspace(void *stream, int64_t bytes) {
 // more of them: the largest power of two up to 16 that gives at most one quarter tile per CU (the kernel fits two
 // on a CU, but past one per CU the growing workspace costs more than the slices save: 128 x 8192 x 8192 37, 44 and
 // 53 us with 4, 8 and 16 slices), keeps every slice at sixteen steps or more and the workspace within bounds.  What it costs is one more launch and a pass over ksplit x M x N floats in
-// each direction (taken at 3 us and 4 TB/s); what it saves is (1 - 1/ksplit) of K/32 quarter-tile steps of about
+// each direction (taken at 6 us, the adding kernel alone runs 4-5, and 4 TB/s); what it saves is (1 - 1/ksplit) of K/32 quarter-tile steps of about
 // 0.235 us.
 int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
   const int64_t cus = props()->multiprocessor_count;
@@ -85,7 +85,7 @@ int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
   if (const int forced = env_int("TTAMD_GEMM_KSPLIT", 0)) s = (K % (forced * 128) == 0 && (int64_t)forced * M * N * 4 <= kSplitKMaxBytes) ? forced : 1;
   if (s == 1) return 1;
   const double saved_us = (double)(K / 32) * (1.0 - 1.0 / s) * 0.235;
-  const double cost_us = 3.0 + (double)s * M * N * 8 / 4.0e6;
+  const double cost_us = 6.0 + (double)s * M * N * 8 / 4.0e6;
   return (saved_us > cost_us || env_int("TTAMD_GEMM_KSPLIT", 0)) ? s : 1;
 }
 
