@@ -54,3 +54,46 @@ def test_concurrent_launches_from_four_threads():
         t.join(timeout=100)
     assert not errors, errors
     assert len(results) == n_threads and not any(t.is_alive() for t in threads)
+
+
+def test_matmuls_in_slices_of_k_from_threads_that_share_a_stream():
+    """A matmul of few tiles under a long K is two launches that share the stream's workspace.  Threads that feed ONE
+    stream (each orders its own work with the others' only through that stream) must not interleave their pairs:
+    small-integer operands, so every result is exact and a slab of another thread's slices would show."""
+    rt.init(0)
+    n_threads, rounds = 4, 30
+    stream = torch.cuda.Stream()
+    errors: list = []
+    done: list = []
+    g = torch.Generator(device="cuda").manual_seed(3)
+    shapes = [(64, 256, 2048), (200, 520, 2048), (130, 264, 4096), (16, 512, 4096)]
+    data = []
+    for (M, N, Kd) in shapes:
+        a = torch.randint(-3, 4, (M, Kd), device="cuda", generator=g).to(torch.bfloat16)
+        b = torch.randint(-3, 4, (Kd, N), device="cuda", generator=g).to(torch.bfloat16)
+        data.append((a, b, (a.float() @ b.float()).to(torch.bfloat16)))
+    torch.cuda.synchronize()
+
+    def worker(tid: int):
+        try:
+            torch.cuda.set_device(0)
+            a, b, want = data[tid]
+            with torch.cuda.stream(stream):
+                outs = []
+                for _ in range(rounds):
+                    outs.append(K.matmul_tma(a, b))
+                    assert rt.last_kernel_name() == "gemm_splitk_reduce_bf16"
+                stream.synchronize()
+                for c in outs:
+                    assert torch.equal(c, want)
+            done.append(tid)
+        except BaseException as e:      # noqa: BLE001 - reported in the main thread
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i, )) for i in range(n_threads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert len(done) == n_threads and not any(t.is_alive() for t in threads)

@@ -203,6 +203,11 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     const int64_t live_rows = M <= 256 ? M : 256;      // of a tile, where the matrix is a single row of tiles
     const int ksplit = pick_ksplit(tiles, live_parts(live_rows, 64), M, N, K);
     if (ksplit > 1) {
+      // From the lookup of the workspace to the second launch nothing of another thread's comes between: two threads
+      // that feed one stream would otherwise interleave their pairs (the second's slices landing under the first's
+      // sums), or one would grow the workspace, which frees the old one, between the other's lookup and launches.
+      static std::mutex pair_mu;
+      std::lock_guard<std::mutex> pair(pair_mu);
       if (void *ws = splitk_workspace(stream, (int64_t)ksplit * M * N * 4)) {
         GemmArgs part = g, sum = g;
         part.c = ws;
