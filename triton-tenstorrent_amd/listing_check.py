@@ -1,4 +1,5 @@
-"""Static check of a gfx950 assembly listing: nothing but another MFMA touches an MFMA's result too early.
+"""Static checks of a gfx950 assembly listing around MFMAs issued from inline assembly: nothing but another MFMA
+touches an MFMA's result too early, and no register-file copy lands right in front of the MFMA that reads it.
 
 The hot kernels issue their MFMAs from inline assembly (that is how the accumulators stay in AGPRs and a
 direct-to-LDS copy rides behind an MFMA).  The compiler does not look inside such a statement, so it does not know
@@ -126,6 +127,46 @@ def mfma_result_hazards(lines: list[str]) -> list[str]:
     return found
 
 
+def accvgpr_copies_in_front_of_an_mfma(lines: list[str], states: int = 2) -> list[str]:
+    """One message per v_accvgpr_read / _write / _mov whose result an MFMA reads fewer than `states` wait states later
+    (straight-line: such a copy sits in the MFMA's own block).  The compiler moves operands between the register
+    files where it likes, and in front of an inline-assembly MFMA it leaves no distance: the MFMA then read the
+    register before the copy had arrived (attention, head dim 256: scores off by a few per cent, exact with one idle
+    state in between; that kernel's MFMAs carry two)."""
+    ins, in_asm = [], False
+    for line in lines:
+        if _LABEL.match(line):
+            ins.append(None)       # a block boundary ends the look-back
+            continue
+        if "ASMSTART" in line or "ASMEND" in line:
+            in_asm = "ASMSTART" in line
+            continue
+        if not line.startswith("\t"):
+            continue
+        text = line.strip()
+        if not text or text[0] in ";.":
+            continue
+        parts = text.split(None, 1)
+        ops = [o.strip().split(" ")[0] for o in parts[1].split(",")] if len(parts) > 1 else []
+        ins.append((parts[0], ops, text, in_asm))
+    found = []
+    for i, cur in enumerate(ins):
+        # (an MFMA that the compiler issued itself has the distance the hardware asks for)
+        if cur is None or not cur[0].startswith("v_mfma") or not cur[3]:
+            continue
+        reads = set()
+        for o in cur[1][1:]:
+            reads |= _regs(o)
+        st, k = 0, i - 1
+        while k >= 0 and st < states and ins[k] is not None:
+            op2, ops2, text2, _ = ins[k]
+            if op2.startswith("v_accvgpr") and ops2 and _regs(ops2[0]) & reads:
+                found.append(f"{st} states in front of `{cur[2]}`: `{text2}`")
+            st += _states(op2, ops2)
+            k -= 1
+    return found
+
+
 def vmcnt_waits_in_mfma_blocks(lines: list[str], min_mfma: int = 32) -> int:
     """Number of `s_waitcnt vmcnt(...)` that the compiler placed (outside inline assembly) in basic blocks with at
     least `min_mfma` MFMAs, i.e. in the K loops.  The kernels track their direct-to-LDS copies by hand; a wait the
@@ -156,7 +197,7 @@ def check_listing(listing: str) -> dict[str, list[str]]:
     out = {}
     for name, lines in split_kernels(listing).items():
         if any("v_mfma" in l for l in lines):
-            h = mfma_result_hazards(lines)
+            h = mfma_result_hazards(lines) + accvgpr_copies_in_front_of_an_mfma(lines)
             if h:
                 out[name] = h
     return out
