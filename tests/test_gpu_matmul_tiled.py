@@ -250,3 +250,45 @@ def test_tiled_clamping_kernel_half_tile_tail(M, N, K_):
     assert rt.last_kernel_name() == "gemm_tiledragged_f16_epi0"
     assert torch.equal(K.untilize(ct, M, N, 32, 32), (a.cuda().float() @ b.cuda().float()).to(torch.float16))
 
+
+
+# ---- few tiles under a long K: slices of K (the tile-major kernel's own instantiation, a row-major workspace) -----
+@pytest.mark.parametrize("M,N,K_", [(64, 45, 2048), (1, 77, 2048), (300, 200, 3072), (200, 520, 2048), (256, 256, 4096)])
+@pytest.mark.parametrize("act", ["", "leaky_relu"])
+def test_tiled_k_slices_vs_oracle(M, N, K_, act):
+    a, b = _rand((M, K_), 31), _rand((K_, N), 32)
+    at, bt = K.tilize(a, 32, 32), K.tilize(b, 32, 32)
+    ct = K.matmul_tiled(at.cuda(), bt.cuda(), M, N, K_, activation=act)
+    assert rt.last_kernel_name() == "gemm_splitk_reduce_f16"
+    ref = orc.matmul_tiled(_bits(at), _bits(bt), M, N, K_, in_dt=orc.F16, leaky_relu=bool(act), acc64=True)
+    gm, rm = orc.untilize(_bits(ct.cpu()), M, N, 32, 32), orc.untilize(ref, M, N, 32, 32)
+    assert _close(_f16(gm), _f16(rm))
+    again = K.matmul_tiled(at.cuda(), bt.cuda(), M, N, K_, activation=act)      # slabs added in slice order: the same bits
+    assert np.array_equal(orc.untilize(_bits(again.cpu()), M, N, 32, 32), gm)
+
+
+def test_tiled_k_slices_exact_padding_untouched_and_ignored():
+    """Small integers, bit for bit; the padding of the C tiles keeps the NaN it was filled with; NaN in the padding
+    of A (rows past M) and of B (columns past N) does not reach the result (K is whole tiles on this route)."""
+    rng = np.random.default_rng(5)
+    for case in range(8):
+        M, N = int(rng.integers(1, 400)), int(rng.integers(1, 600))
+        K_ = int(rng.integers(8, 24)) * 256
+        g = torch.Generator().manual_seed(case)
+        a = torch.randint(-3, 4, (M, K_), generator=g).to(torch.float16)
+        b = torch.randint(-3, 4, (K_, N), generator=g).to(torch.float16)
+        Mp, Np = K.cdiv(M, 32) * 32, K.cdiv(N, 32) * 32
+        an = torch.full((Mp, K_), float("nan"), dtype=torch.float16); an[:M] = a
+        bn = torch.full((K_, Np), float("nan"), dtype=torch.float16); bn[:, :N] = b
+        tm, tn = Mp // 32, Np // 32
+        c = torch.full((tm * tn * 1024, ), float("nan"), dtype=torch.float16, device="cuda")
+        act = "leaky_relu" if case % 3 == 0 else ""
+        K.matmul_kernel[(tm * tn, )](K.tilize(an, 32, 32).cuda(), K.tilize(bn, 32, 32).cuda(), c, M, N, K_, K_, 1, N, 1, N, 1,
+                                     ACTIVATION=act)
+        assert rt.last_kernel_name() == "gemm_splitk_reduce_f16", (M, N, K_)
+        full = c.cpu().reshape(tm, tn, 32, 32).permute(0, 2, 1, 3).reshape(Mp, Np)
+        want = a.float() @ b.float()
+        if act:
+            want = torch.where(want >= 0, want, 0.01 * want)
+        assert torch.equal(full[:M, :N], want.to(torch.float16)), (M, N, K_)
+        assert torch.isnan(full[M:, :]).all() and torch.isnan(full[:, N:]).all(), (M, N, K_)

@@ -128,13 +128,15 @@ __global__ __launch_bounds__(256) void gemm_anytiled_bf16_f16(GemmArgs g) { gemm
 // Second half of a launch whose K was cut into slices (gemm_splitk_* in gemm_tile.h): g.a is the workspace of
 // g.ksplit slabs of M x N fp32 sums.  A thread adds the slabs of eight neighbouring columns in slice order (so the
 // result does not depend on which workgroup finished when), applies scale and epilogue as the one-pass kernels do
-// and stores sixteen bytes of C.  N is a multiple of 8.
+// and stores sixteen bytes of C.  Row-major C: N is a multiple of 8.  Tile-major C (g.tiled: 32x32 tiles, any N):
+// eight neighbouring columns lie inside one tile; a group that reaches past N goes by element, and the padding of the
+// buffer is never written.
 template <int OUT_DT> __device__ __forceinline__ void splitk_reduce_body(const GemmArgs &g) {
-  const int64_t n8 = g.N / 8, groups = (int64_t)g.M * n8, slab = (int64_t)g.M * g.N;
+  const int64_t n8 = g.ldws / 8, groups = (int64_t)g.M * n8, slab = (int64_t)g.M * g.ldws;
   const float *ws = (const float *)g.a;
   for (int64_t it = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; it < groups; it += (int64_t)gridDim.x * blockDim.x) {
     const int64_t m = it / n8, n = (it - m * n8) * 8;
-    const float *p = ws + m * g.N + n;
+    const float *p = ws + m * g.ldws + n;
     f32x4 lo, hi;
     // the slabs' loads all in flight before the first addition (a loop of dependent loads took one memory round trip
     // per slab); the additions stay in slice order
@@ -175,7 +177,17 @@ template <int OUT_DT> __device__ __forceinline__ void splitk_reduce_body(const G
     for (int w = 0; w < 4; ++w)    // rounded as the one-pass kernels round
       pk[w] = OUT_DT == DT_BF16 ? pack_bf16x2(v[2 * w], v[2 * w + 1])
                                 : (uint32_t)f32_to_f16(v[2 * w]) | ((uint32_t)f32_to_f16(v[2 * w + 1]) << 16);
-    *(u32x4 *)((uint16_t *)g.c + m * g.ldc + n) = pk;
+    if (g.tiled) {
+      const int64_t ntn = (g.N + 31) / 32;
+      uint16_t *dst = (uint16_t *)g.c + (((m >> 5) * ntn + (n >> 5)) << 10) + (m & 31) * 32 + (n & 31);
+      if (n + 8 <= g.N) {
+        *(u32x4 *)dst = pk;
+      } else {
+        for (int e = 0; n + e < g.N; ++e) dst[e] = (uint16_t)(e & 1 ? pk[e >> 1] >> 16 : pk[e >> 1] & 0xffffu);
+      }
+    } else {
+      *(u32x4 *)((uint16_t *)g.c + m * g.ldc + n) = pk;
+    }
   }
 }
 extern "C" {

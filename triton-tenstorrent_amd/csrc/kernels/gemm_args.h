@@ -20,6 +20,7 @@ struct GemmArgs {
                             // 0, or a NaN for descriptors with padding == "nan" (backend/driver.py:322-329)
   int32_t tiled;            // operands are tile-major buffers with tiles BM x BK, BK x BN, BM x BN (ld* unused)
   int32_t ksplit;           // gemm_splitk_*: slices of K (K is a multiple of 128 * ksplit); c is then the workspace of
-                            // ksplit x M x N fp32 sums.  gemm_splitk_reduce_*: slabs to add; a is then the workspace
+                            // ksplit x M x ldws fp32 sums.  gemm_splitk_reduce_*: slabs to add; a is then the workspace
+  int64_t ldws;             // leading stride of a slab of that workspace in floats: N rounded up to a multiple of 8
   unsigned long long *probe; // diagnostic: workgroup 0 stores {core-clock cycles, 100 MHz ticks} of its run, or null
 };

@@ -241,7 +241,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // the ring 80 KiB and two workgroups share a CU
   constexpr int B_OFF = ALLQ ? 4096 : A_BYTES;
   static_assert(MB == 4 || ((MB == 2 || (MB == 1 && QUARTERS)) && SPLIT_TAIL), "part tiles exist for the tail passes only");
-  static_assert(!SPLITK || (RAGGED && !TILED && EPI == EPI_NONE && !STREAM), "slices of K: row-major, clamping");
+  static_assert(!SPLITK || (RAGGED && EPI == EPI_NONE && !STREAM), "slices of K: the clamping kernels");
   const int gK = SPLITK ? g.K / g.ksplit : g.K;      // the K of one work item
   // TILED && RAGGED: the buffers are padded to whole 32x32 tiles (zeros), so "the matrix" the fetches are clamped
   // into is the padded one and K needs no more than whole turns of the ring; the stores are clipped at the
@@ -276,7 +276,7 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   // row-major:  A(m,k) at m*lda + k,  B(k,n) at k*ldb + n
   // tile-major: A(m,k) at ((m/32)*ntk + k/32)*1024 + (m%32)*32 + k%32,
   //             B(k,n) at ((k/32)*ntn + n/32)*1024 + (k%32)*32 + n%32          (elements)
-  const int64_t ntk = Kf / 32, ntn = Nf / 32;
+  const int64_t ntk = (SPLITK ? (g.K + 31) / 32 : Kf / 32), ntn = Nf / 32;   // (tiles per tile row of the buffers: of all of K)
   const uint32_t a_voff = TILED ? (uint32_t)((((int64_t)(a_row >> 5) * ntk << 10) + (a_row & 31) * 32 + a_chunk * 8) * 2)
                                 : (uint32_t)(((int64_t)a_row * g.lda + a_chunk * 8) * 2); // bytes, per thread
   const uint32_t b_voff = TILED ? (uint32_t)((((b_chunk >> 2) << 10) + b_kk * 32 + (b_chunk & 3) * 8) * 2)
@@ -448,9 +448,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if (RAGGED && MB < 4 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
-    if constexpr (SPLITK) {
-      ap += (int64_t)slice * gK * 2;
-      bp += (int64_t)slice * gK * g.ldb * 2;
+    if constexpr (SPLITK) {      // the slice's first k: gK / 32 steps further on
+      ap += (int64_t)slice * (gK / 32) * a_kstep;
+      bp += (int64_t)slice * (gK / 32) * b_kstep;
     }
     if (RAGGED || offsets) {
       // per-thread offsets of the tile's copies from ap / bp, one per A slab (RAGGED: rows and column chunks
@@ -778,14 +778,14 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     const int64_t m = m0 + wm * (32 * MB) + i16;
     if constexpr (SPLITK) {
       // the slice's sums as they are: a lane's four columns of a row are sixteen contiguous bytes of the slab
-      float *slab = (float *)g.c + (int64_t)slice * g.M * g.N;
+      float *slab = (float *)g.c + (int64_t)slice * g.M * g.ldws;
 #pragma unroll
       for (int i = 0; i < NA; ++i) {
         const int64_t mi = m + i * 16;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int64_t n = n0 + wn * 128 + j * 16 + G4 * 4;
-          if (mi < g.M && n < g.N) *(f32x4 *)(slab + mi * g.N + n) = acc[i][j];   // (N is a multiple of 8)
+          if (mi < g.M && n < g.N) *(f32x4 *)(slab + mi * g.ldws + n) = acc[i][j];   // (ldws is a multiple of 8)
         }
       }
       continue;
@@ -931,6 +931,12 @@ GEMM_TILE_RAGGED_ALL_EPI(gemm_ragged_f16, DT_F16, DT_F16)
   }
 GEMM_SPLITK(gemm_splitk_bf16, DT_BF16)
 GEMM_SPLITK(gemm_splitk_f16, DT_F16)
+// the same on the tile-major buffers of matmul_kernel (the workspace is row-major all the same)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_splitk_tiled_f16(GemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[4][20480];
+  fast::Ring ring = {{lds[0], lds[1], lds[2], lds[3]}};
+  fast::body<DT_F16, DT_F16, EPI_NONE, true, true, 1, true, true, false, true, true>(g, ring);
+}
 
 // matmul_kernel on tile-major fp16 buffers, plain and with leaky_relu
 #define GEMM_TILED(name, EPI)                                                                      \

@@ -89,6 +89,36 @@ int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
   return (saved_us > cost_us || env_int("TTAMD_GEMM_KSPLIT", 0)) ? s : 1;
 }
 
+// The pair of launches of a matmul computed in slices of K, or kNoWorkspace when the stream is recording or the
+// workspace cannot be had (the caller then launches in one pass).
+constexpr int kNoWorkspace = -12345;
+int launch_in_slices(const GemmArgs &g, int ksplit, int64_t tiles, int64_t live_rows, const char *slices_kernel,
+                     const char *sum_kernel, void *stream) {
+  // From the lookup of the workspace to the second launch nothing of another thread's comes between: two threads
+  // that feed one stream would otherwise interleave their pairs (the second's slices landing under the first's
+  // sums), or one would grow the workspace, which frees the old one, between the other's lookup and launches.
+  static std::mutex pair_mu;
+  std::lock_guard<std::mutex> pair(pair_mu);
+  const int64_t ldws = cdiv64(g.N, 8) * 8;
+  void *ws = splitk_workspace(stream, (int64_t)ksplit * g.M * ldws * 4);
+  if (!ws) return kNoWorkspace;
+  GemmArgs part = g, sum = g;
+  part.c = ws;
+  part.ksplit = sum.ksplit = ksplit;
+  part.ldws = sum.ldws = ldws;
+  part.epi = TT_EPI_NONE;
+  void *pargs[] = {&part};
+  // every tile as its live quarters; the kernel fits two workgroups on a CU
+  const uint32_t pwgs = (uint32_t)std::min<int64_t>(live_parts(live_rows, 64) * tiles * ksplit, 2 * (int64_t)props()->multiprocessor_count);
+  const int lrc = launch("gemm", slices_kernel, dim3(pwgs), dim3(256), 0, stream, pargs, 1);
+  if (lrc) return lrc;
+  sum.a = ws;
+  void *sargs[] = {&sum};
+  const int64_t groups = (int64_t)g.M * (ldws / 8);
+  const uint32_t swgs = (uint32_t)std::min<int64_t>(cdiv64(groups, 256), (int64_t)props()->multiprocessor_count * 8);
+  return launch("gemm", sum_kernel, dim3(swgs), dim3(256), 0, stream, sargs, 1);
+}
+
 int check_desc(const char *who, const char *what, const tt_desc2d *d, int64_t rows, int64_t cols) {
   if (!d) return fail(RT_ERR_INVALID, "%s: null %s descriptor", who, what);
   if (!d->base) return fail(RT_ERR_INVALID, "%s: %s descriptor has a null base", who, what);
@@ -203,29 +233,9 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
     const int64_t live_rows = M <= 256 ? M : 256;      // of a tile, where the matrix is a single row of tiles
     const int ksplit = pick_ksplit(tiles, live_parts(live_rows, 64), M, N, K);
     if (ksplit > 1) {
-      // From the lookup of the workspace to the second launch nothing of another thread's comes between: two threads
-      // that feed one stream would otherwise interleave their pairs (the second's slices landing under the first's
-      // sums), or one would grow the workspace, which frees the old one, between the other's lookup and launches.
-      static std::mutex pair_mu;
-      std::lock_guard<std::mutex> pair(pair_mu);
-      if (void *ws = splitk_workspace(stream, (int64_t)ksplit * M * N * 4)) {
-        GemmArgs part = g, sum = g;
-        part.c = ws;
-        part.ksplit = ksplit;
-        part.epi = TT_EPI_NONE;
-        void *pargs[] = {&part};
-        // every tile as its live quarters, two workgroups per CU
-        const uint32_t pwgs = (uint32_t)std::min<int64_t>(live_parts(live_rows, 64) * tiles * ksplit, 2 * (int64_t)props()->multiprocessor_count);
-        int lrc = launch("gemm", in == TT_BF16 ? "gemm_splitk_bf16" : "gemm_splitk_f16", dim3(pwgs), dim3(256), 0, stream, pargs, 1);
-        if (lrc) return lrc;
-        sum.a = ws;
-        sum.ksplit = ksplit;
-        void *sargs[] = {&sum};
-        const int64_t groups = (int64_t)M * (N / 8);
-        const uint32_t swgs = (uint32_t)std::min<int64_t>(cdiv64(groups, 256), (int64_t)props()->multiprocessor_count * 8);
-        return launch("gemm", out == TT_BF16 ? "gemm_splitk_reduce_bf16" : "gemm_splitk_reduce_f16", dim3(swgs), dim3(256), 0,
-                      stream, sargs, 1);
-      }
+      const int lrc = launch_in_slices(g, ksplit, tiles, live_rows, in == TT_BF16 ? "gemm_splitk_bf16" : "gemm_splitk_f16",
+                                       out == TT_BF16 ? "gemm_splitk_reduce_bf16" : "gemm_splitk_reduce_f16", stream);
+      if (lrc != kNoWorkspace) return lrc;
     }
     const uint32_t wgs = persistent_grid(tiles, true, true, fast_shape ? 256 : live_rows);
     // Diagnostic (TTAMD_GEMM_CLOCK_PROBE=1): workgroup 0 reports its core-clock cycles and
@@ -378,7 +388,14 @@ int tt_matmul_kernel(const void *a_ptr, const void *b_ptr, void *c_ptr, int32_t 
       aligned16(b_ptr) && aligned16(c_ptr) && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const bool whole = M % 256 == 0 && N % 256 == 0 && K % 128 == 0 && K >= 128;
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
-    const uint32_t wgs = persistent_grid(tiles, true);
+    // few tiles under a long K: in slices of K, as for the row-major kernels
+    const int64_t live_rows = M <= 256 ? M : 256;
+    const int ksplit = pick_ksplit(tiles, live_parts(live_rows, 64), M, cdiv64(N, 8) * 8, K);
+    if (ksplit > 1) {
+      const int lrc = launch_in_slices(g, ksplit, tiles, live_rows, "gemm_splitk_tiled_f16", "gemm_splitk_reduce_f16", stream);
+      if (lrc != kNoWorkspace) return lrc;
+    }
+    const uint32_t wgs = persistent_grid(tiles, true, false, whole ? 256 : live_rows);
     char name[48];
     snprintf(name, sizeof(name), "gemm_tiled%s_f16_epi%d", whole ? "" : "ragged", leaky_relu ? 3 : 0);
     return launch("gemm", name, dim3(wgs), dim3(256), 0, stream, args, 1);
