@@ -205,6 +205,27 @@ def test_fp8_scaled_ragged_fast_path(M, N, K_):
     assert close_bf16(decode(c), ref, RTOL, fp8_atol(ref))
 
 
+@pytest.mark.parametrize("M,N,K_", [(100, 336, 4096), (16, 512, 4096), (300, 208, 3072), (256, 256, 4096), (130, 1024, 8192)])
+def test_fp8_scaled_k_slices(M, N, K_):
+    """fp8 launches of few tiles under a long K (a multiple of 512) run in slices of K too: half tiles as parts, the
+    same workspace and adding kernel, the scales applied to the whole sum.  Operands are views into buffers whose
+    surroundings are NaN codes; two launches give the same bits."""
+    g = torch.Generator().manual_seed(M + K_)
+    qa, sa = K.quantize_fp8(torch.randn(M, K_, generator=g))
+    qb, sb = K.quantize_fp8(torch.randn(K_, N, generator=g))
+    abuf = torch.full((M + 2, K_ + 16), 0x7f, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    bbuf = torch.full((K_ + 2, N + 16), 0x7f, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    abuf[:M, :K_] = qa
+    bbuf[:K_, :N] = qb
+    a, b = abuf.cuda()[:M, :K_], bbuf.cuda()[:K_, :N]
+    c = K.matmul_fp8_scaled(a, b, sa, sb)
+    assert rt.last_kernel_name() == "gemm_splitk_reduce_bf16"
+    ref = orc.from_bf16(orc.matmul(bits(qa), bits(qb), in_dt=orc.FP8E4M3, out_dt=orc.BF16,
+                                   scale=float(np.float32(sa) * np.float32(sb)), acc64=True))
+    assert close_bf16(decode(c), ref, RTOL, fp8_atol(ref))
+    assert torch.equal(K.matmul_fp8_scaled(a, b, sa, sb), c)
+
+
 def test_matmul_partial_grid_runs_only_its_programs():
     a, b = _ab(256, 256, 128)
     c = torch.full((256, 256), 7.5, dtype=torch.bfloat16, device="cuda")

@@ -135,12 +135,13 @@ struct PassItems {
   int tail_tiles;
   int parts;       // MB < 4: live parts of a tile (halves: 1..2, quarters: 1..4)
 };
-// ALLQ: every tile is finished as quarters (the kernels of the K slices, whose launches have no whole round).
+// ALLQ: every tile is finished as its live quarters, or halves (the kernels of the K slices, whose launches have no
+// whole round).
 template <int MB, bool SPLIT_TAIL, bool QUARTERS = false, bool ALLQ = false>
 __device__ __forceinline__ PassItems pass_items(int total_tiles, int live_rows) {
   PassItems p = {total_tiles, 0, 0, 1};
-  if constexpr (ALLQ) {
-    p.parts = (live_rows + 63) >> 6;
+  if constexpr (ALLQ) {      // (the fp8 kernels' smallest part is the half)
+    p.parts = MB == 2 ? (live_rows + 127) >> 7 : (live_rows + 63) >> 6;
     p.total = p.parts * total_tiles;
     p.tail_tiles = total_tiles;
   } else if constexpr (SPLIT_TAIL) {

@@ -44,15 +44,22 @@ typedef __attribute__((address_space(3))) void lds_void;
 // operands on its way through: 16384 x 16384 x 1024 runs 28 % faster with streaming stores and x 4096 8.6 %, x 8192
 // the same; 8192^3, whose C fits, slower).  The variants are kernels of their own: the two forms of the epilogue
 // inside one kernel cost the benchmark shapes 1-2 %.
-template <int OUT_DT, bool RAGGED = false, int MB = 4, bool STREAM = false>
+// SPLITK (the clamping half-tile pass alone): K in g.ksplit equal slices, work item = (slice, tile, live half), the
+// slice's fp32 sums into slab `slice` of the workspace at g.c; gemm_splitk_reduce_* adds the slabs, scales and rounds
+// (see the 16-bit kernel).
+template <int OUT_DT, bool RAGGED = false, int MB = 4, bool STREAM = false, bool SPLITK = false>
 __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) {
+  static_assert(!SPLITK || (RAGGED && MB == 2 && !STREAM), "slices of K: the clamping half-tile pass");
+  const int gK = SPLITK ? g.K / g.ksplit : g.K;      // the K of one work item
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = RAGGED ? (g.M + BM - 1) / BM : g.M / BM, tiles_n = RAGGED ? (g.N + BN - 1) / BN : g.N / BN;
-  const fast::PassItems items = fast::pass_items<MB, true>(tiles_m * tiles_n, fast::BM);
+  const int tiles_mv = SPLITK ? tiles_m * g.ksplit : tiles_m;   // SPLITK: row tm + tiles_m * s of the item grid is slice s of tile row tm
+  const fast::PassItems items =
+      fast::pass_items<MB, true, false, SPLITK>(tiles_mv * tiles_n, (SPLITK && tiles_m == 1) ? g.M : fast::BM);
   const int total = items.total;
-  const int nk_real = g.K / BK;                                   // steps that carry data
+  const int nk_real = gK / BK;                                   // steps that carry data
   const int nk = RAGGED ? (nk_real + R - 1) / R * R : nk_real;    // steps per tile, a multiple of R
 
   // ---- global -> LDS: thread t writes byte 16*t of each 4 KiB slab ----
@@ -145,13 +152,18 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   // (whole tiles: the offsets are the same for every tile, so only the first call works them out)
   auto tile_bases = [&](int t, const uint8_t *&ap, const uint8_t *&bp, Voffs &vo, bool offsets = RAGGED) {
     int tm, tn, half;
-    fast::item_tile<MB>(items, min(t, total - 1), tiles_m, tiles_n, tm, tn, half);
+    fast::item_tile<MB>(items, min(t, total - 1), tiles_mv, tiles_n, tm, tn, half);
+    int slice = 0;
+    if constexpr (SPLITK) {
+      slice = tm / tiles_m;
+      tm -= slice * tiles_m;
+    }
     int64_t row0 = (int64_t)tm * BM + half * 128;
     // RAGGED: a lower half that starts past the last row is pointed at the upper half's rows; its stores all
     // fall to the clipping
     if (RAGGED && MB == 2 && row0 >= g.M) row0 = (int64_t)tm * BM;
-    ap = A + row0 * g.lda;
-    bp = B + (int64_t)tn * BN;
+    ap = A + row0 * g.lda + (int64_t)slice * gK;
+    bp = B + (int64_t)tn * BN + (int64_t)slice * gK * g.ldb;
     if (RAGGED || offsets) {
       const int last_row = RAGGED ? g.M - 1 - (int)row0 : BM;
       vo.last_row = last_row;
@@ -352,7 +364,12 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
 
   for (; t < total; t += gridDim.x) {
     int tm, tn, half;
-    fast::item_tile<MB>(items, t, tiles_m, tiles_n, tm, tn, half);
+    fast::item_tile<MB>(items, t, tiles_mv, tiles_n, tm, tn, half);
+    int slice = 0;
+    if constexpr (SPLITK) {
+      slice = tm / tiles_m;
+      tm -= slice * tiles_m;
+    }
     const int64_t m0 = (int64_t)tm * BM + half * 128, n0 = (int64_t)tn * BN;
 #pragma unroll
     for (int i = 0; i < MB; ++i)
@@ -401,7 +418,17 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
       const int64_t mi = m + i * 32;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if constexpr (OUT_DT == DT_FP8) {
+        if constexpr (SPLITK) {
+          // the slice's sums as they are: four columns of a row are sixteen contiguous bytes of the slab
+          float *slab = (float *)g.c + (int64_t)slice * g.M * g.ldws;
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
+            if (mi >= g.M || n >= g.N) continue;
+            *(f32x4 *)(slab + mi * g.ldws + n) =
+                (f32x4){acc[i][j][r4 * 4], acc[i][j][r4 * 4 + 1], acc[i][j][r4 * 4 + 2], acc[i][j][r4 * 4 + 3]};
+          }
+        } else if constexpr (OUT_DT == DT_FP8) {
 #pragma unroll
           for (int r4 = 0; r4 < 4; ++r4) {
             const int64_t n = n0 + wn * 128 + j * 32 + r4 * 8 + hi * 4;
@@ -500,5 +527,15 @@ GEMM_RAGGED_FP8(gemm_ragged_fp8_f16, DT_F16, false)
 GEMM_RAGGED_FP8(gemm_ragged_fp8_fp8, DT_FP8, false)
 GEMM_RAGGED_FP8(gemm_ragged_fp8_bf16_stream, DT_BF16, true)
 GEMM_RAGGED_FP8(gemm_ragged_fp8_f16_stream, DT_F16, true)
+
+// few tiles under a long K: slices of K as work items (see SPLITK in body), fp32 sums into the workspace
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_splitk_fp8(GemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds0[fast8::STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds1[fast8::STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds2[fast8::STAGE];
+  __shared__ __attribute__((aligned(1024))) uint8_t lds3[fast8::STAGE];
+  fast::Ring ring = {{lds0, lds1, lds2, lds3}};
+  fast8::body<DT_BF16, true, 2, false, true>(g, ring);
+}
 
 } // extern "C"

@@ -75,16 +75,18 @@ void *splitk_workspace(void *stream, int64_t bytes) {
 // 53 us with 4, 8 and 16 slices), keeps every slice at sixteen steps or more and the workspace within bounds.  What it costs is one more launch and a pass over ksplit x M x N floats in
 // each direction (taken at 6 us, the adding kernel alone runs 4-5, and 4 TB/s); what it saves is (1 - 1/ksplit) of K/32 quarter-tile steps of about
 // 0.235 us.
-int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
+// (`bk`: K of a step, 32 for the 16-bit kernels and 64 for fp8, whose part is the half tile; `step_us`: what a
+// step of such a part takes)
+int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K, int64_t bk = 32, double step_us = 0.235) {
   const int64_t cus = props()->multiprocessor_count;
   if (env_int("TTAMD_GEMM_NO_SPLITK", 0) || 2 * parts * tiles > cus) return 1;
   int s = 1;
-  while (s < 16 && 2 * s * parts * tiles <= cus && K % (2 * s * 128) == 0 && K / (2 * s) >= 512 &&
+  while (s < 16 && 2 * s * parts * tiles <= cus && K % (2 * s * 4 * bk) == 0 && K / (2 * s) >= 16 * bk &&
          2 * s * M * N * 4 <= kSplitKMaxBytes)
     s *= 2;
-  if (const int forced = env_int("TTAMD_GEMM_KSPLIT", 0)) s = (K % (forced * 128) == 0 && (int64_t)forced * M * N * 4 <= kSplitKMaxBytes) ? forced : 1;
+  if (const int forced = env_int("TTAMD_GEMM_KSPLIT", 0)) s = (K % (forced * 4 * bk) == 0 && (int64_t)forced * M * N * 4 <= kSplitKMaxBytes) ? forced : 1;
   if (s == 1) return 1;
-  const double saved_us = (double)(K / 32) * (1.0 - 1.0 / s) * 0.235;
+  const double saved_us = (double)(K / bk) * (1.0 - 1.0 / s) * step_us;
   const double cost_us = 6.0 + (double)s * M * N * 8 / 4.0e6;
   return (saved_us > cost_us || env_int("TTAMD_GEMM_KSPLIT", 0)) ? s : 1;
 }
@@ -93,7 +95,7 @@ int pick_ksplit(int64_t tiles, int64_t parts, int64_t M, int64_t N, int64_t K) {
 // workspace cannot be had (the caller then launches in one pass).
 constexpr int kNoWorkspace = -12345;
 int launch_in_slices(const GemmArgs &g, int ksplit, int64_t tiles, int64_t live_rows, const char *slices_kernel,
-                     const char *sum_kernel, void *stream) {
+                     const char *sum_kernel, void *stream, int64_t rows_per_part = 64) {
   // From the lookup of the workspace to the second launch nothing of another thread's comes between: two threads
   // that feed one stream would otherwise interleave their pairs (the second's slices landing under the first's
   // sums), or one would grow the workspace, which frees the old one, between the other's lookup and launches.
@@ -108,8 +110,9 @@ int launch_in_slices(const GemmArgs &g, int ksplit, int64_t tiles, int64_t live_
   part.ldws = sum.ldws = ldws;
   part.epi = TT_EPI_NONE;
   void *pargs[] = {&part};
-  // every tile as its live quarters; the kernel fits two workgroups on a CU
-  const uint32_t pwgs = (uint32_t)std::min<int64_t>(live_parts(live_rows, 64) * tiles * ksplit, 2 * (int64_t)props()->multiprocessor_count);
+  // every tile as its live quarters (fp8: halves); the 16-bit kernels fit two workgroups on a CU
+  const uint32_t pwgs = (uint32_t)std::min<int64_t>(live_parts(live_rows, rows_per_part) * tiles * ksplit,
+                                                    (rows_per_part == 64 ? 2 : 1) * (int64_t)props()->multiprocessor_count);
   const int lrc = launch("gemm", slices_kernel, dim3(pwgs), dim3(256), 0, stream, pargs, 1);
   if (lrc) return lrc;
   sum.a = ws;
@@ -270,6 +273,15 @@ int run_matmul(const char *who, const tt_desc2d *a, const tt_desc2d *b, const tt
   const bool fp8_ragged = !fp8_shape && N % 16 == 0 && K % 64 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24);
   if (full_grid && fp8_io && (fp8_shape || fp8_ragged) && fp8_align && !nan_shows && !env_int("TTAMD_GEMM_FORCE_ANY", 0)) {
     const int64_t tiles = cdiv64(M, 256) * cdiv64(N, 256);
+    // few tiles under a long K: in slices of K, as for the 16-bit kernels; the part is the half tile here, whose step
+    // of K = 64 takes 8 MFMAs of 64 cycles
+    const int64_t live_rows8 = M <= 256 ? M : 256;
+    const int ksplit8 = out == TT_FP8E4M3 ? 1 : pick_ksplit(tiles, live_parts(live_rows8, 128), M, N, K, 64, 0.3);
+    if (ksplit8 > 1) {
+      const int lrc = launch_in_slices(g, ksplit8, tiles, live_rows8, "gemm_splitk_fp8",
+                                       out == TT_BF16 ? "gemm_splitk_reduce_bf16" : "gemm_splitk_reduce_f16", stream, 128);
+      if (lrc != kNoWorkspace) return lrc;
+    }
     const uint32_t wgs = persistent_grid(tiles, true);
     void *fargs[] = {&g};
     char fp8_name[64];
