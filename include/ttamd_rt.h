@@ -276,7 +276,7 @@ TTAMD_API int tt_reduce1d_kernel_noalloc(int32_t op, const void *x, void *z, int
  * round-to-nearest-even cast to c->dtype.  grid[0] logical programs, one per
  * BLOCK_SIZE_M x BLOCK_SIZE_N tile in GROUP_SIZE_M-swizzled order.
  * A launch with a 16-bit result (this entry point, _fused, _fp8_scaled and tt_matmul_kernel) whose C has few 256x256 tiles under a long K (at most half the CUs
- * busy even with 64-row pieces of tiles, K a multiple of 256) is computed in slices of K: the slices' fp32 sums pass
+ * busy even with 64-row pieces of tiles, K a multiple of 256, of 512 for fp8) is computed in slices of K: the slices' fp32 sums pass
  * through a workspace of at most 64 MiB that the library keeps per (device, stream), allocated by the first such
  * call on the stream (hipMalloc), grown by a call that needs more (the stream is drained first) and freed by
  * rt_release_stream; the sums are added in slice order, so results do not change from launch to launch, and the
