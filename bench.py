@@ -447,6 +447,18 @@ def main() -> int:
         extra["gemm_fp8_8192"]["parity_rows_ok"] = ok
         parity_failed |= not ok
         del qa, qb, c, ref
+        # few output tiles under a long K, in slices of K: bounded by the one pass over B (one byte an element)
+        skinny8 = {}
+        for (m_, n_, k_) in ((16, 8192, 8192), (128, 8192, 8192)):
+            qa, sa = K.quantize_fp8(torch.randn(m_, k_, device="cuda"))
+            qb, sb = K.quantize_fp8(torch.randn(k_, n_, device="cuda"))
+            avg_ms, per, _ = _events_time(lambda: K.matmul_fp8_scaled(qa, qb, sa, sb), max(3, steps // 4), 2, stream)
+            byts = 1.0 * (m_ * k_ + k_ * n_) + 2.0 * m_ * n_
+            skinny8[f"{m_}x{n_}x{k_}"] = {"kernel": rt.last_kernel_name(), "us": round(avg_ms * 1e3, 1),
+                                          "GBs": round(byts / (avg_ms * 1e-3) / 1e9, 0),
+                                          "frac_of_hbm_peak": round(byts / (avg_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 3)}
+            del qa, qb
+        extra["gemm_fp8_few_tiles_long_k"] = skinny8
     if want("tiled"):
         # the pointer-based matmul_kernel on tile-major fp16 buffers, 32x32x32 tiles, same 8192^3 problem
         at = K.tilize((torch.randn(M, Kd, device="cuda") / math.sqrt(Kd)).to(torch.float16), 32, 32)
