@@ -55,6 +55,24 @@ def test_random_shapes_in_sequence(seed):
         seen.add(rt.last_kernel_name())
         ref = a.double() @ b.double()
         assert _close(c, ref), ("few tiles", i, dt, M, N, Kd, rt.last_kernel_name(), float((c.double() - ref).abs().max()))
+        # the same for fp8 and for the tile-major kernel
+        M, N, Kd = rnd.choice([rdim(1, 300), rdim(1, 1100)]), rdim(16, 2048, 16), rdim(2048, 8192, 512)
+        aq, sa = K.quantize_fp8(torch.randn(M, Kd, device="cuda"))
+        bq, sb = K.quantize_fp8(torch.randn(Kd, N, device="cuda"))
+        c = K.matmul_fp8_scaled(aq, bq, sa, sb)
+        seen.add(rt.last_kernel_name())
+        ref = (aq.double() @ bq.double()) * (sa * sb)
+        assert _close(c, ref, 1e-2, 1e-3 * math.sqrt(Kd)), ("fp8 few tiles", i, M, N, Kd, rt.last_kernel_name())
+        M, N, Kd = rnd.choice([rdim(1, 300), rdim(1, 1100)]), rdim(1, 1500), rdim(1024, 6144, 256)
+        a = (torch.randn(M, Kd, device="cuda") / math.sqrt(Kd)).to(torch.float16)
+        b = torch.randn(Kd, N, device="cuda").to(torch.float16)
+        act = rnd.choice(["", "leaky_relu"])
+        ct = K.matmul_tiled(K.tilize(a, 32, 32), K.tilize(b, 32, 32), M, N, Kd, activation=act)
+        seen.add(rt.last_kernel_name())
+        ref = a.double() @ b.double()
+        if act:
+            ref = torch.where(ref >= 0, ref, 0.01 * ref)
+        assert _close(K.untilize(ct, M, N, 32, 32), ref, 1e-2, 2e-3), ("tile-major few tiles", i, M, N, Kd, act, rt.last_kernel_name())
         # fp8 with scales
         M, N, Kd = rdim(1, 1200), rdim(16, 1300, 16), rdim(64, 1500, 64)
         if rnd.random() < 0.3:
@@ -93,5 +111,5 @@ def test_random_shapes_in_sequence(seed):
         assert int(K.reduce1d("argmax", xr)) == int(xr.argmax()), ("argmax", i, xr.numel())
         assert abs(float(K.reduce1d("sum", xr)) - float(xr.double().sum())) <= 1e-5 * float(xr.double().abs().sum()) + 1e-6
     # the sweep reached the hand-scheduled kernels it is meant for
-    for name in ("gemm_splitk_reduce_bf16", "gemm_ragged_bf16_epi0", "attn_ragged_d256", "attn_tile_d128"):
+    for name in ("gemm_splitk_reduce_bf16", "gemm_splitk_reduce_f16", "gemm_ragged_bf16_epi0", "attn_ragged_d256", "attn_tile_d128"):
         assert name in seen, (name, sorted(seen))
