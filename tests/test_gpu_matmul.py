@@ -766,6 +766,14 @@ def test_repeat_launches_take_the_cached_path_and_keep_the_checks():
     assert torch.equal(K.matmul_tma(abuf[:, :K_], b), want)
     assert torch.equal(K.matmul_tma(a[:1], b), want[:1])
     assert torch.equal(K.matmul_tma(a, b), want)
+    # a dimension of 1 is another specialisation (Triton folds the value): it gets a closure of its own, which serves
+    # the launches that have the 1 in the same places and hands every other one back to the full path
+    plans = []
+    for rows in (1, 1, 1, 40, 1, 1):
+        assert torch.equal(K.matmul_tma(a[:rows], b), want[:rows])
+        plans.append(K.matmul_kernel_tma._plan[3])
+    assert plans[1] is plans[2] and plans[4] is plans[5] and plans[3] is not plans[2]
+    assert torch.equal(K.matmul_tma(a, b[:, :8])[:, :1], want[:, :1])
     # and the same refusals
     c.fill_(7.5)
     with pytest.raises(ValueError):

@@ -236,25 +236,27 @@ def _streaming_direct(fn, n_tensors: int, dtype, tail: tuple, per_program: int):
     return direct
 
 
-def _desc_matmul_direct(fn, bases: list, n_floats: int, tail: tuple):
+def _desc_matmul_direct(fn, bases: list, n_floats: int, tail: tuple, mnk: tuple = (0, 0, 0)):
     """Repeat-launch closure of the descriptor matmuls (see ``_streaming_direct``): the launch arguments are
     ``len(dtypes)`` rank-2 descriptors, then M, N, K, then ``n_floats`` floats.  The closure re-checks what selects
-    the specialisation it was built under (descriptor class, rank, base dtype and device, integer M, N, K that Triton
-    would not fold) and fills the calling thread's own ``tt_desc2d`` blocks, which the library reads during the call
+    the specialisation it was built under (descriptor class, rank, base dtype and device, integer M, N, K of which
+    those that were 1 at the launch that built this, ``mnk``, are 1 again and the others are not: Triton folds the value
+    1 into the specialisation, so a launch that differs there belongs to another launcher) and fills the calling thread's own ``tt_desc2d`` blocks, which the library reads during the call
     only; shapes, strides, alignment and the grid are validated by the library as on the ordinary path."""
     from ..tensor_descriptor import TensorDescriptor
     dtypes = tuple(t.dtype for t in bases)      # of the descriptors' base tensors at the launch that built this
     tensor_type, grid3, check, n_desc = _tensor_type(), rt.Grid3, rt.check, len(dtypes)
     my_blocks = _desc_blocks_per_thread(tuple(_torch_dtype_code(t) for t in bases))
     n_args = n_desc + 3 + n_floats
+    folded = tuple(v == 1 for v in mnk)
 
     def direct(args, grid, stream):
         if len(args) != n_args or len(grid) != 1 or type(grid[0]) is not int:
             return False
         M, N, K = args[n_desc], args[n_desc + 1], args[n_desc + 2]
-        if (type(M) is not int or type(N) is not int or type(K) is not int or not 1 < M < 2147483648
-                or not 1 < N < 2147483648 or not 1 < K < 2147483648):
-            return False
+        for v, one in zip((M, N, K), folded):
+            if type(v) is not int or not 0 < v < 2147483648 or (v == 1) is not one:
+                return False
         blocks, refs = my_blocks()
         for blk, d, dt in zip(blocks, args, dtypes):
             if type(d) is not TensorDescriptor:
@@ -527,12 +529,12 @@ def _bind_matmul_tma(lib, cur, consts, grid, stream):
         sa, sb = float(cur.scalar("scale_a")), float(cur.scalar("scale_b"))
         cur.done()
         if with_mnk:
-            cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_tma_fp8_scaled, bases, 2, (bm, bn, bk, g))
+            cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_tma_fp8_scaled, bases, 2, (bm, bn, bk, g), (M, N, K))
         return lib.tt_matmul_kernel_tma_fp8_scaled(C.byref(a), C.byref(b), C.byref(c), M, N, K, sa, sb, bm, bn, bk,
                                                    g, grid, stream)
     cur.done()
     if with_mnk:
-        cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_tma, bases, 0, (bm, bn, bk, g))
+        cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_tma, bases, 0, (bm, bn, bk, g), (M, N, K))
     return lib.tt_matmul_kernel_tma(C.byref(a), C.byref(b), C.byref(c), M, N, K, bm, bn, bk, g, grid, stream)
 
 
@@ -554,7 +556,7 @@ def _bind_matmul_fused(lib, cur, consts, grid, stream):
     # (the epilogue chosen from the bias's shape and dtype holds for repeat launches only while those stay as they
     # are: the closure is offered for the named epilogues, which do not look at the bias)
     if _EPILOGUES.get(consts.get("EPILOGUE")) is not None and "M" in cur.arg_names:
-        cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_fused, cur.keep[-4:], 0, (bm, bn, bk, g, epi))
+        cur.direct = _desc_matmul_direct(lib.tt_matmul_kernel_fused, cur.keep[-4:], 0, (bm, bn, bk, g, epi), (M, N, K))
     return lib.tt_matmul_kernel_fused(C.byref(a), C.byref(b), C.byref(c), C.byref(bias), M, N, K, bm, bn, bk, g, epi,
                                       grid, stream)
 
