@@ -230,7 +230,7 @@ struct Ring {
 // one kernel, several instantiations spilled copy offsets whose reloads the compiler then waits for inside the K
 // loop, with every copy in flight counted in (tile-major 8192^3: 1585 -> 1482 TFLOP/s).
 //
-// SPLITK: K is cut into g.ksplit equal slices (whole steps each) and a work item is one slice of one macro tile;
+// SPLITK: K is dealt to g.ksplit slices of equal size, a step at a time, and a work item is one slice of one macro tile;
 // slice s of tile (tm, tn) leaves its fp32 sums, nothing applied, in slab s of a workspace of ksplit x M x N floats
 // that g.c points at, and gemm_splitk_reduce adds the slabs in slice order and does the rest.  For a C of few macro
 // tiles under a long K: 128 x 8192 x 8192 has 32 tiles for 256 CUs, each streaming all of K on its own.
@@ -285,8 +285,11 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
   const int64_t a_slab = TILED ? 2 * ntk * 2048 : 64 * g.lda * 2;                  // bytes, uniform
   const int64_t b_rows4 = TILED ? 4 * 32 * 2 : 4 * g.ldb * 2;                       // four k rows of B
   auto b_slab_off = [&](int i) { return ((i & 1) + 4 * (i >> 1)) * b_rows4; };      // slab i's first row, b_row0(i)
-  const int64_t a_kstep = TILED ? 2048 : BK * 2;
-  const int64_t b_kstep = TILED ? ntn * 2048 : (int64_t)BK * g.ldb * 2;
+  // (SPLITK: the slices are dealt step by step, slice s takes steps s, s + ksplit, ...: all slices then walk
+  // through neighbouring rows of B at any one time instead of through ksplit fronts K / ksplit rows apart)
+  const int64_t a_kstep1 = TILED ? 2048 : BK * 2;
+  const int64_t b_kstep1 = TILED ? ntn * 2048 : (int64_t)BK * g.ldb * 2;
+  const int64_t a_kstep = SPLITK ? a_kstep1 * g.ksplit : a_kstep1, b_kstep = SPLITK ? b_kstep1 * g.ksplit : b_kstep1;
   const int lds_wave = wave * 1024;
 
   // ---- LDS -> fragments ----
@@ -449,9 +452,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const Ring &ring) {
     if (RAGGED && MB < 4 && row0 >= Mf) row0 = (int64_t)tm * BM;
     ap = A + (TILED ? (row0 / 32) * ntk * 2048 : row0 * g.lda * 2);
     bp = B + (TILED ? (int64_t)tn * (BN / 32) * 2048 : (int64_t)tn * BN * 2);
-    if constexpr (SPLITK) {      // the slice's first k: gK / 32 steps further on
-      ap += (int64_t)slice * (gK / 32) * a_kstep;
-      bp += (int64_t)slice * (gK / 32) * b_kstep;
+    if constexpr (SPLITK) {      // the slice's first step
+      ap += (int64_t)slice * a_kstep1;
+      bp += (int64_t)slice * b_kstep1;
     }
     if (RAGGED || offsets) {
       // per-thread offsets of the tile's copies from ap / bp, one per A slab (RAGGED: rows and column chunks

@@ -72,7 +72,9 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
   const uint32_t a_voff = (uint32_t)((int64_t)a_row * g.lda + a_chunk * 16);
   const uint32_t b_voff = (uint32_t)((int64_t)b_k * g.ldb + b_chunk * 16);
   const int64_t a_slab = 64 * g.lda, b_slab = 16 * g.ldb;
-  const int64_t b_kstep = (int64_t)BK * g.ldb;
+  // (SPLITK: slice s takes steps s, s + ksplit, ..., as in the 16-bit kernel)
+  const int64_t a_kstep = SPLITK ? (int64_t)BK * g.ksplit : BK;
+  const int64_t b_kstep = (int64_t)BK * g.ldb * (SPLITK ? g.ksplit : 1);
   const int lds_wave = wave * 1024;
 
   // ---- LDS -> fragments ----
@@ -162,8 +164,8 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     // RAGGED: a lower half that starts past the last row is pointed at the upper half's rows; its stores all
     // fall to the clipping
     if (RAGGED && MB == 2 && row0 >= g.M) row0 = (int64_t)tm * BM;
-    ap = A + row0 * g.lda + (int64_t)slice * gK;
-    bp = B + (int64_t)tn * BN + (int64_t)slice * gK * g.ldb;
+    ap = A + row0 * g.lda + (int64_t)slice * BK;
+    bp = B + (int64_t)tn * BN + (int64_t)slice * BK * g.ldb;
     if (RAGGED || offsets) {
       const int last_row = RAGGED ? g.M - 1 - (int)row0 : BM;
       vo.last_row = last_row;
@@ -180,21 +182,21 @@ __device__ __forceinline__ void body(const GemmArgs &g, const fast::Ring &ring) 
     const int k = over ? kk - nk : kk;
     if constexpr (inner) {
       if (i < MB)
-        dma_one(a_cur + (int64_t)k * BK, vo_cur.a[i], stage + i * 4096);
+        dma_one(a_cur + (int64_t)k * a_kstep, vo_cur.a[i], stage + i * 4096);
       else
         dma_one(b_cur + (int64_t)k * b_kstep + (i - MB) * b_slab, vo_cur.b, stage + A_BYTES + (i - MB) * 4096);
     } else if constexpr (RAGGED) {
       const bool zero = k >= nk_real;
       const Voffs &vo = over ? vo_nxt : vo_cur;
       if (i < MB) {
-        const uint8_t *ap = zero ? fast::zero_page : (over ? a_nxt : a_cur) + (int64_t)k * BK;
+        const uint8_t *ap = zero ? fast::zero_page : (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
         dma_one(ap, zero ? z_voff : vo.a[i], stage + i * 4096);
       } else {
         const uint8_t *bp = zero ? fast::zero_page : (over ? b_nxt : b_cur) + (int64_t)k * b_kstep + (i - MB) * b_slab;
         dma_one(bp, zero ? z_voff : vo.b, stage + A_BYTES + (i - MB) * 4096);
       }
     } else if (i < MB) {
-      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * BK;
+      const uint8_t *ap = (over ? a_nxt : a_cur) + (int64_t)k * a_kstep;
       dma_one(ap + i * a_slab, a_voff, stage + i * 4096);
     } else {
       const uint8_t *bp = (over ? b_nxt : b_cur) + (int64_t)k * b_kstep;
