@@ -71,16 +71,16 @@ def _events_time(fn, steps: int, warmup: int, stream: int, tag: str | None = Non
 # dispatch, FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0: what the same counters read for the int32 add, a
 # plain copy-like kernel of known size).  Not measured live: the counters need the profiler around the process.
 # profiles/bench_all_kernels_rocprofv3.md holds the raw readings and the commands.
-TRAFFIC_FROM_COMMIT = "7ea29ab"   # the tree the readings below were taken from
-TRAFFIC_KERNELS_SHA = "92752577e13ee533"   # _kernel_sources_sha() of that tree: a kernel edit after the readings shows in the JSON
+TRAFFIC_FROM_COMMIT = "fddd240"   # the tree the readings below were taken from
+TRAFFIC_KERNELS_SHA = "7b15c66926959939"   # _kernel_sources_sha() of that tree: a kernel edit after the readings shows in the JSON
 MEASURED_TRAFFIC_BYTES = {
-    "gemm_tile_bf16_epi0": int((2 * 795543 + 134170) * 1024),
-    "gemm_tile_bf16_epi2": int((2 * 385356 + 117760) * 1024),
-    "gemm_tile_fp8_bf16": int((2 * 407704 + 157464) * 1024),
-    "gemm_tiled_f16_epi0": int((2 * 790344 + 132864) * 1024),
-    "attn_tile_d128": int((2 * 307474 + 133121) * 1024),     # the causal launches
+    "gemm_tile_bf16_epi0": int((2 * 795938 + 134110) * 1024),
+    "gemm_tile_bf16_epi2": int((2 * 385288 + 117760) * 1024),
+    "gemm_tile_fp8_bf16": int((2 * 407758 + 157285) * 1024),
+    "gemm_tiled_f16_epi0": int((2 * 790342 + 132864) * 1024),
+    "attn_tile_d128": int((2 * 306392 + 133123) * 1024),     # the causal launches
     "ew_add_i32": int((2 * 1048588 + 1048576) * 1024),
-    "ew_sin_f32": int((2 * 524332 + 1048577) * 1024),
+    "ew_sin_f32": int((2 * 524332 + 1048578) * 1024),
 }
 
 
