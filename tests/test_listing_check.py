@@ -72,12 +72,13 @@ def test_a_register_file_copy_right_in_front_of_the_mfma_that_reads_it_is_found(
     mfma = "\tv_mfma_f32_32x32x16_bf16 v[2:17], v[34:37], a[132:135], v[2:17]"
     mf = ["\t;;#ASMSTART", mfma, "\t;;#ASMEND"]
     padded = ["\t;;#ASMSTART", "\ts_nop 1", mfma, "\t;;#ASMEND"]
-    assert len(lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", *mf))) == 1
-    assert len(lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_accvgpr_write_b32 a133, v9", "\ts_nop 0", *mf))) == 1
-    assert lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", *padded)) == []
-    # other registers, other kinds of instruction (the hardware orders those), another block, the compiler's own MFMA
-    assert lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v38, a191", *mf)) == []
-    assert lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_cvt_pk_bf16_f32 v37, v1, v2", *mf)) == []
-    assert lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", ".LBB0_1:", *mf)) == []
-    assert lc.accvgpr_copies_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", mfma)) == []
+    assert len(lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", *mf))) == 1
+    assert len(lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_write_b32 a133, v9", "\ts_nop 0", *mf))) == 1
+    assert lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", *padded)) == []
+    # other registers, an operand that comes from LDS, another block, the compiler's own MFMA
+    assert lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v38, a191", *mf)) == []
+    assert len(lc.valu_writes_in_front_of_an_mfma(kernel("\tv_cvt_pk_bf16_f32 v37, v1, v2", *mf))) == 1
+    assert lc.valu_writes_in_front_of_an_mfma(kernel("\tds_read_b128 v[34:37], v5", "\ts_waitcnt lgkmcnt(0)", *mf)) == []
+    assert lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", ".LBB0_1:", *mf)) == []
+    assert lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", mfma)) == []
     assert list(lc.check_listing("\n".join(kernel("\tv_accvgpr_read_b32 v37, a191", *mf)))) == ["k"]

@@ -1,5 +1,5 @@
 """Static checks of a gfx950 assembly listing around MFMAs issued from inline assembly: nothing but another MFMA
-touches an MFMA's result too early, and no register-file copy lands right in front of the MFMA that reads it.
+touches an MFMA's result too early, and no vector ALU result lands right in front of the MFMA that reads it.
 
 The hot kernels issue their MFMAs from inline assembly (that is how the accumulators stay in AGPRs and a
 direct-to-LDS copy rides behind an MFMA).  The compiler does not look inside such a statement, so it does not know
@@ -127,12 +127,14 @@ def mfma_result_hazards(lines: list[str]) -> list[str]:
     return found
 
 
-def accvgpr_copies_in_front_of_an_mfma(lines: list[str], states: int = 2) -> list[str]:
-    """One message per v_accvgpr_read / _write / _mov whose result an MFMA reads fewer than `states` wait states later
-    (straight-line: such a copy sits in the MFMA's own block).  The compiler moves operands between the register
-    files where it likes, and in front of an inline-assembly MFMA it leaves no distance: the MFMA then read the
-    register before the copy had arrived (attention, head dim 256: scores off by a few per cent, exact with one idle
-    state in between; that kernel's MFMAs carry two)."""
+def valu_writes_in_front_of_an_mfma(lines: list[str], states: int = 2) -> list[str]:
+    """One message per vector ALU instruction (register-file copies v_accvgpr_read / _write / _mov above all) whose
+    result an inline-assembly MFMA reads fewer than `states` wait states later (straight-line: such an instruction
+    sits in the MFMA's own block).  The compiler moves operands between the register files where it likes, and in front
+    of an inline-assembly MFMA it leaves no distance: the MFMA then read the register before the copy had arrived
+    (attention, head dim 256: scores off by a few per cent, exact with one idle state in between; that kernel's MFMAs
+    carry two).  Held for every vector ALU write, not only the copies it was seen with: the kernels that feed an MFMA
+    from the ALU pad their MFMAs, the others feed theirs from LDS reads."""
     ins, in_asm = [], False
     for line in lines:
         if _LABEL.match(line):
@@ -160,7 +162,7 @@ def accvgpr_copies_in_front_of_an_mfma(lines: list[str], states: int = 2) -> lis
         st, k = 0, i - 1
         while k >= 0 and st < states and ins[k] is not None:
             op2, ops2, text2, _ = ins[k]
-            if op2.startswith("v_accvgpr") and ops2 and _regs(ops2[0]) & reads:
+            if op2.startswith("v_") and not op2.startswith("v_mfma") and ops2 and _regs(ops2[0]) & reads:
                 found.append(f"{st} states in front of `{cur[2]}`: `{text2}`")
             st += _states(op2, ops2)
             k -= 1
@@ -197,7 +199,7 @@ def check_listing(listing: str) -> dict[str, list[str]]:
     out = {}
     for name, lines in split_kernels(listing).items():
         if any("v_mfma" in l for l in lines):
-            h = mfma_result_hazards(lines) + accvgpr_copies_in_front_of_an_mfma(lines)
+            h = mfma_result_hazards(lines) + valu_writes_in_front_of_an_mfma(lines)
             if h:
                 out[name] = h
     return out
