@@ -82,3 +82,30 @@ def test_a_register_file_copy_right_in_front_of_the_mfma_that_reads_it_is_found(
     assert lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", ".LBB0_1:", *mf)) == []
     assert lc.valu_writes_in_front_of_an_mfma(kernel("\tv_accvgpr_read_b32 v37, a191", mfma)) == []
     assert list(lc.check_listing("\n".join(kernel("\tv_accvgpr_read_b32 v37, a191", *mf)))) == ["k"]
+
+
+def test_the_build_reads_the_listing_of_its_own_compilation(monkeypatch, tmp_path):
+    """build_code_object hands hipcc -save-temps, checks the listing that lands beside it and refuses the code object
+    when the check finds something (the compiler stands in here: it writes a listing and an object)."""
+    from triton_tenstorrent_amd import build as b
+
+    def compiler(body):
+        def run(cmd, cwd=None):
+            assert "-save-temps" in cmd and cwd is not None
+            out = Path(cmd[cmd.index("-o") + 1])
+            out.write_bytes(b"\x7fELF")
+            Path(cwd, f"probe-hip-amdgcn-amd-amdhsa-{b.ARCH}.s").write_text("\n".join(kernel(*body)))
+        return run
+
+    monkeypatch.setattr(b, "BUILD", tmp_path)
+    monkeypatch.setattr(b, "hipcc", lambda: "hipcc")
+    monkeypatch.setattr(b, "_run", compiler([MFMA, "\ts_nop 7", "\ts_nop 2", "\tv_accvgpr_read_b32 v177, a15"]))
+    assert b.build_code_object("probe") == tmp_path / "probe.hsaco" and (tmp_path / "probe.hsaco").exists()
+    monkeypatch.setattr(b, "_run", compiler([MFMA, "\tv_accvgpr_read_b32 v177, a15"]))
+    try:
+        b.build_code_object("probe")
+    except RuntimeError as e:
+        assert "touched too early" in str(e) and "k:" in str(e)
+    else:
+        raise AssertionError("a listing with a read right behind an MFMA passed the build")
+    assert not (tmp_path / "probe.hsaco").exists()
